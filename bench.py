@@ -1,0 +1,175 @@
+#!/usr/bin/env python3
+"""Benchmark of the BDH decode state step on one MI355X.
+
+Workload (BASELINE config 2, the configuration the metric is quoted on): one layer's
+recurrent state step — RoPE at a position t ~ U[0,4096), readout with the old state and
+rank-1 update — on rho f32 [B=32, h=4, N=8192, d=256] (1 GiB), x = relu(N(mu,1)) with
+mu = Phi^-1(0.05) (about 5 % active neurons), v ~ N(0,1).  One "step" is one call of
+bdh_state_step over the whole batch (32 tokens).  Inputs are resident in HBM before the
+timed region; a ring of distinct (x, v) sets keeps caches from helping.
+
+Prints ONE JSON line (see --help for the knobs).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def cpu_baseline(B, h, N, d, freqs, budget_s=12.0, max_steps=20):
+    """The restated reference CPU path (dense op sequence of src/model/bdh.rs:288-302 plus the
+    rotate), timed on this host on a bounded number of steps of the same workload."""
+    from oracle.bdh_oracle import COracle
+
+    orc = COracle()
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    rng = np.random.default_rng(1)
+    rho = (0.01 * rng.standard_normal((B, h, N, d), dtype=np.float32))
+    x = np.maximum(rng.standard_normal((B, h, N), dtype=np.float32) - np.float32(1.6449), 0)
+    v = rng.standard_normal((B, d), dtype=np.float32)
+    orc.state_step_dense(x, v, freqs, 17, rho)  # warm-up (page faults, thread pool)
+    steps, t0 = 0, time.perf_counter()
+    while steps < max_steps and (time.perf_counter() - t0) < budget_s:
+        orc.state_step_dense(x, v, freqs, 100 + steps, rho)
+        steps += 1
+    dt = time.perf_counter() - t0
+    return {
+        "value": B * steps / dt,
+        "unit": "tokens/s",
+        "cores": min(threads, B * h),
+        "kind": "port",
+        "sample": f"{steps} dense steps of the same config-2 shape (rho f32 [{B},{h},{N},{d}]), "
+                  f"C restatement of the reference op sequence, OpenMP over (b,h) slices, {dt / steps * 1e3:.1f} ms/step",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--heads", type=int, default=4)
+    ap.add_argument("--latent", type=int, default=8192)
+    ap.add_argument("--embd", type=int, default=256)
+    ap.add_argument("--density", type=float, default=0.05)
+    ap.add_argument("--rho-dtype", choices=["f32", "bf16"], default="f32")
+    ap.add_argument("--ring", type=int, default=16, help="number of distinct (x, v) input sets")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from scipy.stats import norm
+
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible; the HIP path is the only path", file=sys.stderr)
+        sys.exit(1)
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.kernel.linear_attention import build_freqs
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    dev = torch.device("cuda:0")
+    B, h, N, d = args.batch, args.heads, args.latent, args.embd
+    ctx = ffi.default_context(0)
+    lib = ctx.lib
+    g = torch.Generator(device=dev).manual_seed(2)
+    tdt = torch.float32 if args.rho_dtype == "f32" else torch.bfloat16
+    esz = 4 if args.rho_dtype == "f32" else 2
+    rho = (0.01 * torch.randn((B, h, N, d), device=dev, generator=g)).to(tdt).contiguous()
+    mu = float(norm.ppf(args.density))
+    xs = [torch.relu(torch.randn((B, h, N), device=dev, generator=g) + mu).contiguous() for _ in range(args.ring)]
+    vs = [torch.randn((B, d), device=dev, generator=g).contiguous() for _ in range(args.ring)]
+    freqs_host = build_freqs(N, 65536.0, RotaryEmbedding.ROPE).reshape(-1)
+    freqs = freqs_host.to(dev)
+    out = torch.empty((B, h, d), device=dev)
+    rows = torch.zeros((B, h), device=dev, dtype=torch.int32)
+    positions = np.random.default_rng(3).integers(0, 4096, size=args.steps + args.warmup)
+    rdt = ffi.F32 if args.rho_dtype == "f32" else ffi.BF16
+
+    # touched rows per input set (R of the algorithmic-bytes formula), measured by the kernel itself
+    R = []
+    scratch = rho.clone()
+    for i in range(args.ring):
+        ctx.check(lib.bdh_state_step(ctx.handle, B, h, N, d, ffi.ROPE, xs[i].data_ptr(), vs[i].data_ptr(),
+                                     freqs.data_ptr(), 0, None, None, scratch.data_ptr(), rdt, out.data_ptr(), None,
+                                     rows.data_ptr()))
+        R.append(int(rows.sum().item()))
+    del scratch
+    R_mean = float(np.mean(R))
+    bytes_per_step = 2.0 * R_mean * d * esz + 4.0 * B * h * N + 4.0 * B * d + 4.0 * B * h * d + 4.0 * N
+
+    fn, hnd = lib.bdh_state_step, ctx.handle
+    call_args = [(hnd, B, h, N, d, ffi.ROPE, xs[i % args.ring].data_ptr(), vs[i % args.ring].data_ptr(),
+                  freqs.data_ptr(), int(positions[i]), None, None, rho.data_ptr(), rdt, out.data_ptr(), None, None)
+                 for i in range(args.steps + args.warmup)]
+    for i in range(args.warmup):
+        ctx.check(fn(*call_args[i]))
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    rc_bad = 0
+    t0 = time.perf_counter()
+    start.record()  # the context launches on torch's current stream, so these events bracket the kernels
+    for i in range(args.warmup, args.warmup + args.steps):
+        rc_bad |= fn(*call_args[i])
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ctx.check(rc_bad)
+    gpu_ms = start.elapsed_time(stop)
+    ms_per_step = max(gpu_ms, wall * 1e3) / args.steps  # the slower of the two clocks
+    kernel_us = gpu_ms / args.steps * 1e3
+    achieved = bytes_per_step / (kernel_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "decode tokens/sec at batch B (single-layer state step) + achieved HBM GB/s",
+        "value": B * args.steps / (ms_per_step * args.steps * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.rho_dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": f"BASELINE config 2: single-layer decode state step, rho {args.rho_dtype} [{B},{h},{N},{d}], "
+                        f"x=relu(N(mu,1)) {args.density:.0%} active, RoPE position ~U[0,4096), {args.ring} input sets",
+            "batch": B, "heads": h, "latent_per_head": N, "n_embd": d, "density": args.density,
+            "touched_rows_per_step": R_mean, "algorithmic_bytes_per_step": bytes_per_step,
+            "gpu_event_ms_total": gpu_ms, "wall_ms_total": wall * 1e3,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "kernel": "k_step_rope_f32 (+ k_step_finalize); duration = HIP-event time of the timed region / steps",
+            "launch_us": kernel_us,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(B, h, N, d, freqs_host.numpy())
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,207 @@
+// Context management, argument validation and the host-side tables of the C ABI.
+#include <cmath>
+#include <new>
+
+#include "bdh_internal.h"
+
+int bdh_fail(bdh_ctx *ctx, int status, const char *fmt, ...) {
+  if (ctx) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(ctx->err, sizeof(ctx->err), fmt, ap);
+    va_end(ap);
+  }
+  return status;
+}
+
+int bdh_ws_reserve(bdh_ctx *ctx, size_t bytes) {
+  if (bytes <= ctx->ws_bytes) return BDH_OK;
+  bytes = bdh_align_up(bytes, size_t(1) << 20);
+  if (ctx->ws) {
+    BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    BDH_HIP_CHECK(ctx, hipFree(ctx->ws));
+    ctx->ws = nullptr;
+    ctx->ws_bytes = 0;
+  }
+  hipError_t e = hipMalloc(&ctx->ws, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return bdh_fail(ctx, BDH_E_NOMEM, "workspace of %zu bytes: %s", bytes, hipGetErrorString(e));
+  }
+  ctx->ws_bytes = bytes;
+  return BDH_OK;
+}
+
+extern "C" {
+
+const char *bdh_version(void) { return "bdh_mi355x 0.1.0 (gfx950)"; }
+
+const char *bdh_status_string(int status) {
+  switch (status) {
+    case BDH_OK: return "ok";
+    case BDH_E_INVAL: return "invalid argument";
+    case BDH_E_SHAPE: return "unsupported shape";
+    case BDH_E_ALIGN: return "misaligned pointer";
+    case BDH_E_HIP: return "HIP runtime error";
+    case BDH_E_NOMEM: return "out of device memory";
+    case BDH_E_UNSUPPORTED: return "unsupported combination";
+    default: return "unknown status";
+  }
+}
+
+int bdh_ctx_create(int device_id, void *hip_stream, bdh_ctx **out) {
+  if (!out) return BDH_E_INVAL;
+  *out = nullptr;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+    (void)hipGetLastError();
+    return BDH_E_HIP;  // no device: there is no CPU path to fall back to
+  }
+  if (device_id < 0 || device_id >= count) return BDH_E_INVAL;
+  bdh_ctx *ctx = new (std::nothrow) bdh_ctx();
+  if (!ctx) return BDH_E_NOMEM;
+  ctx->device = device_id;
+  ctx->stream = static_cast<hipStream_t>(hip_stream);
+  if (hipSetDevice(device_id) != hipSuccess) {
+    delete ctx;
+    return BDH_E_HIP;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device_id) != hipSuccess) {
+    delete ctx;
+    return BDH_E_HIP;
+  }
+  ctx->n_cu = prop.multiProcessorCount;
+  *out = ctx;
+  return BDH_OK;
+}
+
+int bdh_ctx_destroy(bdh_ctx *ctx) {
+  if (!ctx) return BDH_OK;
+  if (ctx->ws) {
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->ws);
+  }
+  delete ctx;
+  return BDH_OK;
+}
+
+int bdh_ctx_set_stream(bdh_ctx *ctx, void *hip_stream) {
+  if (!ctx) return BDH_E_INVAL;
+  ctx->stream = static_cast<hipStream_t>(hip_stream);
+  return BDH_OK;
+}
+
+int bdh_ctx_synchronize(bdh_ctx *ctx) {
+  if (!ctx) return BDH_E_INVAL;
+  BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+  return BDH_OK;
+}
+
+const char *bdh_last_error(const bdh_ctx *ctx) { return ctx ? ctx->err : "null context"; }
+
+int bdh_build_freqs(int latent, float theta, int rotary, float *freqs_host) {
+  if (latent < 0 || !freqs_host) return BDH_E_INVAL;
+  if (rotary != BDH_ROPE && rotary != BDH_ALIBI && rotary != BDH_POPE) return BDH_E_INVAL;
+  const float two_pi = 2.0f * 3.14159265358979323846f;
+  for (int i = 0; i < latent; ++i) {
+    float value = 0.0f;
+    if (rotary == BDH_ROPE) {
+      const float e = (floorf((float)i / 2.0f) * 2.0f) / (float)latent;
+      value = 1.0f / powf(theta, e) / two_pi;
+    } else if (rotary == BDH_POPE) {
+      const float e = (float)i / (float)latent;
+      value = 1.0f / powf(theta, e) / two_pi;
+    }
+    freqs_host[i] = value;
+  }
+  return BDH_OK;
+}
+
+int bdh_default_alibi_slopes(int n_head, float *slopes_host) {
+  if (n_head < 0 || (n_head > 0 && !slopes_host)) return BDH_E_INVAL;
+  for (int i = 0; i < n_head; ++i) slopes_host[i] = 1.0f / powf(2.0f, (float)i / (float)n_head);
+  return BDH_OK;
+}
+
+static int validate_state_args(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary,
+                               const float *x, const float *v, const float *freqs,
+                               int64_t position, void *rho, int rho_dtype, float *out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (B < 0 || h < 0 || T < 0 || N < 0 || d < 0)
+    return bdh_fail(ctx, BDH_E_INVAL, "negative dimension B=%d h=%d T=%d N=%d d=%d", B, h, T, N, d);
+  if (rotary != BDH_ROPE && rotary != BDH_ALIBI && rotary != BDH_POPE)
+    return bdh_fail(ctx, BDH_E_INVAL, "rotary %d is not a bdh_rotary value", rotary);
+  if (rho_dtype != BDH_F32 && rho_dtype != BDH_BF16)
+    return bdh_fail(ctx, BDH_E_INVAL, "rho_dtype %d is not a bdh_dtype value", rho_dtype);
+  if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
+  if (h > 64) return bdh_fail(ctx, BDH_E_SHAPE, "n_head %d > 64", h);
+  if (rotary == BDH_ROPE && (N & 1))
+    return bdh_fail(ctx, BDH_E_SHAPE, "RoPE needs an even latent size, got N=%d", N);
+  const bool empty = (B == 0 || h == 0 || T == 0);
+  if (!empty) {
+    if (!v || !out || (N > 0 && (!x || !rho)) || (rotary != BDH_ALIBI && N > 0 && !freqs))
+      return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+    if (!bdh_aligned(x, 8) || !bdh_aligned(v, 16) || !bdh_aligned(rho, 16) || !bdh_aligned(out, 16) ||
+        !bdh_aligned(freqs, 8))
+      return bdh_fail(ctx, BDH_E_ALIGN, "x/freqs need 8-byte, v/rho/out 16-byte alignment");
+  }
+  return BDH_OK;
+}
+
+int bdh_recurrent_attention(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary,
+                            const float *x, const float *v, const float *freqs,
+                            int64_t position, const int32_t *positions_dev,
+                            const float *alibi_slopes_host, void *rho, int rho_dtype,
+                            float *out, uint64_t *active_bitmask, int32_t *rows_touched) {
+  int rc = validate_state_args(ctx, B, h, T, N, d, rotary, x, v, freqs, position, rho, rho_dtype, out);
+  if (rc != BDH_OK) return rc;
+  if (B == 0 || h == 0 || T == 0) return BDH_OK;
+  float slopes[64];
+  if (rotary == BDH_ALIBI) {
+    if (alibi_slopes_host)
+      memcpy(slopes, alibi_slopes_host, sizeof(float) * h);
+    else
+      bdh_default_alibi_slopes(h, slopes);
+  }
+  StateStepParams p{B, h, T, N, d, rotary, rho_dtype, x, v, freqs, position, positions_dev,
+                    rotary == BDH_ALIBI ? slopes : nullptr, rho, out, active_bitmask, rows_touched};
+  return bdh_launch_state_steps(ctx, p);
+}
+
+int bdh_state_step(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const float *x,
+                   const float *v, const float *freqs, int64_t position,
+                   const int32_t *positions_dev, const float *alibi_slopes_host, void *rho,
+                   int rho_dtype, float *out, uint64_t *active_bitmask, int32_t *rows_touched) {
+  return bdh_recurrent_attention(ctx, B, h, 1, N, d, rotary, x, v, freqs, position, positions_dev,
+                                 alibi_slopes_host, rho, rho_dtype, out, active_bitmask,
+                                 rows_touched);
+}
+
+int bdh_relu_lowrank(bdh_ctx *ctx, int B, int h_in, int T, int d, int h, int N, const float *in,
+                     const float *weight, const float *bias, float threshold, int block_size,
+                     const uint8_t *active_blocks_host, int n_blocks, const float *gate,
+                     float *out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (B < 0 || T < 0 || d < 0 || h < 0 || N < 0)
+    return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
+  if (h_in != 1 && h_in != h)
+    return bdh_fail(ctx, BDH_E_SHAPE, "input head dim %d must be 1 or %d", h_in, h);
+  if (active_blocks_host && (block_size < 1 || n_blocks < 0))
+    return bdh_fail(ctx, BDH_E_INVAL, "bad block pattern");
+  if (B == 0 || T == 0 || h == 0 || N == 0) return BDH_OK;
+  if (!out || !weight || (d > 0 && !in)) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  ReluLowrankParams p{B, h_in, T, d, h, N, in, weight, bias, threshold, block_size,
+                      active_blocks_host, n_blocks, gate, out};
+  return bdh_launch_relu_lowrank(ctx, p);
+}
+
+int bdh_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (rows < 0 || d < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
+  if (rows == 0 || d == 0) return BDH_OK;
+  if (!in || !out) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  return bdh_launch_layer_norm(ctx, rows, d, in, out);
+}
+
+}  // extern "C"

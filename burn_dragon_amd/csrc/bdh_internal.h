@@ -1,0 +1,101 @@
+// Internal declarations shared by the translation units of libbdh_mi355x.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/bdh_mi355x.h"
+
+struct bdh_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  // growable device workspace (partials, counters); owned by the context
+  void *ws = nullptr;
+  size_t ws_bytes = 0;
+  int n_cu = 0;
+  char err[512] = {0};
+};
+
+struct bdh_model {
+  bdh_ctx *ctx = nullptr;
+  bdh_model_config cfg{};
+  bdh_model_weights w{};
+  float *freqs = nullptr;   // device [N]
+  float slopes[64] = {0};   // host, ALiBi only
+  // activation scratch, grown on demand to the largest (B,T) seen
+  void *act = nullptr;
+  size_t act_bytes = 0;
+};
+
+int bdh_fail(bdh_ctx *ctx, int status, const char *fmt, ...);
+
+// Grows ctx->ws to at least `bytes` (synchronises the stream before freeing the old one).
+int bdh_ws_reserve(bdh_ctx *ctx, size_t bytes);
+
+#define BDH_HIP_CHECK(ctx, call)                                                        \
+  do {                                                                                  \
+    hipError_t e_ = (call);                                                             \
+    if (e_ != hipSuccess)                                                               \
+      return bdh_fail((ctx), BDH_E_HIP, "%s failed: %s (%s:%d)", #call,                 \
+                      hipGetErrorString(e_), __FILE__, __LINE__);                       \
+  } while (0)
+
+#define BDH_LAUNCH_CHECK(ctx, what)                                                     \
+  do {                                                                                  \
+    hipError_t e_ = hipGetLastError();                                                  \
+    if (e_ != hipSuccess)                                                               \
+      return bdh_fail((ctx), BDH_E_HIP, "launch of %s failed: %s", (what),              \
+                      hipGetErrorString(e_));                                           \
+  } while (0)
+
+static inline size_t bdh_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+static inline bool bdh_aligned(const void *p, size_t a) {
+  return (reinterpret_cast<uintptr_t>(p) % a) == 0;
+}
+
+// ---- launchers implemented in the kernel translation units --------------------------
+struct StateStepParams {
+  int B, h, T, N, d, rotary, rho_dtype;
+  const float *x, *v, *freqs;
+  int64_t position;
+  const int32_t *positions_dev;
+  const float *slopes_host;  // resolved (never null for ALiBi)
+  void *rho;
+  float *out;
+  uint64_t *bitmask;
+  int32_t *rows_touched;
+};
+int bdh_launch_state_steps(bdh_ctx *ctx, const StateStepParams &p);
+
+// Variant used inside the fused model step: the readout is LayerNorm-ed on the fly
+// (src/model/bdh.rs:359) when out_ln != nullptr.
+int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
+
+struct ReluLowrankParams {
+  int B, h_in, T, d, h, N;
+  const float *in, *weight, *bias;
+  float threshold;
+  int block_size;
+  const uint8_t *active_blocks_host;
+  int n_blocks;
+  const float *gate;
+  float *out;
+};
+int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p);
+int bdh_launch_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);
+
+// embed gather + LN (src/model/bdh.rs:319-322); tokens validated on the device: an id
+// outside [0,V) writes NaN rows (the reference would panic in the gather).
+int bdh_launch_embed_ln(bdh_ctx *ctx, const int64_t *tokens, int64_t rows, int d, int V,
+                        const float *embed, float *out);
+// mlp = mixed . decoder with mixed[b*T+t, hh*N+n] = xy[b,hh,t,n]; cur = LN(cur + LN(mlp))
+// (src/model/bdh.rs:383,436-441)
+int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
+                                const float *xy, const float *decoder, float *cur);
+// logits = cur . lm_head (+ argmax of the last token per sequence) (src/model/bdh.rs:446-449)
+int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cur,
+                       const float *lm_head, float *logits, int64_t *next_tokens);

@@ -1,0 +1,142 @@
+// The whole cached step, BDH::forward_with_state (src/model/bdh.rs:309-450), as a
+// stream-ordered sequence of the kernels of this library.
+#include <new>
+#include <vector>
+
+#include "bdh_internal.h"
+
+namespace {
+
+int ensure_act(bdh_model *m, size_t bytes) {
+  if (bytes <= m->act_bytes) return BDH_OK;
+  bdh_ctx *ctx = m->ctx;
+  if (m->act) {
+    BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    BDH_HIP_CHECK(ctx, hipFree(m->act));
+    m->act = nullptr;
+    m->act_bytes = 0;
+  }
+  bytes = bdh_align_up(bytes, size_t(1) << 20);
+  hipError_t e = hipMalloc(&m->act, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return bdh_fail(ctx, BDH_E_NOMEM, "activation scratch of %zu bytes: %s", bytes, hipGetErrorString(e));
+  }
+  m->act_bytes = bytes;
+  return BDH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int bdh_model_create(bdh_ctx *ctx, const bdh_model_config *c, const bdh_model_weights *w, bdh_model **out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (!c || !w || !out) return bdh_fail(ctx, BDH_E_INVAL, "null argument");
+  *out = nullptr;
+  if (c->n_layer < 1 || c->n_embd < 1 || c->n_head < 1 || c->latent < 1 || c->vocab < 1)
+    return bdh_fail(ctx, BDH_E_INVAL, "non-positive model dimension");
+  if (c->n_head > 64) return bdh_fail(ctx, BDH_E_SHAPE, "n_head %d > 64", c->n_head);
+  if (c->rotary != BDH_ROPE && c->rotary != BDH_ALIBI && c->rotary != BDH_POPE)
+    return bdh_fail(ctx, BDH_E_INVAL, "rotary %d is not a bdh_rotary value", c->rotary);
+  if (c->rotary == BDH_ROPE && (c->latent & 1))
+    return bdh_fail(ctx, BDH_E_SHAPE, "RoPE needs an even latent size, got %d", c->latent);
+  if ((c->n_embd & 3) || c->n_embd > 1024)
+    return bdh_fail(ctx, BDH_E_SHAPE, "n_embd must be a multiple of 4 and <= 1024, got %d", c->n_embd);
+  if (!w->embed || !w->encoder || !w->encoder_v || !w->decoder || !w->lm_head)
+    return bdh_fail(ctx, BDH_E_INVAL, "null weight pointer");
+  bdh_model *m = new (std::nothrow) bdh_model();
+  if (!m) return bdh_fail(ctx, BDH_E_NOMEM, "host allocation failed");
+  m->ctx = ctx;
+  m->cfg = *c;
+  m->cfg.alibi_slopes_host = nullptr;
+  m->w = *w;
+  if (c->rotary == BDH_ALIBI) {
+    if (c->alibi_slopes_host)
+      memcpy(m->slopes, c->alibi_slopes_host, sizeof(float) * c->n_head);
+    else
+      bdh_default_alibi_slopes(c->n_head, m->slopes);
+  }
+  std::vector<float> f(c->latent);
+  bdh_build_freqs(c->latent, c->rope_theta, c->rotary, f.data());
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&m->freqs), sizeof(float) * (size_t)c->latent);
+  if (e == hipSuccess) e = hipMemcpy(m->freqs, f.data(), sizeof(float) * (size_t)c->latent, hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    if (m->freqs) (void)hipFree(m->freqs);
+    delete m;
+    return bdh_fail(ctx, BDH_E_HIP, "freqs table upload: %s", hipGetErrorString(e));
+  }
+  *out = m;
+  return BDH_OK;
+}
+
+int bdh_model_destroy(bdh_model *m) {
+  if (!m) return BDH_OK;
+  if (m->ctx) (void)hipStreamSynchronize(m->ctx->stream);
+  if (m->freqs) (void)hipFree(m->freqs);
+  if (m->act) (void)hipFree(m->act);
+  delete m;
+  return BDH_OK;
+}
+
+size_t bdh_model_state_bytes(const bdh_model *m, int B, int rho_dtype) {
+  if (!m || B < 0) return 0;
+  const size_t Nq = m->cfg.rotary == BDH_POPE ? 2 * (size_t)m->cfg.latent : (size_t)m->cfg.latent;
+  const size_t es = rho_dtype == BDH_BF16 ? 2 : 4;
+  return (size_t)m->cfg.n_layer * B * m->cfg.n_head * Nq * m->cfg.n_embd * es;
+}
+
+int bdh_model_forward(bdh_model *m, const int64_t *tokens, int B, int T, void *rho, int rho_dtype,
+                      int64_t position, float *logits, int64_t *next_tokens, float *x_tap) {
+  if (!m) return BDH_E_INVAL;
+  bdh_ctx *ctx = m->ctx;
+  if (B < 0 || T < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative batch or time");
+  if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
+  if (rho_dtype != BDH_F32 && rho_dtype != BDH_BF16) return bdh_fail(ctx, BDH_E_INVAL, "bad rho_dtype");
+  if (B == 0 || T == 0) return BDH_OK;
+  if (!tokens || !rho || !logits) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  if (!bdh_aligned(rho, 16)) return bdh_fail(ctx, BDH_E_ALIGN, "rho needs 16-byte alignment");
+  const bdh_model_config &c = m->cfg;
+  const int d = c.n_embd, h = c.n_head, N = c.latent, V = c.vocab, L = c.n_layer;
+  const size_t Nq = c.rotary == BDH_POPE ? 2 * (size_t)N : (size_t)N;
+  const size_t M = (size_t)B * T;
+
+  // activation scratch: cur [M,d] | x [B,h,T,N] | xy [B,h,T,N] | attn [B,h,T,d] | attn_ln [B,h,T,d]
+  const size_t n_cur = bdh_align_up(M * d, 64), n_x = bdh_align_up(M * h * N, 64), n_a = bdh_align_up(M * h * d, 64);
+  int rc = ensure_act(m, sizeof(float) * (n_cur + 2 * n_x + 2 * n_a));
+  if (rc != BDH_OK) return rc;
+  float *cur = static_cast<float *>(m->act);
+  float *x = cur + n_cur;
+  float *xy = x + n_x;
+  float *attn = xy + n_x;
+  float *attn_ln = attn + n_a;
+
+  rc = bdh_launch_embed_ln(ctx, tokens, (int64_t)M, d, V, m->w.embed, cur);  // :319-322
+  if (rc != BDH_OK) return rc;
+  const size_t rho_layer_bytes = (size_t)B * h * Nq * d * (rho_dtype == BDH_BF16 ? 2 : 4);
+  for (int l = 0; l < L; ++l) {  // :336 — the same weights in every layer
+    float *x_l = x_tap ? x_tap + (size_t)l * M * h * N : x;
+    // :337-351  x = relu(cur . encoder - thr)
+    ReluLowrankParams px{B, 1, T, d, h, N, cur, m->w.encoder, nullptr, c.relu_threshold, 1, nullptr, 0, nullptr, x_l};
+    rc = bdh_launch_relu_lowrank(ctx, px);
+    if (rc != BDH_OK) return rc;
+    // :353-359  recurrent attention (value = cur) and LayerNorm of its output
+    StateStepParams ps{B, h, T, N, d, c.rotary, rho_dtype, x_l, cur, m->freqs, position, nullptr,
+                       c.rotary == BDH_ALIBI ? m->slopes : nullptr,
+                       static_cast<char *>(rho) + (size_t)l * rho_layer_bytes, attn, nullptr, nullptr};
+    rc = bdh_launch_state_steps_ln(ctx, ps, attn_ln);
+    if (rc != BDH_OK) return rc;
+    // :361-381  xy = x * relu(LN(attn) . encoder_v - thr)
+    ReluLowrankParams py{B, h, T, d, h, N, attn_ln, m->w.encoder_v, nullptr, c.relu_threshold, 1, nullptr, 0, x_l, xy};
+    rc = bdh_launch_relu_lowrank(ctx, py);
+    if (rc != BDH_OK) return rc;
+    // :383,436-441  cur = LN(cur + LN(mixed . decoder))
+    rc = bdh_launch_decoder_residual(ctx, B, T, h, N, d, xy, m->w.decoder, cur);
+    if (rc != BDH_OK) return rc;
+  }
+  // :446-449
+  return bdh_launch_lm_head(ctx, B, T, d, V, cur, m->w.lm_head, logits, next_tokens);
+}
+
+}  // extern "C"

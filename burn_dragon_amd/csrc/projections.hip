@@ -1,0 +1,410 @@
+// Dense stages around the state step: ReLU low-rank projections (D_x, D_y), LayerNorm,
+// embedding gather, the decoder E with the residual LayerNorms, and lm_head.
+// Reference semantics: src/kernel/relu_lowrank.rs:7-37, src/model/bdh.rs:86-89, :319-322,
+// :346-350, :370-384, :436-449.
+#include "bdh_internal.h"
+
+namespace {
+
+constexpr float kLnEps = 1e-5f;  // src/model/bdh.rs:17
+
+// Sum of `v` over a 256-thread workgroup; every thread gets the result.
+__device__ __forceinline__ float block_sum_256(float v, float *s_part) {
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  __syncthreads();  // protects s_part against the previous use
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return s_part[0] + s_part[1] + s_part[2] + s_part[3];
+}
+
+// ------------------------------------------------------------------------------------
+// relu_lowrank: out[b,hh,t,n] = relu(sum_k in[b,hh|0,t,k] w[hh,k,n] + bias - thr) * mask
+// One thread per latent column n (coalesced weight rows), RT input rows per workgroup
+// staged in LDS, one k-sequential fmaf chain per output.
+// ------------------------------------------------------------------------------------
+template <int RT, int UK>
+__global__ __launch_bounds__(256) void k_relu_lowrank(const float *__restrict__ in, int h_in, int T, int d,
+                                                      const float *__restrict__ w, int h, int N,
+                                                      const float *__restrict__ bias, float thr,
+                                                      const unsigned char *__restrict__ block_active,
+                                                      int block_size, int n_blocks,
+                                                      const float *__restrict__ gate, float *__restrict__ out,
+                                                      int M) {
+  extern __shared__ float s_in[];  // [RT][d]
+  const int tid = threadIdx.x;
+  const int hh = blockIdx.y;
+  const int n = blockIdx.x * 256 + tid;
+  const int m0 = blockIdx.z * RT;
+  for (int i = tid; i < RT * d; i += 256) {
+    const int r = i / d, k = i - r * d;
+    const int m = m0 + r;
+    float val = 0.0f;
+    if (m < M) {
+      const int b = m / T, t = m - b * T;
+      val = in[(((long)b * h_in + (h_in == 1 ? 0 : hh)) * T + t) * d + k];
+    }
+    s_in[i] = val;
+  }
+  __syncthreads();
+  if (n >= N) return;
+
+  float acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = 0.0f;
+  const float *wp = w + (long)hh * d * N + n;
+  int k0 = 0;
+  for (; k0 + UK <= d; k0 += UK) {
+    float wv[UK];
+#pragma unroll
+    for (int u = 0; u < UK; ++u) wv[u] = wp[(long)(k0 + u) * N];
+#pragma unroll
+    for (int u = 0; u < UK; ++u)
+#pragma unroll
+      for (int r = 0; r < RT; ++r) acc[r] = __builtin_fmaf(s_in[r * d + k0 + u], wv[u], acc[r]);
+  }
+  for (; k0 < d; ++k0) {
+    const float wv = wp[(long)k0 * N];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) acc[r] = __builtin_fmaf(s_in[r * d + k0], wv, acc[r]);
+  }
+
+  const float bv = bias ? bias[(long)hh * N + n] : 0.0f;
+  float maskv = 1.0f;
+  if (block_active) {
+    const int blk = n / block_size;
+    maskv = (blk < n_blocks && block_active[blk]) ? 1.0f : 0.0f;
+  }
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int m = m0 + r;
+    if (m < M) {
+      const int b = m / T, t = m - b * T;
+      float p = acc[r];
+      if (bias) p = p + bv;
+      if (thr != 0.0f) p = p - thr;
+      float y = p > 0.0f ? p : 0.0f;
+      if (block_active) y = y * maskv;
+      const long o = (((long)b * h + hh) * T + t) * N + n;
+      if (gate) y = gate[o] * y;
+      out[o] = y;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// LayerNorm rows (one workgroup per row); in == out allowed.  The row is staged in LDS and
+// every thread walks it in index order, so mean and variance are the same left-to-right f32
+// sums a scalar loop produces, independent of the launch shape.
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ void ln_stats_in_order(const float *s_row, int d, float &mean, float &den) {
+  float sum = 0.0f;
+  for (int i = 0; i < d; ++i) sum += s_row[i];
+  mean = sum / (float)d;
+  float sq = 0.0f;
+  for (int i = 0; i < d; ++i) {
+    const float c = s_row[i] - mean;
+    sq += c * c;
+  }
+  den = sqrtf(sq / (float)d + kLnEps);
+}
+
+__global__ __launch_bounds__(256) void k_layer_norm(const float *__restrict__ in, float *__restrict__ out, int d) {
+  extern __shared__ float s_row[];
+  const float *x = in + (long)blockIdx.x * d;
+  float *y = out + (long)blockIdx.x * d;
+  for (int c = threadIdx.x; c < d; c += 256) s_row[c] = x[c];
+  __syncthreads();
+  float mean, den;
+  ln_stats_in_order(s_row, d, mean, den);
+  for (int c = threadIdx.x; c < d; c += 256) y[c] = (s_row[c] - mean) / den;
+}
+
+// embed gather + LayerNorm (src/model/bdh.rs:319-322)
+__global__ __launch_bounds__(256) void k_embed_ln(const int64_t *__restrict__ tokens, int d, int V,
+                                                  const float *__restrict__ embed, float *__restrict__ out) {
+  extern __shared__ float s_row[];
+  const int64_t tok = tokens[blockIdx.x];
+  float *y = out + (long)blockIdx.x * d;
+  if (tok < 0 || tok >= V) {  // the reference's gather would panic; poison the row instead
+    for (int c = threadIdx.x; c < d; c += 256) y[c] = __int_as_float(0x7fc00000);
+    return;
+  }
+  const float *x = embed + (long)tok * d;
+  for (int c = threadIdx.x; c < d; c += 256) s_row[c] = x[c];
+  __syncthreads();
+  float mean, den;
+  ln_stats_in_order(s_row, d, mean, den);
+  for (int c = threadIdx.x; c < d; c += 256) y[c] = (s_row[c] - mean) / den;
+}
+
+// ------------------------------------------------------------------------------------
+// decoder: partial[kb][m][:] = sum_{k in block kb} mixed[m,k] * E[k,:]
+// mixed[m = b*T+t, k = hh*N+n] = xy[b,hh,t,n].  Rows of E whose xy is zero for every row
+// of the tile are never loaded.
+// ------------------------------------------------------------------------------------
+template <int RT>
+__global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict__ xy,
+                                                         const float *__restrict__ E,
+                                                         float *__restrict__ partial, int T, int h, int N,
+                                                         int d, int KB, int M) {
+  extern __shared__ float s_mem[];  // [RT][KB] xy tile, then reused for the wave reduction
+  constexpr int MAXV = 4;           // d <= 1024: up to 4 float4... columns c = (j*64+lane)*4
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int kb = blockIdx.x;
+  const int m0 = blockIdx.y * RT;
+  const int K = h * N;
+  const int nv = (d + 255) >> 8;  // float4 groups per lane
+  float *s_xy = s_mem;
+  for (int i = tid; i < RT * KB; i += 256) {
+    const int r = i / KB, kk = i - r * KB;
+    const int m = m0 + r, k = kb * KB + kk;
+    float val = 0.0f;
+    if (m < M && k < K) {
+      const int b = m / T, t = m - b * T;
+      const int hh = k / N, n = k - hh * N;
+      val = xy[(((long)b * h + hh) * T + t) * N + n];
+    }
+    s_xy[i] = val;
+  }
+  __syncthreads();
+
+  float4 acc[RT][MAXV];
+#pragma unroll
+  for (int r = 0; r < RT; ++r)
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) acc[r][j] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  for (int kk = wave; kk < KB; kk += 4) {
+    const int k = kb * KB + kk;
+    if (k >= K) break;
+    float xs[RT];
+    bool any = false;
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      xs[r] = s_xy[r * KB + kk];
+      any = any || (xs[r] != 0.0f);
+    }
+    if (!any) continue;
+    const float *erow = E + (long)k * d;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+      const int c = (j * 64 + lane) * 4;
+      if (j < nv && c < d) {
+        const float4 e = *reinterpret_cast<const float4 *>(erow + c);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+          acc[r][j].x = __builtin_fmaf(xs[r], e.x, acc[r][j].x);
+          acc[r][j].y = __builtin_fmaf(xs[r], e.y, acc[r][j].y);
+          acc[r][j].z = __builtin_fmaf(xs[r], e.z, acc[r][j].z);
+          acc[r][j].w = __builtin_fmaf(xs[r], e.w, acc[r][j].w);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // cross-wave reduction, one row of the tile at a time, through LDS [4][d]
+  float *s_red = s_mem;
+  for (int r = 0; r < RT; ++r) {
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j) {
+      const int c = (j * 64 + lane) * 4;
+      if (j < nv && c < d) *reinterpret_cast<float4 *>(s_red + wave * d + c) = acc[r][j];
+    }
+    __syncthreads();
+    const int m = m0 + r;
+    if (m < M)
+      for (int c = tid; c < d; c += 256)
+        partial[((long)kb * M + m) * d + c] = s_red[c] + s_red[d + c] + s_red[2 * d + c] + s_red[3 * d + c];
+    __syncthreads();
+  }
+}
+
+// cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))   (src/model/bdh.rs:438-441)
+__global__ __launch_bounds__(256) void k_decoder_finalize(const float *__restrict__ partial, int KBN, int M,
+                                                          int d, float *__restrict__ cur) {
+  __shared__ float s_part[4];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  float vals[4];
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 256 + tid;
+    float v = 0.0f;
+    if (c < d) {
+      for (int kb = 0; kb < KBN; ++kb) v += partial[((long)kb * M + m) * d + c];
+      s += v;
+    }
+    vals[j] = v;
+  }
+  float mean = block_sum_256(s, s_part) / (float)d;
+  float q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (j * 256 + tid < d) {
+      const float t = vals[j] - mean;
+      q += t * t;
+    }
+  float den = sqrtf(block_sum_256(q, s_part) / (float)d + kLnEps);
+  s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 256 + tid;
+    if (c < d) {
+      const float mlp = (vals[j] - mean) / den;
+      vals[j] = cur[(long)m * d + c] + mlp;
+      s += vals[j];
+    }
+  }
+  mean = block_sum_256(s, s_part) / (float)d;
+  q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (j * 256 + tid < d) {
+      const float t = vals[j] - mean;
+      q += t * t;
+    }
+  den = sqrtf(block_sum_256(q, s_part) / (float)d + kLnEps);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 256 + tid;
+    if (c < d) cur[(long)m * d + c] = (vals[j] - mean) / den;
+  }
+}
+
+// logits[m,:] = cur[m,:] . lm_head ; optional argmax of the last token of each sequence
+__global__ __launch_bounds__(256) void k_lm_head(const float *__restrict__ cur, const float *__restrict__ W,
+                                                 int T, int d, int V, float *__restrict__ logits,
+                                                 int64_t *__restrict__ next_tokens) {
+  extern __shared__ float s_cur[];  // [d]
+  __shared__ float s_best[4];
+  __shared__ int s_arg[4];
+  const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int k = tid; k < d; k += 256) s_cur[k] = cur[(long)m * d + k];
+  __syncthreads();
+  float best = -INFINITY;
+  int arg = 0x7fffffff;
+  for (int c = tid; c < V; c += 256) {
+    float acc = 0.0f;
+    for (int k = 0; k < d; ++k) acc = __builtin_fmaf(s_cur[k], W[(long)k * V + c], acc);
+    logits[(long)m * V + c] = acc;
+    if (acc > best) {  // strided visit in increasing c: keeps the lowest index on ties
+      best = acc;
+      arg = c;
+    }
+  }
+  const int b = m / T, t = m - b * T;
+  if (!next_tokens || t != T - 1) return;
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o);
+    const int oa = __shfl_xor(arg, o);
+    if (ob > best || (ob == best && oa < arg)) {
+      best = ob;
+      arg = oa;
+    }
+  }
+  if (lane == 0) {
+    s_best[wave] = best;
+    s_arg[wave] = arg;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (s_best[w] > best || (s_best[w] == best && s_arg[w] < arg)) {
+        best = s_best[w];
+        arg = s_arg[w];
+      }
+    next_tokens[b] = arg == 0x7fffffff ? 0 : arg;
+  }
+}
+
+template <int RT>
+void launch_relu(hipStream_t st, dim3 grid, size_t lds, const ReluLowrankParams &p, const unsigned char *mask,
+                 int M) {
+  hipLaunchKernelGGL((k_relu_lowrank<RT, 16>), grid, dim3(256), lds, st, p.in, p.h_in, p.T, p.d, p.weight, p.h,
+                     p.N, p.bias, p.threshold, mask, p.block_size, p.n_blocks, p.gate, p.out, M);
+}
+
+}  // namespace
+
+int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
+  const long M = (long)p.B * p.T;
+  if (M > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "B*T too large");
+  const unsigned char *mask_dev = nullptr;
+  if (p.active_blocks_host) {
+    int rc = bdh_ws_reserve(ctx, (size_t)p.n_blocks + 256);
+    if (rc != BDH_OK) return rc;
+    // pageable source: the runtime stages the copy, so the host buffer may be reused on return
+    if (p.n_blocks > 0)
+      BDH_HIP_CHECK(ctx, hipMemcpyAsync(ctx->ws, p.active_blocks_host, (size_t)p.n_blocks,
+                                        hipMemcpyHostToDevice, ctx->stream));
+    mask_dev = static_cast<const unsigned char *>(ctx->ws);
+  }
+  const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
+  const size_t lds = sizeof(float) * (size_t)RT * (p.d > 0 ? p.d : 1);
+  if (lds > 64 * 1024) return bdh_fail(ctx, BDH_E_SHAPE, "d=%d too large for the projection tile", p.d);
+  const long row_tiles = (M + RT - 1) / RT;
+  if (row_tiles > 65535 || p.h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (row tiles %ld)", row_tiles);
+  dim3 grid((p.N + 255) / 256, p.h, (unsigned)row_tiles);
+  switch (RT) {
+    case 8: launch_relu<8>(ctx->stream, grid, lds, p, mask_dev, (int)M); break;
+    case 4: launch_relu<4>(ctx->stream, grid, lds, p, mask_dev, (int)M); break;
+    case 2: launch_relu<2>(ctx->stream, grid, lds, p, mask_dev, (int)M); break;
+    default: launch_relu<1>(ctx->stream, grid, lds, p, mask_dev, (int)M); break;
+  }
+  BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank");
+  return BDH_OK;
+}
+
+int bdh_launch_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out) {
+  if (rows > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many rows");
+  if (d > 16384) return bdh_fail(ctx, BDH_E_SHAPE, "LayerNorm row of %d floats does not fit in LDS", d);
+  hipLaunchKernelGGL(k_layer_norm, dim3((unsigned)rows), dim3(256), sizeof(float) * (size_t)d, ctx->stream, in, out, d);
+  BDH_LAUNCH_CHECK(ctx, "k_layer_norm");
+  return BDH_OK;
+}
+
+int bdh_launch_embed_ln(bdh_ctx *ctx, const int64_t *tokens, int64_t rows, int d, int V, const float *embed,
+                        float *out) {
+  hipLaunchKernelGGL(k_embed_ln, dim3((unsigned)rows), dim3(256), sizeof(float) * (size_t)d, ctx->stream, tokens, d, V, embed, out);
+  BDH_LAUNCH_CHECK(ctx, "k_embed_ln");
+  return BDH_OK;
+}
+
+int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d, const float *xy,
+                                const float *decoder, float *cur) {
+  const int M = B * T;
+  const long K = (long)h * N;
+  if (d > 1024 || (d & 3)) return bdh_fail(ctx, BDH_E_SHAPE, "decoder needs d %% 4 == 0 and d <= 1024, got %d", d);
+  const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
+  const int row_tiles = (M + RT - 1) / RT;
+  // k-block size: enough workgroups to fill the chip, few enough partials
+  int KB = 1024;
+  while (KB > 64 && ((K + KB - 1) / KB) * row_tiles < 4L * (ctx->n_cu > 0 ? ctx->n_cu : 256)) KB >>= 1;
+  const int KBN = (int)((K + KB - 1) / KB);
+  size_t lds = sizeof(float) * (size_t)RT * KB;
+  if (lds < sizeof(float) * 4u * d) lds = sizeof(float) * 4u * d;
+  const size_t pbytes = sizeof(float) * (size_t)KBN * M * d;
+  int rc = bdh_ws_reserve(ctx, pbytes);
+  if (rc != BDH_OK) return rc;
+  float *partial = static_cast<float *>(ctx->ws);
+  dim3 grid(KBN, row_tiles);
+  switch (RT) {
+    case 8: hipLaunchKernelGGL((k_decoder_partial<8>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
+    case 4: hipLaunchKernelGGL((k_decoder_partial<4>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
+    case 2: hipLaunchKernelGGL((k_decoder_partial<2>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
+    default: hipLaunchKernelGGL((k_decoder_partial<1>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
+  }
+  BDH_LAUNCH_CHECK(ctx, "k_decoder_partial");
+  hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(256), 0, ctx->stream, partial, KBN, M, d, cur);
+  BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
+  return BDH_OK;
+}
+
+int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cur, const float *lm_head,
+                       float *logits, int64_t *next_tokens) {
+  const int M = B * T;
+  hipLaunchKernelGGL(k_lm_head, dim3(M), dim3(256), sizeof(float) * (size_t)d, ctx->stream, cur, lm_head, T, d,
+                     V, logits, next_tokens);
+  BDH_LAUNCH_CHECK(ctx, "k_lm_head");
+  return BDH_OK;
+}

@@ -1,0 +1,499 @@
+// The recurrent state step of the BDH cached path on gfx950:
+//   rotate (RoPE / PoPE / none)  ->  readout with the OLD state  ->  rank-1 update.
+// Reference semantics: src/model/bdh.rs:258-307 and src/model/attention.rs:305-349.
+//
+// Layout in HBM: rho [B,h,Nq,d] row-major; one state row = d contiguous values.  The two
+// rows of a RoPE lane pair (2j, 2j+1) are adjacent, so an active pair is one contiguous
+// 2*d*sizeof(T) chunk.  A 64-lane wavefront covers one d=256 f32 row with one 16-byte
+// load per lane (1 KiB, eight 128-byte segments).
+//
+// Fast path (RoPE, d in {256,512}): one workgroup owns WAVES*64 lane pairs of one
+// (b,h) slice.  Lane l of wave w loads pair w*64+l of x, rotates it, and the wavefront
+// ballot gives the 64-bit active-pair mask; popcount prefix sums compact the active pairs
+// of the workgroup into an LDS list, which the waves then walk round-robin, U pairs in
+// flight per wave.  Every touched byte of rho is read once and written once.  The readout
+// is reduced across waves in LDS and written as one partial per workgroup; a second small
+// kernel adds the partials in a fixed order (deterministic, no atomics).
+#include <hip/hip_bf16.h>
+
+#include "bdh_internal.h"
+
+namespace {
+
+// f32(2*PI) exactly as `2.0 * PI` evaluates with std::f32::consts::PI
+// (src/model/attention.rs:343)
+constexpr float kTwoPi = 6.28318530717958647692f;
+
+__device__ __forceinline__ float rope_phase(float pos, float f) {
+  const float raw = pos * f;  // contraction is off for this file: two roundings, as the reference
+  return (raw - floorf(raw)) * kTwoPi;
+}
+
+__device__ __forceinline__ float softplus1(float x) { return logf(expf(x * 1.0f) + 1.0f) / 1.0f; }
+
+__device__ __forceinline__ float bf16_to_f32(unsigned short v) {
+  return __uint_as_float(static_cast<unsigned int>(v) << 16);
+}
+__device__ __forceinline__ unsigned short f32_to_bf16(float f) {  // round to nearest even
+  unsigned int u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<unsigned short>((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<unsigned short>(u >> 16);
+}
+
+// spread the 32 bits of v to the even bit positions of a 64-bit word
+__device__ __forceinline__ unsigned long long spread_bits(unsigned int v) {
+  unsigned long long x = v;
+  x = (x | (x << 16)) & 0x0000FFFF0000FFFFull;
+  x = (x | (x << 8)) & 0x00FF00FF00FF00FFull;
+  x = (x | (x << 4)) & 0x0F0F0F0F0F0F0F0Full;
+  x = (x | (x << 2)) & 0x3333333333333333ull;
+  x = (x | (x << 1)) & 0x5555555555555555ull;
+  return x;
+}
+
+struct HeadScalars {
+  float v[64];
+};
+
+struct StepPtrs {
+  const float *x;        // token t of slice 0
+  long x_slice_stride;   // elements between (b,h) slices
+  const float *v;        // token t of batch 0
+  long v_batch_stride;
+  const float *freqs;
+  float pos_scalar;             // f32(position + t)
+  const int32_t *pos_dev;       // optional per-sequence start positions
+  int pos_add;                  // t, added to pos_dev[b]
+  float *partial;               // [slices, S, d]
+  int *pair_cnt;                // [slices, S]
+  unsigned long long *bitmask;  // token t of slice 0, or null
+  long bitmask_slice_stride;
+  int h, N, S;
+};
+
+// ------------------------------------------------------------------------------------
+// fast path: RoPE, f32 state, D in {256, 512}
+// ------------------------------------------------------------------------------------
+template <int D, int WAVES, int U>
+__global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float *__restrict__ rho) {
+  constexpr int VPL = D / 256;     // float4 per lane per row
+  constexpr int PPB = WAVES * 64;  // lane pairs per workgroup
+  __shared__ int s_cnt[WAVES];
+  __shared__ unsigned short s_idx[PPB];
+  __shared__ float2 s_q[PPB];
+  __shared__ float4 s_red[WAVES][D / 4];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int slice = blockIdx.x / a.S;
+  const int seg = blockIdx.x - slice * a.S;
+  const int b = slice / a.h;
+  const int NP = a.N >> 1;
+  const int p = seg * PPB + tid;
+
+  float2 xv = make_float2(0.0f, 0.0f), fv = make_float2(0.0f, 0.0f);
+  if (p < NP) {
+    xv = reinterpret_cast<const float2 *>(a.x + (long)slice * a.x_slice_stride)[p];
+    fv = reinterpret_cast<const float2 *>(a.freqs)[p];
+  }
+  const float pos = a.pos_dev ? (float)((long)a.pos_dev[b] + a.pos_add) : a.pos_scalar;
+
+  const bool ae = xv.x != 0.0f, ao = xv.y != 0.0f;
+  const bool act = ae || ao;
+  const unsigned long long m_act = __ballot(act);
+
+  // element bitmask: two 64-bit words per wave (128 consecutive neurons)
+  if (a.bitmask) {
+    const unsigned long long me = __ballot(ae), mo = __ballot(ao);
+    if (lane == 0) {
+      const int w0 = (seg * PPB + wave * 64) >> 5;
+      const int NW = (a.N + 63) >> 6;
+      unsigned long long *bm = a.bitmask + (long)slice * a.bitmask_slice_stride;
+      if (w0 < NW) bm[w0] = spread_bits((unsigned int)me) | (spread_bits((unsigned int)mo) << 1);
+      if (w0 + 1 < NW)
+        bm[w0 + 1] = spread_bits((unsigned int)(me >> 32)) | (spread_bits((unsigned int)(mo >> 32)) << 1);
+    }
+  }
+
+  // rotate this lane's pair (src/model/attention.rs:305-321):
+  //   q[2j]   = x[2j]  *cos(ph[2j])   + (-x[2j+1])*sin(ph[2j])
+  //   q[2j+1] = x[2j+1]*cos(ph[2j+1]) +   x[2j]   *sin(ph[2j+1])
+  float2 q = make_float2(0.0f, 0.0f);
+  if (act) {
+    float s0, c0, s1, c1;
+    sincosf(rope_phase(pos, fv.x), &s0, &c0);
+    if (fv.y == fv.x) {
+      s1 = s0;
+      c1 = c0;
+    } else {
+      sincosf(rope_phase(pos, fv.y), &s1, &c1);
+    }
+    const float a0 = xv.x * c0, r0 = (-xv.y) * s0;
+    const float a1 = xv.y * c1, r1 = xv.x * s1;
+    q.x = a0 + r0;
+    q.y = a1 + r1;
+  }
+
+  // workgroup-wide compaction of the active pairs
+  if (lane == 0) s_cnt[wave] = __popcll(m_act);
+  __syncthreads();
+  int offset = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const int c = s_cnt[w];
+    if (w < wave) offset += c;
+    total += c;
+  }
+  if (act) {
+    const int rank = offset + __popcll(m_act & ((1ull << lane) - 1ull));
+    s_idx[rank] = (unsigned short)tid;
+    s_q[rank] = q;
+  }
+  __syncthreads();
+
+  float4 acc[VPL];
+  float4 vv[VPL];
+  {
+    const float4 *vrow = reinterpret_cast<const float4 *>(a.v + (long)b * a.v_batch_stride);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      vv[j] = vrow[j * 64 + lane];
+    }
+  }
+  float *base = rho + ((long)slice * a.N + 2L * seg * PPB) * D;
+
+  for (int i0 = wave; i0 < total; i0 += WAVES * U) {
+    float4 r0[U][VPL], r1[U][VPL];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * WAVES;
+      if (i < total) {
+        const float4 *rp = reinterpret_cast<const float4 *>(base + (long)s_idx[i] * (2 * D));
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          r0[u][j] = rp[j * 64 + lane];
+          r1[u][j] = rp[D / 4 + j * 64 + lane];
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * WAVES;
+      if (i < total) {
+        const float2 qq = s_q[i];
+        float4 *wp = reinterpret_cast<float4 *>(base + (long)s_idx[i] * (2 * D));
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          float4 e = r0[u][j], o = r1[u][j];
+          // readout with the old state (src/model/bdh.rs:293-295)
+          acc[j].x = __builtin_fmaf(e.x, qq.x, acc[j].x);
+          acc[j].y = __builtin_fmaf(e.y, qq.x, acc[j].y);
+          acc[j].z = __builtin_fmaf(e.z, qq.x, acc[j].z);
+          acc[j].w = __builtin_fmaf(e.w, qq.x, acc[j].w);
+          acc[j].x = __builtin_fmaf(o.x, qq.y, acc[j].x);
+          acc[j].y = __builtin_fmaf(o.y, qq.y, acc[j].y);
+          acc[j].z = __builtin_fmaf(o.z, qq.y, acc[j].z);
+          acc[j].w = __builtin_fmaf(o.w, qq.y, acc[j].w);
+          // rank-1 update: rho + (q*v), product rounded before the add (src/model/bdh.rs:298)
+          const float4 vj = vv[j];
+          float t;
+          t = qq.x * vj.x; e.x = e.x + t;
+          t = qq.x * vj.y; e.y = e.y + t;
+          t = qq.x * vj.z; e.z = e.z + t;
+          t = qq.x * vj.w; e.w = e.w + t;
+          t = qq.y * vj.x; o.x = o.x + t;
+          t = qq.y * vj.y; o.y = o.y + t;
+          t = qq.y * vj.z; o.z = o.z + t;
+          t = qq.y * vj.w; o.w = o.w + t;
+          wp[j * 64 + lane] = e;
+          wp[D / 4 + j * 64 + lane] = o;
+        }
+      }
+    }
+  }
+
+  // cross-wave reduction of the readout, fixed order
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) s_red[wave][j * 64 + lane] = acc[j];
+  __syncthreads();
+  float *pout = a.partial + (long)blockIdx.x * D;
+  for (int c4 = tid; c4 < D / 4; c4 += PPB) {
+    float4 s = s_red[0][c4];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      const float4 t = s_red[w][c4];
+      s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    reinterpret_cast<float4 *>(pout)[c4] = s;
+  }
+  if (tid == 0) a.pair_cnt[blockIdx.x] = total;
+}
+
+// ------------------------------------------------------------------------------------
+// generic path: any d <= 1024, any rotary, f32 or bf16 state.  One workgroup owns ROWS
+// state rows of one slice; waves take rows round-robin, lanes stride over columns.
+// ------------------------------------------------------------------------------------
+constexpr int kGenRows = 64;
+constexpr int kGenMaxCols = 16;  // d <= 64 * 16
+
+template <typename RhoT>
+__device__ __forceinline__ float rho_load(const RhoT *p);
+template <>
+__device__ __forceinline__ float rho_load<float>(const float *p) { return *p; }
+template <>
+__device__ __forceinline__ float rho_load<unsigned short>(const unsigned short *p) { return bf16_to_f32(*p); }
+__device__ __forceinline__ void rho_store(float *p, float v) { *p = v; }
+__device__ __forceinline__ void rho_store(unsigned short *p, float v) { *p = f32_to_bf16(v); }
+
+template <typename RhoT>
+__global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restrict__ rho, int d, int Nq,
+                                                      int rotary, int has_decay, HeadScalars decay) {
+  __shared__ float s_red[4][64 * kGenMaxCols];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slice = blockIdx.x / a.S;
+  const int seg = blockIdx.x - slice * a.S;
+  const int b = slice / a.h, hh = slice - b * a.h;
+  const float pos = a.pos_dev ? (float)((long)a.pos_dev[b] + a.pos_add) : a.pos_scalar;
+  const float *xs = a.x + (long)slice * a.x_slice_stride;
+  const float *vrow = a.v + (long)b * a.v_batch_stride;
+  const float dec = has_decay ? decay.v[hh] : 1.0f;
+  const int ncol = (d + 63) >> 6;
+
+  float acc[kGenMaxCols];
+#pragma unroll
+  for (int j = 0; j < kGenMaxCols; ++j) acc[j] = 0.0f;
+
+  for (int r = wave; r < kGenRows; r += 4) {
+    const int n = seg * kGenRows + r;
+    if (n >= Nq) break;
+    float qn;
+    bool touch;
+    if (rotary == BDH_ROPE) {
+      const float xn = xs[n], xo = xs[n ^ 1];
+      touch = (xn != 0.0f) || (xo != 0.0f);
+      float s, c;
+      sincosf(rope_phase(pos, a.freqs[n]), &s, &c);
+      const float rot = (n & 1) ? xo : -xo;
+      const float t0 = xn * c, t1 = rot * s;
+      qn = t0 + t1;
+    } else if (rotary == BDH_POPE) {
+      const int m = n < a.N ? n : n - a.N;
+      const float mag = softplus1(xs[m]);
+      const float ph = rope_phase(pos, a.freqs[m]);
+      qn = n < a.N ? mag * cosf(ph) : mag * sinf(ph);
+      touch = true;
+    } else {
+      qn = xs[n];
+      touch = (qn != 0.0f);
+    }
+    if (!touch && !has_decay) continue;
+    RhoT *row = rho + ((long)slice * Nq + n) * d;
+#pragma unroll
+    for (int j = 0; j < kGenMaxCols; ++j) {
+      const int c = j * 64 + lane;
+      if (j < ncol && c < d) {
+        float rv = rho_load<RhoT>(row + c);
+        acc[j] = __builtin_fmaf(rv, qn, acc[j]);
+        const float outer = qn * vrow[c];
+        rv = rv + outer;
+        if (has_decay) rv = rv * dec;  // src/model/bdh.rs:299-301
+        rho_store(row + c, rv);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kGenMaxCols; ++j) s_red[wave][j * 64 + lane] = acc[j];
+  __syncthreads();
+  float *pout = a.partial + (long)blockIdx.x * d;
+  for (int c = tid; c < d; c += 256) {
+    float s = s_red[0][c];
+    s += s_red[1][c];
+    s += s_red[2][c];
+    s += s_red[3][c];
+    pout[c] = s;
+  }
+}
+
+// bitmask + touched-row count for the generic path: one workgroup per slice
+__global__ __launch_bounds__(256) void k_bitmask_rows(StepPtrs a, int rotary, int Nq, int *__restrict__ rows,
+                                                      long rows_slice_stride) {
+  __shared__ int s_pairs[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slice = blockIdx.x;
+  const float *xs = a.x + (long)slice * a.x_slice_stride;
+  const int NW = (a.N + 63) >> 6;
+  int pairs = 0;
+  for (int w = wave; w < NW; w += 4) {
+    const int n = w * 64 + lane;
+    const float xv = n < a.N ? xs[n] : 0.0f;
+    const unsigned long long m = __ballot(xv != 0.0f);
+    if (a.bitmask && lane == 0) a.bitmask[(long)slice * a.bitmask_slice_stride + w] = m;
+    const unsigned long long pm = (m | (m >> 1)) & 0x5555555555555555ull;
+    pairs += __popcll(pm);
+  }
+  if (lane == 0) s_pairs[wave] = pairs;
+  __syncthreads();
+  if (tid == 0 && rows) {
+    const int np = s_pairs[0] + s_pairs[1] + s_pairs[2] + s_pairs[3];
+    rows[(long)slice * rows_slice_stride] = rotary == BDH_ROPE ? 2 * np : Nq;
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// second stage: out[slice,:] = sum over the S partials in index order; optional
+// LayerNorm of the result (src/model/bdh.rs:359) and touched-row count.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__ partial,
+                                                       const int *__restrict__ pair_cnt, int S, int d,
+                                                       float *__restrict__ out, long out_slice_stride,
+                                                       float *__restrict__ out_ln, int *__restrict__ rows,
+                                                       long rows_slice_stride) {
+  __shared__ float s_part[4];
+  __shared__ float s_stat[2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slice = blockIdx.x;
+  const float *p = partial + (long)slice * S * d;
+  float vals[4];  // d <= 1024
+  float lsum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 256 + tid;
+    float s = 0.0f;
+    if (c < d) {
+      for (int g = 0; g < S; ++g) s += p[(long)g * d + c];
+      out[(long)slice * out_slice_stride + c] = s;
+      lsum += s;
+    }
+    vals[j] = s;
+  }
+  if (rows && pair_cnt && tid == 0) {
+    int np = 0;
+    for (int g = 0; g < S; ++g) np += pair_cnt[(long)slice * S + g];
+    rows[(long)slice * rows_slice_stride] = 2 * np;
+  }
+  if (!out_ln) return;
+  // LayerNorm over d: mean, biased variance, (x-mean)/sqrt(var+eps)
+  for (int o = 32; o > 0; o >>= 1) lsum += __shfl_xor(lsum, o);
+  if (lane == 0) s_part[wave] = lsum;
+  __syncthreads();
+  if (tid == 0) s_stat[0] = (s_part[0] + s_part[1] + s_part[2] + s_part[3]) / (float)d;
+  __syncthreads();
+  const float mean = s_stat[0];
+  float lsq = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 256 + tid;
+    if (c < d) {
+      const float t = vals[j] - mean;
+      lsq += t * t;
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) lsq += __shfl_xor(lsq, o);
+  __syncthreads();
+  if (lane == 0) s_part[wave] = lsq;
+  __syncthreads();
+  if (tid == 0) s_stat[1] = sqrtf((s_part[0] + s_part[1] + s_part[2] + s_part[3]) / (float)d + 1e-5f);
+  __syncthreads();
+  const float den = s_stat[1];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 256 + tid;
+    if (c < d) out_ln[(long)slice * out_slice_stride + c] = (vals[j] - mean) / den;
+  }
+}
+
+template <int D, int WAVES, int U>
+void launch_fast(hipStream_t st, int blocks, const StepPtrs &a, float *rho) {
+  hipLaunchKernelGGL((k_step_rope_f32<D, WAVES, U>), dim3(blocks), dim3(WAVES * 64), 0, st, a, rho);
+}
+
+}  // namespace
+
+int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out_ln) {
+  const int B = p.B, h = p.h, T = p.T, N = p.N, d = p.d;
+  const int Nq = p.rotary == BDH_POPE ? 2 * N : N;
+  const int slices = B * h;
+  if (d > 64 * kGenMaxCols) return bdh_fail(ctx, BDH_E_SHAPE, "d=%d exceeds the supported maximum %d", d, 64 * kGenMaxCols);
+  if (N > 65536 * 2 && p.rotary == BDH_ROPE) { /* pair index within a workgroup is 16 bit: always fits */ }
+  if ((long)slices > 0x7fffffffL / 4096) return bdh_fail(ctx, BDH_E_SHAPE, "B*h too large");
+
+  const bool fast = p.rotary == BDH_ROPE && p.rho_dtype == BDH_F32 && (d == 256 || d == 512) && N >= 2;
+  constexpr int WAVES = 4;
+  const int S = fast ? ((N / 2) + WAVES * 64 - 1) / (WAVES * 64) : (Nq + kGenRows - 1) / kGenRows;
+  if (N == 0 || d == 0) {
+    // nothing to read or update: the readout is an empty sum
+    if (d > 0) BDH_HIP_CHECK(ctx, hipMemsetAsync(p.out, 0, sizeof(float) * (size_t)slices * T * d, ctx->stream));
+    if (out_ln && d > 0) return bdh_fail(ctx, BDH_E_SHAPE, "LayerNorm of an empty readout");
+    if (p.rows_touched) BDH_HIP_CHECK(ctx, hipMemsetAsync(p.rows_touched, 0, sizeof(int32_t) * (size_t)slices * T, ctx->stream));
+    return BDH_OK;
+  }
+  const size_t partial_bytes = bdh_align_up(sizeof(float) * (size_t)slices * S * d, 256);
+  const size_t cnt_bytes = bdh_align_up(sizeof(int) * (size_t)slices * S, 256);
+  int rc = bdh_ws_reserve(ctx, partial_bytes + cnt_bytes);
+  if (rc != BDH_OK) return rc;
+  float *partial = static_cast<float *>(ctx->ws);
+  int *pair_cnt = reinterpret_cast<int *>(static_cast<char *>(ctx->ws) + partial_bytes);
+
+  HeadScalars decay{};
+  const int has_decay = p.rotary == BDH_ALIBI;
+  if (has_decay)
+    for (int i = 0; i < h; ++i) decay.v[i] = expf(-p.slopes_host[i]);  // src/model/attention.rs:181-186
+
+  const int NW = (N + 63) / 64;
+  for (int t = 0; t < T; ++t) {
+    StepPtrs a{};
+    a.x = p.x + (long)t * N;
+    a.x_slice_stride = (long)T * N;
+    a.v = p.v + (long)t * d;
+    a.v_batch_stride = (long)T * d;
+    a.freqs = p.freqs;
+    a.pos_scalar = (float)(p.position + (int64_t)t);
+    a.pos_dev = p.positions_dev;
+    a.pos_add = t;
+    a.partial = partial;
+    a.pair_cnt = pair_cnt;
+    a.bitmask = p.bitmask ? reinterpret_cast<unsigned long long *>(p.bitmask) + (long)t * NW : nullptr;
+    a.bitmask_slice_stride = (long)T * NW;
+    a.h = h;
+    a.N = N;
+    a.S = S;
+    float *out_t = p.out + (long)t * d;
+    float *out_ln_t = out_ln ? out_ln + (long)t * d : nullptr;
+    int32_t *rows_t = p.rows_touched ? p.rows_touched + t : nullptr;
+    if (fast) {
+      float *rho = static_cast<float *>(p.rho);
+      if (d == 256)
+        launch_fast<256, WAVES, 4>(ctx->stream, slices * S, a, rho);
+      else
+        launch_fast<512, WAVES, 2>(ctx->stream, slices * S, a, rho);
+      BDH_LAUNCH_CHECK(ctx, "k_step_rope_f32");
+      hipLaunchKernelGGL(k_step_finalize, dim3(slices), dim3(256), 0, ctx->stream, partial, pair_cnt, S, d,
+                         out_t, (long)T * d, out_ln_t, rows_t, (long)T);
+      BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
+    } else {
+      if (p.rho_dtype == BDH_F32)
+        hipLaunchKernelGGL(k_step_generic<float>, dim3(slices * S), dim3(256), 0, ctx->stream, a,
+                           static_cast<float *>(p.rho), d, Nq, p.rotary, has_decay, decay);
+      else
+        hipLaunchKernelGGL(k_step_generic<unsigned short>, dim3(slices * S), dim3(256), 0, ctx->stream, a,
+                           static_cast<unsigned short *>(p.rho), d, Nq, p.rotary, has_decay, decay);
+      BDH_LAUNCH_CHECK(ctx, "k_step_generic");
+      hipLaunchKernelGGL(k_step_finalize, dim3(slices), dim3(256), 0, ctx->stream, partial,
+                         (const int *)nullptr, S, d, out_t, (long)T * d, out_ln_t, (int *)nullptr, (long)T);
+      BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
+      if (a.bitmask || rows_t) {
+        hipLaunchKernelGGL(k_bitmask_rows, dim3(slices), dim3(256), 0, ctx->stream, a, p.rotary, Nq, rows_t,
+                           (long)T);
+        BDH_LAUNCH_CHECK(ctx, "k_bitmask_rows");
+      }
+    }
+  }
+  return BDH_OK;
+}
+
+int bdh_launch_state_steps(bdh_ctx *ctx, const StateStepParams &p) {
+  return bdh_launch_state_steps_ln(ctx, p, nullptr);
+}

@@ -1,0 +1,43 @@
+"""LayerState / ModelState (reference: src/model/state.rs:5-57)."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import torch
+
+
+@dataclass
+class LayerState:
+    rho: Optional[torch.Tensor] = None  # [B,h,Nq,d]
+
+
+@dataclass
+class ModelState:
+    layers: List[LayerState] = field(default_factory=list)
+    position: int = 0
+    # all layers share one allocation [L,B,h,Nq,d]; layers[i].rho are views into it
+    storage: Optional[torch.Tensor] = None
+
+    @classmethod
+    def new(cls, num_layers: int) -> "ModelState":
+        return cls(layers=[LayerState() for _ in range(num_layers)], position=0)
+
+    def reset(self) -> None:
+        for layer in self.layers:
+            layer.rho = None
+        self.storage = None
+        self.position = 0
+
+    def len(self) -> int:
+        return self.position
+
+    def __len__(self) -> int:
+        return self.position
+
+    def is_empty(self) -> bool:
+        return self.position == 0
+
+    def trim(self, max_len: int) -> None:
+        """A no-op, as in the reference (src/model/state.rs:55-57)."""
+        _ = max_len

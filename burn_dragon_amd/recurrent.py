@@ -1,0 +1,54 @@
+"""The recurrent state step through the C ABI (reference: BDH::recurrent_attention,
+src/model/bdh.rs:258-307, including the rotate at :265)."""
+from __future__ import annotations
+
+from typing import Optional
+
+import numpy as np
+import torch
+
+from . import ffi
+from .positional import RotaryEmbedding
+
+
+def recurrent_attention(query: torch.Tensor, value: torch.Tensor, rho: torch.Tensor, freqs: torch.Tensor,
+                        position: int, rotary_embedding: RotaryEmbedding = RotaryEmbedding.ROPE,
+                        alibi_slopes=None, positions: Optional[torch.Tensor] = None, want_bitmask: bool = False,
+                        want_rows: bool = False, ctx: Optional[ffi.Context] = None):
+    """query [B,h,T,N] (un-rotated), value [B,1,T,d] or [B,T,d], rho [B,h,Nq,d] (updated in
+    place, f32 or bf16).  Returns out [B,h,T,d] (+ bitmask [B,h,T,ceil(N/64)] int64 view of the
+    uint64 words, + rows_touched [B,h,T] int32 when asked)."""
+    ctx = ctx or ffi.default_context(query.device.index or 0)
+    B, h, T, N = query.shape
+    d = value.shape[-1]
+    rot = RotaryEmbedding.parse(rotary_embedding)
+    Nq = 2 * N if rot == RotaryEmbedding.POPE else N
+    assert query.dtype == torch.float32 and query.is_contiguous()
+    value = value.reshape(B, T, d)
+    assert value.dtype == torch.float32 and value.is_contiguous()
+    assert rho.is_contiguous() and tuple(rho.shape) == (B, h, Nq, d), "rho must be [B,h,Nq,d]"
+    dt = {torch.float32: ffi.F32, torch.bfloat16: ffi.BF16}[rho.dtype]
+    freqs = freqs.reshape(-1)
+    out = torch.empty((B, h, T, d), device=query.device, dtype=torch.float32)
+    bm = torch.zeros((B, h, T, (N + 63) // 64), device=query.device, dtype=torch.int64) if want_bitmask else None
+    rows = torch.zeros((B, h, T), device=query.device, dtype=torch.int32) if want_rows else None
+    slopes = None if alibi_slopes is None else np.ascontiguousarray(alibi_slopes, np.float32)
+    ctx.check(ctx.lib.bdh_recurrent_attention(ctx.handle, B, h, T, N, d, int(rot), ffi.ptr(query), ffi.ptr(value),
+                                              ffi.ptr(freqs), int(position), ffi.ptr(positions), ffi.ptr(slopes),
+                                              ffi.ptr(rho), dt, ffi.ptr(out), ffi.ptr(bm), ffi.ptr(rows)))
+    res = [out]
+    if want_bitmask:
+        res.append(bm)
+    if want_rows:
+        res.append(rows)
+    return res[0] if len(res) == 1 else tuple(res)
+
+
+def layer_norm(x: torch.Tensor, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
+    """BDH::layer_norm (src/model/bdh.rs:86-89)."""
+    ctx = ctx or ffi.default_context(x.device.index or 0)
+    x = x.contiguous().float()
+    out = torch.empty_like(x)
+    d = x.shape[-1]
+    ctx.check(ctx.lib.bdh_layer_norm(ctx.handle, x.numel() // max(d, 1), d, ffi.ptr(x), ffi.ptr(out)))
+    return out

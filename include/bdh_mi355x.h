@@ -1,0 +1,223 @@
+/*
+ * bdh_mi355x.h — C ABI of libbdh_mi355x.so: the BDH (Dragon Hatchling) cached-inference
+ * hot path of mosure/burn_dragon, hand-written for AMD MI355X (gfx950, CDNA4).
+ *
+ * The reference has no FFI of its own: the path sits behind generic Rust functions over
+ * burn::tensor::Tensor (src/lib.rs:8,31-38).  Each entry point below names the reference
+ * function it replaces (paths relative to the reference tree); a Rust `-sys` crate or any
+ * other FFI binds exactly these symbols.
+ *
+ * Conventions
+ *   - All `const float*` / `void*` data arguments are caller-owned DEVICE pointers unless
+ *     the parameter name ends in `_host`.  Tensors are row-major contiguous, last index
+ *     fastest, in the reference's layouts.
+ *   - Calls are asynchronous: work is enqueued on the context's HIP stream and the call
+ *     returns; the caller synchronises the stream before reading results on the host.
+ *   - Every function returns 0 (BDH_OK) or a negative bdh_status.  Nothing aborts or throws
+ *     across this boundary (the reference panics on contract violations:
+ *     src/model/bdh.rs:314-318, src/model/config.rs:143-153).  bdh_last_error() gives the
+ *     text of the last failure on a context.
+ *   - A context is not re-entrant; independent contexts may be used from different threads.
+ *   - There is no CPU fallback: without a HIP device every compute entry point fails.
+ */
+#ifndef BDH_MI355X_H
+#define BDH_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct bdh_ctx bdh_ctx;     /* opaque: device, stream, workspace */
+typedef struct bdh_model bdh_model; /* opaque: weights view + per-model tables */
+
+enum bdh_status {
+  BDH_OK = 0,
+  BDH_E_INVAL = -1,       /* null pointer / bad enum / bad scalar */
+  BDH_E_SHAPE = -2,       /* dimension not supported (e.g. odd latent with RoPE) */
+  BDH_E_ALIGN = -3,       /* pointer not aligned as required */
+  BDH_E_HIP = -4,         /* a HIP runtime call failed */
+  BDH_E_NOMEM = -5,       /* workspace allocation failed */
+  BDH_E_UNSUPPORTED = -6  /* combination not implemented */
+};
+
+/* src/positional.rs:8-15 (RotaryEmbedding; Alibi is the reference's default) */
+enum bdh_rotary { BDH_ROPE = 0, BDH_ALIBI = 1, BDH_POPE = 2 };
+
+/* storage type of the recurrent state rho.  The reference keeps it in f32; bf16 storage
+ * with f32 accumulation is an extension of this library. */
+enum bdh_dtype { BDH_F32 = 0, BDH_BF16 = 1 };
+
+/* ---- library / context ------------------------------------------------------------ */
+const char *bdh_version(void);
+const char *bdh_status_string(int status);
+
+/* hip_stream: a hipStream_t (NULL = the default stream).  Replaces the Burn device handle
+ * every reference call receives (`&B::Device`, e.g. src/model/bdh.rs:37). */
+int bdh_ctx_create(int device_id, void *hip_stream, bdh_ctx **out);
+int bdh_ctx_destroy(bdh_ctx *ctx);
+int bdh_ctx_set_stream(bdh_ctx *ctx, void *hip_stream);
+int bdh_ctx_synchronize(bdh_ctx *ctx);
+const char *bdh_last_error(const bdh_ctx *ctx);
+
+/* ---- host-side tables (computed on the host in the reference as well) --------------- */
+/* src/model/attention.rs:351-373  Attention::build_freqs -> freqs_host[latent] */
+int bdh_build_freqs(int latent, float theta, int rotary, float *freqs_host);
+/* src/kernel/linear_attention.rs:152-163  default_alibi_slopes -> slopes_host[n_head] */
+int bdh_default_alibi_slopes(int n_head, float *slopes_host);
+
+/* ---- a5 + a4: the recurrent state step ------------------------------------------- */
+/*
+ * Replaces BDH::recurrent_attention (src/model/bdh.rs:258-307) including the
+ * rotate_positions call at :265 (src/model/attention.rs:332-349, rope :305-321,
+ * pope :323-330).
+ *
+ *   x        [B,h,T,N]   un-rotated sparse activations (the `query` argument)
+ *   v        [B,T,d]     value = the layer input `current` [B,1,T,d], shared by heads
+ *   freqs    [N]         table from bdh_build_freqs (ignored for BDH_ALIBI)
+ *   position             start position of token 0 (state.position, src/model/bdh.rs:334)
+ *   positions_dev        optional DEVICE int32[B]: per-sequence start positions that
+ *                        override `position` (NULL = one shared position as in the
+ *                        reference, src/model/state.rs:14)
+ *   alibi_slopes_host    host float[h], BDH_ALIBI only (NULL = default slopes); after every
+ *                        token rho[:,h] is scaled by exp(-slope_h) (src/model/bdh.rs:299-301)
+ *   rho      [B,h,Nq,d]  recurrent state, updated IN PLACE (the reference moves it out and
+ *                        back, :274,:304, so the step owns it); Nq = N, or 2N for BDH_POPE.
+ *                        The caller zero-fills it where the reference would create zeros
+ *                        (:274-284).
+ *   out      [B,h,T,d]   out_t = sum_n rho_before_t[n,:] * q_t[n]   (readout BEFORE update)
+ *   active_bitmask       optional uint64 [B,h,T,ceil(N/64)]: bit n%64 of word n/64 is set
+ *                        iff x[b,h,t,n] != 0 (== x > 0 for ReLU outputs)
+ *   rows_touched         optional int32 [B,h,T]: number of state rows read and written for
+ *                        that token (RoPE: both rows of every lane pair with a non-zero
+ *                        element; ALiBi/PoPE: Nq)
+ *
+ * RoPE requires even N (src/model/attention.rs:310).  T = 1 is the decode step.
+ */
+int bdh_recurrent_attention(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary,
+                            const float *x, const float *v, const float *freqs,
+                            int64_t position, const int32_t *positions_dev,
+                            const float *alibi_slopes_host, void *rho, int rho_dtype,
+                            float *out, uint64_t *active_bitmask, int32_t *rows_touched);
+
+/* The decode step: bdh_recurrent_attention with T = 1 (x [B,h,N], v [B,d], out [B,h,d]). */
+int bdh_state_step(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const float *x,
+                   const float *v, const float *freqs, int64_t position,
+                   const int32_t *positions_dev, const float *alibi_slopes_host, void *rho,
+                   int rho_dtype, float *out, uint64_t *active_bitmask,
+                   int32_t *rows_touched);
+
+/* ---- a3 / a7: ReLU low-rank projection ------------------------------------------- */
+/*
+ * Replaces kernel::relu_lowrank::fused_forward (src/kernel/relu_lowrank.rs:7-37) and the
+ * unfused sequence at src/model/bdh.rs:346-350 and :370-374.
+ *
+ *   in      [B,h_in,T,d]  h_in = 1 (shared by heads, the D_x call) or h (the D_y call)
+ *   weight  [h,d,N]
+ *   bias    [h,N] or NULL                       (relu_lowrank.rs:19-23)
+ *   threshold                                   (relu_lowrank.rs:25-27)
+ *   block_size, active_blocks_host[n_blocks]    BlockPattern1d (src/kernel/block_sparse.rs:
+ *                        11-63): one byte per latent block, NULL = dense pattern
+ *   gate    [B,h,T,N] or NULL: when given, out = gate * relu(...) (the x (.) y product of
+ *                        src/model/bdh.rs:380 fused into the D_y projection)
+ *   out     [B,h,T,N] = relu(in . weight + bias - threshold) * mask
+ *
+ * Each output element is one k-sequential f32 fused-multiply-add chain, so the set
+ * {n : out > 0} does not depend on the launch shape.
+ */
+int bdh_relu_lowrank(bdh_ctx *ctx, int B, int h_in, int T, int d, int h, int N,
+                     const float *in, const float *weight, const float *bias, float threshold,
+                     int block_size, const uint8_t *active_blocks_host, int n_blocks,
+                     const float *gate, float *out);
+
+/* BDH::layer_norm (src/model/bdh.rs:86-89): biased variance, eps 1e-5, no affine.
+ * in/out [rows,d]; in == out is allowed. */
+int bdh_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);
+
+/* ---- a10: parallel (training-path) causal linear attention ------------------------- */
+/*
+ * Replaces kernel::linear_attention::fused_state_aligned (src/kernel/linear_attention.rs:
+ * 11-115) and, with the dense pattern, Attention::forward (src/model/attention.rs:142-175).
+ *   query [B,h,T,N] un-rotated, value [B,T,dv] (dim 1 of size 1 repeated over heads),
+ *   freqs [N], alibi_slopes_host [h] or NULL, time-block size and optional sparse
+ *   (row,col) block pairs (BlockPattern2d, src/kernel/block_sparse.rs:66-117),
+ *   positions 0..T.  out [B,h,T,dv] = (sum of masked score blocks . V) / (sum|score| + 1e-6).
+ *   row_normalize = 0 drops the division and gives the un-normalised causal form that
+ *   equals the recurrent path.
+ */
+int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N, int dv,
+                            const float *query, const float *value, const float *freqs,
+                            const float *alibi_slopes_host, int block_size,
+                            const int32_t *block_pairs_host, int n_pairs, int rotary,
+                            int row_normalize, float *out);
+
+/* ---- chunked prefill (dense MFMA form of the recurrent path) ------------------------ */
+/*
+ * The recurrent path of src/model/bdh.rs:258-307 for T tokens at once, RoPE only, computed
+ * chunk-wise on the bf16 matrix cores with f32 accumulation:
+ *   out_c = tril(-1)(Q_c Q_c^T) V_c + Q_c rho ;  rho += Q_c^T V_c      per chunk c
+ * The reference has no such function (its prefill walks tokens serially, src/generation.rs:
+ * 74-104); the sequential loop is the definition of the result.
+ *   x   [B,h,T,N] bf16 (raw 16-bit) un-rotated activations
+ *   v   [B,T,d]   bf16
+ *   rho [B,h,N,d] f32 in/out,  out [B,h,T,d] f32
+ */
+int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
+                        const uint16_t *v_bf16, const float *freqs, int64_t position,
+                        float *rho, float *out);
+
+/* ---- a1: the whole cached step ------------------------------------------------------- */
+/* src/model/config.rs:113-164 (BDHConfig) + :10-31 (FusedKernelConfig), as plain scalars */
+typedef struct bdh_model_config {
+  int32_t n_layer;
+  int32_t n_embd;   /* d */
+  int32_t n_head;   /* h */
+  int32_t latent;   /* N per head = mlp_internal_dim_multiplier * n_embd / n_head */
+  int32_t vocab;    /* V */
+  int32_t rotary;   /* enum bdh_rotary */
+  float rope_theta;      /* 65536 */
+  float relu_threshold;  /* 0 */
+  const float *alibi_slopes_host; /* [h] or NULL */
+} bdh_model_config;
+
+/* device pointers, in the record order of the reference module (src/model/bdh.rs:27-33) */
+typedef struct bdh_model_weights {
+  const float *embed;     /* [V,d] */
+  const float *encoder;   /* [h,d,N]   D_x */
+  const float *encoder_v; /* [h,d,N]   D_y */
+  const float *decoder;   /* [h*N,d]   E   */
+  const float *lm_head;   /* [d,V] */
+} bdh_model_weights;
+
+/* Replaces BDH::new as far as inference needs it (src/model/bdh.rs:37-84): records the
+ * weight pointers (not copied; they must outlive the model) and builds the freqs table
+ * (Attention::new, src/model/attention.rs:113-140). */
+int bdh_model_create(bdh_ctx *ctx, const bdh_model_config *config,
+                     const bdh_model_weights *weights, bdh_model **out);
+int bdh_model_destroy(bdh_model *model);
+
+/* bytes of recurrent state for one sequence batch: L * B * h * Nq * d * sizeof(rho_dtype)
+ * (ModelState, src/model/state.rs:5-15; one rho per layer) */
+size_t bdh_model_state_bytes(const bdh_model *model, int B, int rho_dtype);
+
+/*
+ * Replaces BDH::forward_with_state (src/model/bdh.rs:309-450).
+ *   tokens   [B,T] int64 device
+ *   rho      [L,B,h,Nq,d] in place; zero-filled by the caller for a fresh state
+ *   position state.position before the call; the caller advances it by T afterwards
+ *            (src/model/bdh.rs:445)
+ *   logits   [B,T,V]
+ *   next_tokens  optional int64 [B] device: argmax of the last position's logits (greedy
+ *            decoding, the top_k = 1 case of src/generation.rs:26-72, kept on the device)
+ *   x_tap    optional [L,B,h,T,N]: the sparse activations x of every layer
+ */
+int bdh_model_forward(bdh_model *model, const int64_t *tokens, int B, int T, void *rho,
+                      int rho_dtype, int64_t position, float *logits, int64_t *next_tokens,
+                      float *x_tap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BDH_MI355X_H */

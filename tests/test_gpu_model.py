@@ -1,0 +1,204 @@
+"""GPU parity of the projections (relu_lowrank, layer_norm) and of the whole cached step
+(BDH::forward_with_state) against the CPU oracle, through the C ABI.
+
+Tolerance for logits: 1e-3 relative on the max-norm (north_star, f32 state).  Active-neuron
+sets of the first layer are bit-exact against the oracle (both sides evaluate one k-sequential
+f32 FMA chain per pre-activation); deeper layers inherit readout reassociation noise, so their
+sets are compared away from zero pre-activations and the mismatch count is reported.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bdh_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def bda():
+    if not torch.cuda.is_available():
+        pytest.fail("no HIP device: the GPU tests must run on the MI355X box")
+    import burn_dragon_amd
+
+    return burn_dragon_amd
+
+
+def rel_err(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def assert_close(lhs, rhs, atol, rtol):
+    lhs, rhs = np.asarray(lhs, np.float64), np.asarray(rhs, np.float64)
+    assert lhs.shape == rhs.shape
+    assert not (np.abs(lhs - rhs) > atol + rtol * np.abs(rhs)).any(), f"max diff {np.abs(lhs - rhs).max()}"
+
+
+def test_relu_lowrank_fused_matches_reference(bda):
+    """tests/fused_kernel_tests.rs:35-68 on the device path: input [2,1,5,6], weight [1,3,6,8],
+    bias [3,1,8], threshold 0.25, BlockPattern1d::from_blocks(3,[0,2]); atol = rtol = 1e-5."""
+    from burn_dragon_amd.kernel import relu_lowrank
+
+    g = torch.Generator().manual_seed(42)
+    inp = torch.randn((2, 1, 5, 6), generator=g)
+    weight = torch.randn((1, 3, 6, 8), generator=g)
+    bias = 0.5 * torch.randn((3, 1, 8), generator=g)
+    layout = bda.BlockPattern1d.from_blocks(3, [0, 2])
+    fused = relu_lowrank.fused_forward(inp.to(DEV), weight.to(DEV), bias.to(DEV), 0.25, layout)
+    reference = torch.relu(inp.double().matmul(weight.double()) + bias.double().reshape(1, 3, 1, 8) - 0.25)
+    reference = reference * torch.tensor([1, 1, 1, 0, 0, 0, 1, 1], dtype=torch.float64)
+    assert_close(fused.cpu().numpy(), reference.numpy(), 1e-5, 1e-5)
+
+
+@pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (32, 1, 1), (1, 64, 4)])
+def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
+    """One k-sequential FMA chain per output on both sides: values, and therefore the active
+    sets, are identical bit for bit whatever the launch tiling."""
+    from burn_dragon_amd.kernel import relu_lowrank
+
+    h, d, N = 4, 256, 640
+    rng = np.random.default_rng(B * 100 + T)
+    inp = rng.standard_normal((B, h_in, T, d)).astype(np.float32)
+    weight = (0.02 * rng.standard_normal((h, d, N))).astype(np.float32)
+    gate = np.maximum(rng.standard_normal((B, h, T, N)), 0).astype(np.float32)
+    ref = corc.relu_lowrank(inp, weight)
+    got = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
+                                     bda.BlockPattern1d.dense(64))
+    assert np.array_equal(got.cpu().numpy(), ref)
+    assert 0.4 < (ref > 0).mean() < 0.6
+    gated = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
+                                       bda.BlockPattern1d.dense(64), gate=torch.from_numpy(gate).to(DEV))
+    assert np.array_equal(gated.cpu().numpy(), gate * ref)
+
+
+def test_layer_norm_matches_oracle_and_library(bda, corc):
+    from burn_dragon_amd.recurrent import layer_norm
+
+    rng = np.random.default_rng(3)
+    for d in (16, 256, 512, 1000):
+        x = (2.0 * rng.standard_normal((7, 3, d)) + 0.5).astype(np.float32)
+        got = layer_norm(torch.from_numpy(x).to(DEV)).cpu().numpy()
+        assert_close(got, corc.layer_norm(x), 2e-6, 1e-5)
+        assert_close(got, torch.nn.functional.layer_norm(torch.from_numpy(x), (d,), eps=1e-5).numpy(), 2e-6, 1e-5)
+
+
+def _shape_from_cfg(cfg):
+    return orc.BDHShape(n_layer=cfg.n_layer, n_embd=cfg.n_embd, n_head=cfg.n_head,
+                        mlp_internal_dim_multiplier=cfg.mlp_internal_dim_multiplier, vocab_size=cfg.vocab_size,
+                        rotary=int(cfg.fused_kernels.rotary_embedding), rope_theta=cfg.fused_kernels.rope_theta,
+                        relu_threshold=cfg.fused_kernels.relu_threshold, alibi_slopes=cfg.fused_kernels.alibi_slopes)
+
+
+def _model_pair(bda, cfg, seed):
+    shape = _shape_from_cfg(cfg)
+    w = orc.init_weights(shape, seed)
+    model = bda.BDH(cfg, DEV, weights={"embed": w.embed, "encoder": w.encoder, "encoder_v": w.encoder_v,
+                                       "decoder": w.decoder, "lm_head": w.lm_head})
+    return shape, w, model
+
+
+@pytest.mark.parametrize("rotary", ["rope", "pope", "alibi"])
+def test_inference_paths_run_across_configs(bda, corc, rotary):
+    """tests/model_paths.rs:66-91: L=2, d=16, h=2, mult=4, V=32, tokens [[0,1,2,3],[4,5,6,7]] ->
+    logits [2,4,32], state.position == 4 — plus the values, against the oracle."""
+    cfg = bda.BDHConfig(n_layer=2, n_embd=16, n_head=2, mlp_internal_dim_multiplier=4, vocab_size=32, dropout=0.0)
+    cfg.fused_kernels.set_block_sizes(4, 4)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse(rotary))
+    shape, w, model = _model_pair(bda, cfg, seed=11)
+    tokens = np.arange(8).reshape(2, 4)
+    state = model.init_state()
+    logits = model.forward_with_state(torch.from_numpy(tokens), state)
+    torch.cuda.synchronize()
+    assert tuple(logits.shape) == (2, 4, 32)
+    assert state.position == 4
+    Nq = model.latent_q
+    rho_ref = np.zeros((2, 2, 2, Nq, 16), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, tokens, rho_ref, 0, sparse_state=False)
+    assert pos == 4
+    assert rel_err(logits.cpu().numpy(), logits_ref) < 1e-3
+    assert rel_err(state.storage.cpu().numpy(), rho_ref) < 1e-3
+    # a second call continues from the stored state and position
+    more = np.array([[9], [10]])
+    logits2 = model.forward_with_state(torch.from_numpy(more), state)
+    logits2_ref, pos, _, _ = corc.forward_with_state(shape, w, more, rho_ref, 4, sparse_state=False)
+    assert state.position == 5 == pos
+    assert rel_err(logits2.cpu().numpy(), logits2_ref) < 1e-3
+
+
+def test_config1_architecture_prefill_and_greedy_decode(bda, corc):
+    """BASELINE config 1 architecture (V=256, d=256, h=4, N=8192, RoPE) with L=2 and a short
+    run so the oracle finishes in seconds: 16-byte prompt, 8 greedy tokens, batch 1."""
+    cfg = bda.BDHConfig(n_layer=2, n_embd=256, n_head=4, mlp_internal_dim_multiplier=128, vocab_size=256)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    shape, w, model = _model_pair(bda, cfg, seed=5)
+    assert model.latent == 8192
+    rng = np.random.default_rng(0)
+    prompt = rng.integers(0, 256, size=(1, 16))
+    L, h, N, d = 2, 4, 8192, 256
+    state = model.init_state()
+    x_tap = torch.zeros((L, 1, h, 16, N), device=DEV)
+    logits, nxt = model.forward_with_state(torch.from_numpy(prompt), state, want_next=True, x_tap=x_tap)
+    torch.cuda.synchronize()
+    rho_ref = np.zeros((L, 1, h, N, d), np.float32)
+    logits_ref, pos, x_ref, _ = corc.forward_with_state(shape, w, prompt, rho_ref, 0, taps=True)
+    assert rel_err(logits.cpu().numpy(), logits_ref) < 1e-3
+    # active sets: layer 0 bit-exact; deeper layers identical wherever |pre-activation| is not ~0
+    x_gpu = x_tap.cpu().numpy()
+    assert np.array_equal(x_gpu[0] > 0, x_ref[0] > 0)
+    assert np.array_equal(x_gpu[0], x_ref[0])
+    flips = ((x_gpu[1] > 0) != (x_ref[1] > 0))
+    assert flips.mean() < 1e-3
+    assert np.maximum(x_gpu[1], x_ref[1])[flips].max(initial=0.0) < 1e-4
+    dens = (x_ref > 0).mean()
+    assert 0.4 < dens < 0.6  # random-init weights: about half the neurons fire
+    tokens_gpu, tokens_ref = [], []
+    tok_ref = corc.greedy_token(logits_ref[0, -1])
+    assert int(nxt[0]) == tok_ref
+    position = pos
+    for _ in range(8):
+        tokens_ref.append(tok_ref)
+        tokens_gpu.append(int(nxt[0]))
+        lg, nxt = model.forward_with_state(nxt.reshape(1, 1), state, want_next=True)
+        lr, position, _, _ = corc.forward_with_state(shape, w, np.array([[tok_ref]]), rho_ref, position)
+        assert rel_err(lg.cpu().numpy(), lr) < 1e-3
+        tok_ref = corc.greedy_token(lr[0, -1])
+    assert tokens_gpu == tokens_ref
+    assert state.position == 24 == position
+    assert rel_err(state.storage.cpu().numpy(), rho_ref) < 1e-3
+
+
+def test_decode_equals_prefill_on_device(bda):
+    """T tokens in one call == T single-token calls carrying the state."""
+    cfg = bda.BDHConfig(n_layer=3, n_embd=256, n_head=4, mlp_internal_dim_multiplier=8, vocab_size=64)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    model = bda.BDH(cfg, DEV, seed=9)
+    tokens = torch.randint(0, 64, (4, 6), generator=torch.Generator().manual_seed(1))
+    sa, sb = model.init_state(), model.init_state()
+    la = model.forward_with_state(tokens, sa)
+    rows = [model.forward_with_state(tokens[:, t : t + 1], sb) for t in range(6)]
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat(rows, 1), la)
+    assert torch.equal(sa.storage, sb.storage) and sa.position == sb.position == 6
+
+
+def test_bad_token_poisons_only_its_row(bda):
+    cfg = bda.BDHConfig(n_layer=1, n_embd=16, n_head=2, mlp_internal_dim_multiplier=4, vocab_size=32)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    model = bda.BDH(cfg, DEV, seed=2)
+    logits = model.forward_with_state(torch.tensor([[3], [99]]), model.init_state())
+    torch.cuda.synchronize()
+    assert torch.isfinite(logits[0]).all() and torch.isnan(logits[1]).all()
+
+
+def test_model_create_rejects_bad_configs(bda):
+    from burn_dragon_amd import ffi
+
+    cfg = bda.BDHConfig(n_layer=1, n_embd=16, n_head=2, mlp_internal_dim_multiplier=1, vocab_size=8)  # N = 8
+    cfg.n_head = 16  # latent_per_head = 1: odd, RoPE must refuse it (src/model/attention.rs:310)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    with pytest.raises(ffi.BdhError) as err:
+        bda.BDH(cfg, DEV, seed=1)
+    assert err.value.status == ffi.E_SHAPE

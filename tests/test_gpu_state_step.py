@@ -1,0 +1,243 @@
+"""GPU parity of the recurrent state step (bdh_state_step / bdh_recurrent_attention) against the
+CPU oracle, through the C ABI.
+
+Tolerances: BASELINE north_star asks 1e-3 relative for an f32 state and 2e-2 for a bf16 state;
+the f32 checks here are much tighter (the only differences are the device sincos, <= 2 ulp, and
+the summation order of the readout).  Index artefacts (active bitmask, touched-row counts) are
+bit-exact.  Untouched state rows must be bit-identical.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bdh_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    if not torch.cuda.is_available():
+        pytest.fail("no HIP device: the GPU tests must run on the MI355X box")
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    return ffi, recurrent_attention
+
+
+def make_inputs(seed, B, h, T, N, d, density, rho_scale=0.01):
+    rng = np.random.default_rng(seed)
+    if density >= 1.0:
+        x = (np.abs(rng.standard_normal((B, h, T, N))) + 0.1).astype(np.float32)
+    elif density <= 0.0:
+        x = np.zeros((B, h, T, N), np.float32)
+    else:
+        from scipy.stats import norm
+
+        mu = norm.ppf(density)
+        x = np.maximum(rng.standard_normal((B, h, T, N)) + mu, 0).astype(np.float32)
+    v = rng.standard_normal((B, T, d)).astype(np.float32)
+    rho = (rho_scale * rng.standard_normal((B, h, N, d))).astype(np.float32)
+    return x, v, rho
+
+
+def rel_err(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def run_gpu(recurrent_attention, x, v, rho, freqs, position, rotary, slopes=None, positions=None, dtype=torch.float32):
+    dev = "cuda:0"
+    xt, vt = torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev)
+    rt = torch.from_numpy(rho).to(dev).to(dtype).contiguous()
+    ft = torch.from_numpy(freqs).to(dev)
+    pt = None if positions is None else torch.from_numpy(np.asarray(positions, np.int32)).to(dev)
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    out, bm, rows = recurrent_attention(xt, vt, rt, ft, position, RotaryEmbedding(rotary), slopes, pt,
+                                        want_bitmask=True, want_rows=True)
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), rt.float().cpu().numpy(), bm.cpu().numpy().view(np.uint64), rows.cpu().numpy()
+
+
+@pytest.mark.parametrize("d", [256, 512])
+@pytest.mark.parametrize("N,density", [(512, 0.05), (640, 0.5), (130, 1.0), (1024, 0.0), (2048, 0.02)])
+def test_fast_path_decode_step_matches_oracle(gpu, corc, N, d, density):
+    _, recurrent_attention = gpu
+    B, h, T = 3, 2, 1
+    x, v, rho = make_inputs(100 + N + d, B, h, T, N, d, density)
+    freqs = corc.build_freqs(N)
+    position = 1234
+    q = corc.rotate(x, freqs, orc.ROPE, position)
+    out_ref, rho_ref = corc.recurrent_attention(q, v, rho)
+    out, rho_new, bm, rows = run_gpu(recurrent_attention, x, v, rho, freqs, position, orc.ROPE)
+    assert rel_err(out, out_ref) < 2e-5
+    assert rel_err(rho_new, rho_ref) < 1e-6
+    # bit-exact index artefacts
+    assert np.array_equal(bm[:, :, 0], orc.active_bitmask(np.pad(x[:, :, 0], ((0, 0), (0, 0), (0, (-N) % 64)))))
+    assert np.array_equal(rows[:, :, 0], orc.pair_closed_rows(x[:, :, 0]))
+    # rows of inactive pairs are bit-identical to the input state
+    inactive = ~np.repeat((x[:, :, 0] != 0).reshape(B, h, N // 2, 2).any(-1), 2, axis=-1)
+    assert np.array_equal(rho_new[inactive], rho[inactive])
+
+
+def test_update_is_bit_exact_when_rotation_is_exact(gpu, corc):
+    """At position 0 cos = 1 and sin = 0 exactly, so q == x on both sides and the rank-1 update
+    rho + (q*v) (product rounded, then added: src/model/bdh.rs:298) must agree bit for bit."""
+    _, recurrent_attention = gpu
+    B, h, N, d = 2, 2, 512, 256
+    x, v, rho = make_inputs(7, B, h, 1, N, d, 0.3)
+    freqs = corc.build_freqs(N)
+    _, rho_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.ROPE, 0), v, rho)
+    _, rho_new, _, _ = run_gpu(recurrent_attention, x, v, rho, freqs, 0, orc.ROPE)
+    assert np.array_equal(rho_new, rho_ref)
+
+
+def test_first_token_reads_zero_state_and_writes_outer_product(gpu, corc):
+    _, recurrent_attention = gpu
+    B, h, N, d = 2, 2, 256, 256
+    x, v, _ = make_inputs(8, B, h, 1, N, d, 0.2)
+    freqs = corc.build_freqs(N)
+    out, rho_new, _, _ = run_gpu(recurrent_attention, x, v, np.zeros((B, h, N, d), np.float32), freqs, 0, orc.ROPE)
+    assert not out.any()
+    assert np.array_equal(rho_new, x[:, :, 0, :, None] * v[:, None, 0, None, :])
+
+
+@pytest.mark.parametrize("rotary", [orc.ROPE, orc.ALIBI, orc.POPE])
+def test_generic_path_small_shapes_all_rotaries(gpu, corc, rotary):
+    """tests/model_paths.rs shapes (N=32, d=16): the generic kernel, T > 1, all three rotaries."""
+    _, recurrent_attention = gpu
+    B, h, T, N, d = 2, 2, 5, 32, 16
+    x, v, rho = make_inputs(20 + rotary, B, h, T, N, d, 0.4)
+    freqs = corc.build_freqs(N, 65536.0, rotary)
+    slopes = np.array([0.5, 0.125], np.float32) if rotary == orc.ALIBI else None
+    decay = None if slopes is None else corc.alibi_decay(slopes)
+    Nq = 2 * N if rotary == orc.POPE else N
+    rho = (0.01 * np.random.default_rng(1).standard_normal((B, h, Nq, d))).astype(np.float32)
+    q = corc.rotate(x, freqs, rotary, 17)
+    out_ref, rho_ref = corc.recurrent_attention(q, v, rho, decay)
+    out, rho_new, bm, rows = run_gpu(recurrent_attention, x, v, rho, freqs, 17, rotary, slopes)
+    assert rel_err(out, out_ref) < 2e-5
+    assert rel_err(rho_new, rho_ref) < 2e-6
+    assert np.array_equal(bm, orc.active_bitmask(np.pad(x, ((0, 0), (0, 0), (0, 0), (0, 32)))))
+    expect_rows = orc.pair_closed_rows(x) if rotary == orc.ROPE else np.full((B, h, T), Nq)
+    assert np.array_equal(rows, expect_rows)
+
+
+def test_prefill_loop_equals_sequential_steps_and_causal_closed_form(gpu, corc):
+    _, recurrent_attention = gpu
+    B, h, T, N, d = 2, 2, 6, 256, 256
+    x, v, _ = make_inputs(31, B, h, T, N, d, 0.1)
+    rho0 = np.zeros((B, h, N, d), np.float32)
+    freqs = corc.build_freqs(N)
+    out, rho_new, _, _ = run_gpu(recurrent_attention, x, v, rho0, freqs, 40, orc.ROPE)
+    q = corc.rotate(x, freqs, orc.ROPE, 40)
+    out_ref, rho_ref = corc.recurrent_attention(q, v, rho0, sparse=True)
+    assert rel_err(out, out_ref) < 2e-5 and rel_err(rho_new, rho_ref) < 1e-6
+    # closed forms in float64: out = tril(-1)(QQ^T)V, final state = Q^T V
+    q64, v64 = q.astype(np.float64), v.astype(np.float64)
+    assert rel_err(out, orc.causal_unnormalised(q64, v64)) < 1e-5
+    assert rel_err(rho_new, np.einsum("bhtn,btd->bhnd", q64, v64)) < 1e-5
+    # chunk consistency on the device: [0,2) then [2,6) == one call
+    dev = "cuda:0"
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    rt = torch.zeros((B, h, N, d), device=dev)
+    xt, vt, ft = torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev), torch.from_numpy(freqs).to(dev)
+    o1 = recurrent_attention(xt[:, :, :2].contiguous(), vt[:, :2].contiguous(), rt, ft, 40, RotaryEmbedding.ROPE)
+    o2 = recurrent_attention(xt[:, :, 2:].contiguous(), vt[:, 2:].contiguous(), rt, ft, 42, RotaryEmbedding.ROPE)
+    torch.cuda.synchronize()
+    assert np.array_equal(torch.cat([o1, o2], 2).cpu().numpy(), out)
+    assert np.array_equal(rt.cpu().numpy(), rho_new)
+
+
+def test_per_sequence_positions(gpu, corc):
+    _, recurrent_attention = gpu
+    B, h, N, d = 3, 2, 256, 256
+    x, v, rho = make_inputs(41, B, h, 1, N, d, 0.2)
+    freqs = corc.build_freqs(N)
+    positions = [5, 900, 4095]
+    out, rho_new, _, _ = run_gpu(recurrent_attention, x, v, rho, freqs, 0, orc.ROPE, positions=positions)
+    for b, p in enumerate(positions):
+        q = corc.rotate(x[b : b + 1], freqs, orc.ROPE, p)
+        o_ref, r_ref = corc.recurrent_attention(q, v[b : b + 1], rho[b : b + 1])
+        assert rel_err(out[b : b + 1], o_ref) < 2e-5 and rel_err(rho_new[b : b + 1], r_ref) < 1e-6
+
+
+def test_bf16_state_within_tolerance(gpu, corc):
+    """bf16 storage, f32 accumulate: 2e-2 relative (north_star)."""
+    _, recurrent_attention = gpu
+    B, h, T, N, d = 2, 2, 4, 256, 256
+    x, v, rho = make_inputs(51, B, h, T, N, d, 0.2, rho_scale=0.05)
+    rho_b = torch.from_numpy(rho).to(torch.bfloat16).float().numpy()  # the state both sides start from
+    freqs = corc.build_freqs(N)
+    out, rho_new, _, _ = run_gpu(recurrent_attention, x, v, rho_b, freqs, 9, orc.ROPE, dtype=torch.bfloat16)
+    out_ref, rho_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.ROPE, 9), v, rho_b)
+    assert rel_err(out, out_ref) < 2e-2 and rel_err(rho_new, rho_ref) < 2e-2
+
+
+def test_deterministic_across_runs(gpu, corc):
+    _, recurrent_attention = gpu
+    B, h, N, d = 4, 4, 2048, 256
+    x, v, rho = make_inputs(61, B, h, 1, N, d, 0.05)
+    freqs = corc.build_freqs(N)
+    a = run_gpu(recurrent_attention, x, v, rho, freqs, 77, orc.ROPE)
+    b = run_gpu(recurrent_attention, x, v, rho, freqs, 77, orc.ROPE)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+def test_argument_errors_do_not_abort(gpu):
+    ffi, _ = gpu
+    ctx = ffi.default_context(0)
+    lib = ctx.lib
+    t = torch.zeros(1024, device="cuda:0")
+    p = t.data_ptr()
+    # odd latent with RoPE (src/model/attention.rs:310 would fail the reshape)
+    assert lib.bdh_state_step(ctx.handle, 1, 1, 3, 4, ffi.ROPE, p, p, p, 0, None, None, p, ffi.F32, p, None, None) == ffi.E_SHAPE
+    assert b"even" in lib.bdh_last_error(ctx.handle)
+    assert lib.bdh_state_step(ctx.handle, 1, 1, 4, 4, 9, p, p, p, 0, None, None, p, ffi.F32, p, None, None) == ffi.E_INVAL
+    assert lib.bdh_state_step(ctx.handle, 1, 1, 4, 4, ffi.ROPE, p, p, p, -1, None, None, p, ffi.F32, p, None, None) == ffi.E_INVAL
+    assert lib.bdh_state_step(ctx.handle, 1, 1, 4, 4, ffi.ROPE, None, p, p, 0, None, None, p, ffi.F32, p, None, None) == ffi.E_INVAL
+    assert lib.bdh_state_step(ctx.handle, 1, 1, 4, 4, ffi.ROPE, p, p, p, 0, None, None, p + 4, ffi.F32, p, None, None) == ffi.E_ALIGN
+    # empty batch is a no-op
+    assert lib.bdh_state_step(ctx.handle, 0, 4, 8, 4, ffi.ROPE, None, None, None, 0, None, None, None, ffi.F32, None, None, None) == ffi.OK
+
+
+def test_full_size_config2_properties(gpu, corc):
+    """BASELINE config 2 at its real shape: rho f32 [32,4,8192,256] (1 GiB), 5 % density.
+    Checked (a) against the oracle on one batch entry, (b) everywhere against an f32 torch
+    statement of the same step, (c) by the invariant that inactive rows keep their bits."""
+    _, recurrent_attention = gpu
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    B, h, N, d = 32, 4, 8192, 256
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(5)
+    rho = 0.01 * torch.randn((B, h, N, d), device=dev, generator=g)
+    x = torch.relu(torch.randn((B, h, 1, N), device=dev, generator=g) - 1.6449)
+    v = torch.randn((B, 1, d), device=dev, generator=g)
+    freqs_np = corc.build_freqs(N)
+    freqs = torch.from_numpy(freqs_np).to(dev)
+    position = 3071
+    rho_before = rho.clone()
+    out, bm, rows = recurrent_attention(x, v, rho, freqs, position, RotaryEmbedding.ROPE, want_bitmask=True, want_rows=True)
+    torch.cuda.synchronize()
+    x_np = x.cpu().numpy()
+    # (a) oracle on batch entry 0 (dense faithful form)
+    q_np = corc.rotate(x_np, freqs_np, orc.ROPE, position)
+    o_ref, r_ref = corc.recurrent_attention(q_np[:1], v[:1].cpu().numpy(), rho_before[:1].cpu().numpy())
+    assert rel_err(out[:1].cpu().numpy(), o_ref) < 2e-5
+    assert rel_err(rho[:1].cpu().numpy(), r_ref) < 1e-6
+    # (b) torch f32 statement on every element, q taken from the oracle's rotate
+    q = torch.from_numpy(q_np).to(dev)[:, :, 0]
+    out_t = torch.einsum("bhnd,bhn->bhd", rho_before, q)
+    assert rel_err(out[:, :, 0].cpu().numpy(), out_t.cpu().numpy()) < 5e-5
+    rho_t = rho_before + q[..., None] * v[:, None, 0, None, :]
+    assert float((rho - rho_t).abs().max()) < 1e-6
+    # (c) index artefacts and untouched rows
+    assert np.array_equal(bm.cpu().numpy().view(np.uint64)[:, :, 0], orc.active_bitmask(x_np[:, :, 0]))
+    assert np.array_equal(rows.cpu().numpy()[:, :, 0], orc.pair_closed_rows(x_np[:, :, 0]))
+    active_rows = torch.from_numpy(np.repeat((x_np[:, :, 0] != 0).reshape(B, h, N // 2, 2).any(-1), 2, axis=-1)).to(dev)
+    assert torch.equal(rho[~active_rows], rho_before[~active_rows])
+    frac = float(active_rows.float().mean())
+    assert 0.09 < frac < 0.105  # 1 - 0.95^2 = 9.75 % of the rows
