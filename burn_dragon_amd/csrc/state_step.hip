@@ -346,14 +346,13 @@ __global__ __launch_bounds__(256) void k_bitmask_rows(StepPtrs a, int rotary, in
 // second stage: out[slice,:] = sum over the S partials in index order; optional
 // LayerNorm of the result (src/model/bdh.rs:359) and touched-row count.
 // ------------------------------------------------------------------------------------
+template <bool LN>
 __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__ partial,
                                                        const int *__restrict__ pair_cnt, int S, int d,
                                                        float *__restrict__ out, long out_slice_stride,
                                                        float *__restrict__ out_ln, int *__restrict__ rows,
                                                        long rows_slice_stride) {
-  __shared__ float s_part[4];
-  __shared__ float s_stat[2];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x;
   const int slice = blockIdx.x;
   const float *p = partial + (long)slice * S * d;
   float vals[4];  // d <= 1024
@@ -363,6 +362,7 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
     const int c = j * 256 + tid;
     float s = 0.0f;
     if (c < d) {
+#pragma unroll 16
       for (int g = 0; g < S; ++g) s += p[(long)g * d + c];
       out[(long)slice * out_slice_stride + c] = s;
       lsum += s;
@@ -371,11 +371,15 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
   }
   if (rows && pair_cnt && tid == 0) {
     int np = 0;
+#pragma unroll 16
     for (int g = 0; g < S; ++g) np += pair_cnt[(long)slice * S + g];
     rows[(long)slice * rows_slice_stride] = 2 * np;
   }
-  if (!out_ln) return;
+  if (!LN) return;
   // LayerNorm over d: mean, biased variance, (x-mean)/sqrt(var+eps)
+  __shared__ float s_part[4];
+  __shared__ float s_stat[2];
+  const int lane = tid & 63, wave = tid >> 6;
   for (int o = 32; o > 0; o >>= 1) lsum += __shfl_xor(lsum, o);
   if (lane == 0) s_part[wave] = lsum;
   __syncthreads();
@@ -403,6 +407,16 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
     const int c = j * 256 + tid;
     if (c < d) out_ln[(long)slice * out_slice_stride + c] = (vals[j] - mean) / den;
   }
+}
+
+void launch_finalize(hipStream_t st, int slices, const float *partial, const int *pair_cnt, int S, int d, float *out,
+                     long out_stride, float *out_ln, int *rows, long rows_stride) {
+  if (out_ln)
+    hipLaunchKernelGGL(k_step_finalize<true>, dim3(slices), dim3(256), 0, st, partial, pair_cnt, S, d, out, out_stride,
+                       out_ln, rows, rows_stride);
+  else
+    hipLaunchKernelGGL(k_step_finalize<false>, dim3(slices), dim3(256), 0, st, partial, pair_cnt, S, d, out,
+                       out_stride, out_ln, rows, rows_stride);
 }
 
 template <int D, int WAVES, int U>
@@ -466,12 +480,11 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
     if (fast) {
       float *rho = static_cast<float *>(p.rho);
       if (d == 256)
-        launch_fast<256, WAVES, 4>(ctx->stream, slices * S, a, rho);
+        launch_fast<256, WAVES, 2>(ctx->stream, slices * S, a, rho);
       else
         launch_fast<512, WAVES, 2>(ctx->stream, slices * S, a, rho);
       BDH_LAUNCH_CHECK(ctx, "k_step_rope_f32");
-      hipLaunchKernelGGL(k_step_finalize, dim3(slices), dim3(256), 0, ctx->stream, partial, pair_cnt, S, d,
-                         out_t, (long)T * d, out_ln_t, rows_t, (long)T);
+      launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
     } else {
       if (p.rho_dtype == BDH_F32)
@@ -481,8 +494,7 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
         hipLaunchKernelGGL(k_step_generic<unsigned short>, dim3(slices * S), dim3(256), 0, ctx->stream, a,
                            static_cast<unsigned short *>(p.rho), d, Nq, p.rotary, has_decay, decay);
       BDH_LAUNCH_CHECK(ctx, "k_step_generic");
-      hipLaunchKernelGGL(k_step_finalize, dim3(slices), dim3(256), 0, ctx->stream, partial,
-                         (const int *)nullptr, S, d, out_t, (long)T * d, out_ln_t, (int *)nullptr, (long)T);
+      launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
       if (a.bitmask || rows_t) {
         hipLaunchKernelGGL(k_bitmask_rows, dim3(slices), dim3(256), 0, ctx->stream, a, p.rotary, Nq, rows_t,
