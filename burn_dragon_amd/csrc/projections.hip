@@ -333,10 +333,12 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
   if (p.active_blocks_host) {
     int rc = bdh_ws_reserve(ctx, (size_t)p.n_blocks + 256);
     if (rc != BDH_OK) return rc;
-    // pageable source: the runtime stages the copy, so the host buffer may be reused on return
-    if (p.n_blocks > 0)
+    // the caller's host buffer may go away on return: finish the copy before returning
+    if (p.n_blocks > 0) {
       BDH_HIP_CHECK(ctx, hipMemcpyAsync(ctx->ws, p.active_blocks_host, (size_t)p.n_blocks,
                                         hipMemcpyHostToDevice, ctx->stream));
+      BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    }
     mask_dev = static_cast<const unsigned char *>(ctx->ws);
   }
   const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));

@@ -233,6 +233,151 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
 }
 
 // ------------------------------------------------------------------------------------
+// fast path: RoPE, bf16 state (f32 accumulate), D in {256, 512}.  A lane pair's two rows are
+// 4*D contiguous bytes; each lane owns D/256 16-byte pieces (8 bf16) of that chunk.
+// ------------------------------------------------------------------------------------
+template <int D, int WAVES, int U>
+__global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsigned short *__restrict__ rho) {
+  constexpr int PL = D / 256;      // 16-byte pieces per lane per pair (D=256: 1, D=512: 2)
+  constexpr int PPB = WAVES * 64;
+  __shared__ int s_cnt[WAVES];
+  __shared__ unsigned short s_idx[PPB];
+  __shared__ float2 s_q[PPB];
+  __shared__ float s_red[WAVES][2][D];  // per wave, per row of the pair
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slice = blockIdx.x / a.S;
+  const int seg = blockIdx.x - slice * a.S;
+  const int b = slice / a.h;
+  const int NP = a.N >> 1;
+  const int p = seg * PPB + tid;
+
+  float2 xv = make_float2(0.0f, 0.0f), fv = make_float2(0.0f, 0.0f);
+  if (p < NP) {
+    xv = reinterpret_cast<const float2 *>(a.x + (long)slice * a.x_slice_stride)[p];
+    fv = reinterpret_cast<const float2 *>(a.freqs)[p];
+  }
+  const float pos = a.pos_dev ? (float)((long)a.pos_dev[b] + a.pos_add) : a.pos_scalar;
+  const bool ae = xv.x != 0.0f, ao = xv.y != 0.0f;
+  const bool act = ae || ao;
+  const unsigned long long m_act = __ballot(act);
+  if (a.bitmask) {
+    const unsigned long long me = __ballot(ae), mo = __ballot(ao);
+    if (lane == 0) {
+      const int w0 = (seg * PPB + wave * 64) >> 5;
+      const int NW = (a.N + 63) >> 6;
+      unsigned long long *bm = a.bitmask + (long)slice * a.bitmask_slice_stride;
+      if (w0 < NW) bm[w0] = spread_bits((unsigned int)me) | (spread_bits((unsigned int)mo) << 1);
+      if (w0 + 1 < NW)
+        bm[w0 + 1] = spread_bits((unsigned int)(me >> 32)) | (spread_bits((unsigned int)(mo >> 32)) << 1);
+    }
+  }
+  float2 q = make_float2(0.0f, 0.0f);
+  if (act) {
+    float s0, c0, s1, c1;
+    sincosf(rope_phase(pos, fv.x), &s0, &c0);
+    if (fv.y == fv.x) {
+      s1 = s0;
+      c1 = c0;
+    } else {
+      sincosf(rope_phase(pos, fv.y), &s1, &c1);
+    }
+    const float a0 = xv.x * c0, r0 = (-xv.y) * s0;
+    const float a1 = xv.y * c1, r1 = xv.x * s1;
+    q.x = a0 + r0;
+    q.y = a1 + r1;
+  }
+  if (lane == 0) s_cnt[wave] = __popcll(m_act);
+  __syncthreads();
+  int offset = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const int c = s_cnt[w];
+    if (w < wave) offset += c;
+    total += c;
+  }
+  if (act) {
+    const int rank = offset + __popcll(m_act & ((1ull << lane) - 1ull));
+    s_idx[rank] = (unsigned short)tid;
+    s_q[rank] = q;
+  }
+  __syncthreads();
+
+  // piece j of this lane covers elements e0 = (j*64 + lane)*8 .. +7 of the 2*D-element pair chunk
+  int prow[PL], pcol[PL];
+  float vv[PL][8], acc[PL][8];
+  const float *vrow = a.v + (long)b * a.v_batch_stride;
+#pragma unroll
+  for (int j = 0; j < PL; ++j) {
+    const int e0 = (j * 64 + lane) * 8;
+    prow[j] = e0 / D;
+    pcol[j] = e0 - prow[j] * D;
+    const float4 v0 = *reinterpret_cast<const float4 *>(vrow + pcol[j]);
+    const float4 v1 = *reinterpret_cast<const float4 *>(vrow + pcol[j] + 4);
+    vv[j][0] = v0.x; vv[j][1] = v0.y; vv[j][2] = v0.z; vv[j][3] = v0.w;
+    vv[j][4] = v1.x; vv[j][5] = v1.y; vv[j][6] = v1.z; vv[j][7] = v1.w;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[j][e] = 0.0f;
+  }
+  unsigned short *base = rho + ((long)slice * a.N + 2L * seg * PPB) * D;
+
+  for (int i0 = wave; i0 < total; i0 += WAVES * U) {
+    uint4 r[U][PL];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * WAVES;
+      if (i < total) {
+        const uint4 *rp = reinterpret_cast<const uint4 *>(base + (long)s_idx[i] * (2 * D));
+#pragma unroll
+        for (int j = 0; j < PL; ++j) r[u][j] = rp[j * 64 + lane];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * WAVES;
+      if (i < total) {
+        const float2 qq = s_q[i];
+        uint4 *wp = reinterpret_cast<uint4 *>(base + (long)s_idx[i] * (2 * D));
+#pragma unroll
+        for (int j = 0; j < PL; ++j) {
+          const float qf = prow[j] ? qq.y : qq.x;
+          const unsigned int w[4] = {r[u][j].x, r[u][j].y, r[u][j].z, r[u][j].w};
+          unsigned int o[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            float lo = __uint_as_float(w[k] << 16), hi = __uint_as_float(w[k] & 0xffff0000u);
+            acc[j][2 * k] = __builtin_fmaf(lo, qf, acc[j][2 * k]);
+            acc[j][2 * k + 1] = __builtin_fmaf(hi, qf, acc[j][2 * k + 1]);
+            const float t0 = qf * vv[j][2 * k], t1 = qf * vv[j][2 * k + 1];
+            lo = lo + t0;
+            hi = hi + t1;
+            o[k] = (unsigned int)f32_to_bf16(lo) | ((unsigned int)f32_to_bf16(hi) << 16);
+          }
+          wp[j * 64 + lane] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < PL; ++j) {
+    // D=256: both rows are covered by one piece (lanes 0-31 row 0, 32-63 row 1);
+    // D=512: piece 0 is row 0, piece 1 is row 1.
+    float *dst = &s_red[wave][prow[j]][pcol[j]];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dst[e] = acc[j][e];
+  }
+  __syncthreads();
+  float *pout = a.partial + (long)blockIdx.x * D;
+  for (int c = tid; c < D; c += PPB) {
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) s += s_red[w][0][c] + s_red[w][1][c];
+    pout[c] = s;
+  }
+  if (tid == 0) a.pair_cnt[blockIdx.x] = total;
+}
+
+// ------------------------------------------------------------------------------------
 // generic path: any d <= 1024, any rotary, f32 or bf16 state.  One workgroup owns ROWS
 // state rows of one slice; waves take rows round-robin, lanes stride over columns.
 // ------------------------------------------------------------------------------------
@@ -434,7 +579,7 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   if (N > 65536 * 2 && p.rotary == BDH_ROPE) { /* pair index within a workgroup is 16 bit: always fits */ }
   if ((long)slices > 0x7fffffffL / 4096) return bdh_fail(ctx, BDH_E_SHAPE, "B*h too large");
 
-  const bool fast = p.rotary == BDH_ROPE && p.rho_dtype == BDH_F32 && (d == 256 || d == 512) && N >= 2;
+  const bool fast = p.rotary == BDH_ROPE && (d == 256 || d == 512) && N >= 2;
   constexpr int WAVES = 4;
   const int S = fast ? ((N / 2) + WAVES * 64 - 1) / (WAVES * 64) : (Nq + kGenRows - 1) / kGenRows;
   if (N == 0 || d == 0) {
@@ -478,12 +623,20 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
     float *out_ln_t = out_ln ? out_ln + (long)t * d : nullptr;
     int32_t *rows_t = p.rows_touched ? p.rows_touched + t : nullptr;
     if (fast) {
-      float *rho = static_cast<float *>(p.rho);
-      if (d == 256)
-        launch_fast<256, WAVES, 2>(ctx->stream, slices * S, a, rho);
-      else
-        launch_fast<512, WAVES, 2>(ctx->stream, slices * S, a, rho);
-      BDH_LAUNCH_CHECK(ctx, "k_step_rope_f32");
+      if (p.rho_dtype == BDH_F32) {
+        float *rho = static_cast<float *>(p.rho);
+        if (d == 256)
+          launch_fast<256, WAVES, 2>(ctx->stream, slices * S, a, rho);
+        else
+          launch_fast<512, WAVES, 2>(ctx->stream, slices * S, a, rho);
+      } else {
+        unsigned short *rho = static_cast<unsigned short *>(p.rho);
+        if (d == 256)
+          hipLaunchKernelGGL((k_step_rope_bf16<256, WAVES, 4>), dim3(slices * S), dim3(WAVES * 64), 0, ctx->stream, a, rho);
+        else
+          hipLaunchKernelGGL((k_step_rope_bf16<512, WAVES, 2>), dim3(slices * S), dim3(WAVES * 64), 0, ctx->stream, a, rho);
+      }
+      BDH_LAUNCH_CHECK(ctx, "k_step_rope");
       launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
     } else {

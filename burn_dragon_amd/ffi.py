@@ -85,7 +85,7 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_layer_norm.argtypes = [P, c_int64, c_int, P, P]
     lib.bdh_fused_state_aligned.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, P, c_int, P, c_int, c_int,
                                             c_int, P]
-    lib.bdh_prefill_chunked.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, P, P]
+    lib.bdh_prefill_chunked.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, c_int, P, P]
     lib.bdh_model_create.argtypes = [P, POINTER(ModelConfigC), POINTER(ModelWeightsC), POINTER(P)]
     lib.bdh_model_destroy.argtypes = [P]
     lib.bdh_model_state_bytes.restype = c_size_t

@@ -52,3 +52,23 @@ def layer_norm(x: torch.Tensor, ctx: Optional[ffi.Context] = None) -> torch.Tens
     d = x.shape[-1]
     ctx.check(ctx.lib.bdh_layer_norm(ctx.handle, x.numel() // max(d, 1), d, ffi.ptr(x), ffi.ptr(out)))
     return out
+
+
+def prefill_chunked(x_bf16: torch.Tensor, v_bf16: torch.Tensor, rho: torch.Tensor, freqs: torch.Tensor,
+                    position: int, state_is_zero: bool = False, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
+    """The recurrent path (src/model/bdh.rs:258-307, RoPE) for T tokens at once on the bf16 matrix
+    cores.  x_bf16 [B,h,T,N] bfloat16 un-rotated, v_bf16 [B,T,d] bfloat16, rho [B,h,N,d] float32
+    (updated in place).  Returns out [B,h,T,d] float32."""
+    ctx = ctx or ffi.default_context(x_bf16.device.index or 0)
+    B, h, T, N = x_bf16.shape
+    d = v_bf16.shape[-1]
+    assert x_bf16.dtype == torch.bfloat16 and x_bf16.is_contiguous()
+    v_bf16 = v_bf16.reshape(B, T, d)
+    assert v_bf16.dtype == torch.bfloat16 and v_bf16.is_contiguous()
+    assert rho.dtype == torch.float32 and rho.is_contiguous() and tuple(rho.shape) == (B, h, N, d)
+    out = torch.empty((B, h, T, d), device=x_bf16.device, dtype=torch.float32)
+    freqs = freqs.reshape(-1)
+    ctx.check(ctx.lib.bdh_prefill_chunked(ctx.handle, B, h, T, N, d, ffi.ptr(x_bf16), ffi.ptr(v_bf16),
+                                          ffi.ptr(freqs), int(position), int(bool(state_is_zero)), ffi.ptr(rho),
+                                          ffi.ptr(out)))
+    return out

@@ -155,18 +155,22 @@ int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N, int dv,
 
 /* ---- chunked prefill (dense MFMA form of the recurrent path) ------------------------ */
 /*
- * The recurrent path of src/model/bdh.rs:258-307 for T tokens at once, RoPE only, computed
- * chunk-wise on the bf16 matrix cores with f32 accumulation:
- *   out_c = tril(-1)(Q_c Q_c^T) V_c + Q_c rho ;  rho += Q_c^T V_c      per chunk c
+ * The recurrent path of src/model/bdh.rs:258-307 for T tokens at once, RoPE only, computed on
+ * the bf16 matrix cores with f32 accumulation:
+ *   out = tril(-1)(Q Q^T) V + Q rho0 ;  rho = rho0 + Q^T V ,  Q = bf16(rope(x))
  * The reference has no such function (its prefill walks tokens serially, src/generation.rs:
- * 74-104); the sequential loop is the definition of the result.
- *   x   [B,h,T,N] bf16 (raw 16-bit) un-rotated activations
- *   v   [B,T,d]   bf16
+ * 74-104, src/model/bdh.rs:288); the sequential loop is the definition of the result.
+ *   x   [B,h,T,N] bf16 (raw 16-bit patterns) un-rotated activations
+ *   v   [B,T,d]   bf16, shared by the heads of a batch entry
+ *   position      start position of token 0
+ *   state_is_zero non-zero: the caller promises rho holds zeros (a fresh state, src/model/
+ *                 state.rs:27-45); the Q rho0 product is skipped and rho is overwritten
  *   rho [B,h,N,d] f32 in/out,  out [B,h,T,d] f32
+ * N and d must be multiples of 8.
  */
 int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
                         const uint16_t *v_bf16, const float *freqs, int64_t position,
-                        float *rho, float *out);
+                        int state_is_zero, float *rho, float *out);
 
 /* ---- a1: the whole cached step ------------------------------------------------------- */
 /* src/model/config.rs:113-164 (BDHConfig) + :10-31 (FusedKernelConfig), as plain scalars */

@@ -1,0 +1,173 @@
+"""GPU parity of the all-tokens-at-once forms: the f32 block-tiled normalised attention
+(bdh_fused_state_aligned, the reference's training-path kernel) and the bf16 matrix-core
+chunked prefill (bdh_prefill_chunked), through the C ABI, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bdh_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def bda():
+    if not torch.cuda.is_available():
+        pytest.fail("no HIP device: the GPU tests must run on the MI355X box")
+    import burn_dragon_amd
+
+    return burn_dragon_amd
+
+
+def assert_close(lhs, rhs, atol, rtol):
+    """tests/fused_kernel_tests.rs:13-33."""
+    lhs, rhs = np.asarray(lhs, np.float64), np.asarray(rhs, np.float64)
+    assert lhs.shape == rhs.shape
+    assert not (np.abs(lhs - rhs) > atol + rtol * np.abs(rhs)).any(), f"max diff {np.abs(lhs - rhs).max()}"
+
+
+def rel_err(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+# ------------------------------------------------------------ fused_state_aligned
+@pytest.mark.parametrize("rotary,seed", [("rope", 1337), ("pope", 2024)])
+def test_fused_attention_matches_reference(bda, corc, rotary, seed):
+    """tests/fused_kernel_tests.rs:70-170 on the device path: B=1, h=2, T=6, N=8, dv=6,
+    BlockPattern2d::dense(3); fused == dense tril(-1) + row-normalise, tolerance 1e-4."""
+    from burn_dragon_amd.kernel import linear_attention
+
+    rot = bda.RotaryEmbedding.parse(rotary)
+    g = torch.Generator().manual_seed(seed)
+    query = torch.randn((1, 2, 6, 8), generator=g)
+    value = torch.randn((1, 1, 6, 6), generator=g)
+    freqs = linear_attention.build_freqs(8, 65536.0, rot)
+    fused = linear_attention.fused_state_aligned(query.to(DEV), value.to(DEV), freqs.to(DEV), None,
+                                                 bda.BlockPattern2d.dense(3), rot)
+    torch.cuda.synchronize()
+    # dense reference in float64, as the reference test writes it
+    q = orc.rotate(query.double().numpy(), freqs.double().numpy().reshape(-1), int(rot), 0)
+    scores = np.tril(q @ np.swapaxes(q, 2, 3), -1)
+    scores = scores / (np.abs(scores).sum(3, keepdims=True) + 1e-6)
+    reference = scores @ value.double().numpy()
+    assert_close(fused.cpu().numpy(), reference, 1e-4, 1e-4)
+    # and the oracle's blocked form
+    ref_c = corc.fused_state_aligned(query.numpy(), value.numpy()[:, 0], freqs.numpy().reshape(-1), None, 3, int(rot))
+    assert_close(fused.cpu().numpy(), ref_c, 1e-4, 1e-4)
+
+
+def test_fused_attention_alibi_sparse_pattern_and_unnormalised(bda, corc):
+    from burn_dragon_amd.kernel import linear_attention
+
+    rng = np.random.default_rng(3)
+    B, h, T, N, dv = 2, 2, 11, 16, 5
+    query = np.abs(rng.standard_normal((B, h, T, N))).astype(np.float32)
+    value = rng.standard_normal((B, T, dv)).astype(np.float32)
+    slopes = np.array([0.5, 0.25], np.float32)
+    zeros = np.zeros(N, np.float32)
+    qt, vt = torch.from_numpy(query).to(DEV), torch.from_numpy(value[:, None]).to(DEV)
+    # ALiBi, dense pattern, ragged last block (the term is added to whole blocks: linear_attention.rs:97-100)
+    got = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(zeros), torch.from_numpy(slopes),
+                                               bda.BlockPattern2d.dense(4), bda.RotaryEmbedding.ALIBI)
+    assert_close(got.cpu().numpy(), corc.fused_state_aligned(query, value, zeros, slopes, 4, orc.ALIBI), 1e-4, 1e-4)
+    # sparse (row, col) block pairs; row block 1 has no active column -> zeros (linear_attention.rs:70-73)
+    pairs = {(0, 0), (2, 0), (2, 2)}
+    freqs = corc.build_freqs(N)
+    got = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs), None,
+                                               bda.BlockPattern2d.from_pairs(4, pairs), bda.RotaryEmbedding.ROPE)
+    ref = corc.fused_state_aligned(query, value, freqs, None, 4, orc.ROPE, pairs=pairs)
+    assert_close(got.cpu().numpy(), ref, 1e-4, 1e-4)
+    assert not got[:, :, 4:8].any()
+    # row_normalize = 0 equals the recurrent path started from a zero state at position 0
+    got = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs), None, bda.BlockPattern2d.dense(4),
+                                               bda.RotaryEmbedding.ROPE, row_normalize=False)
+    out_rec, _ = corc.recurrent_attention(corc.rotate(query, freqs, orc.ROPE, 0), value, np.zeros((B, h, N, dv), np.float32))
+    assert_close(got.cpu().numpy(), out_rec, 1e-4, 1e-4)
+
+
+# ---------------------------------------------------------------- chunked prefill
+def _prefill_case(seed, B, h, T, N, d, density, rho0_scale):
+    from scipy.stats import norm
+
+    g = torch.Generator().manual_seed(seed)
+    x = torch.relu(torch.randn((B, h, T, N), generator=g) + float(norm.ppf(density))).to(torch.bfloat16)
+    v = torch.randn((B, T, d), generator=g).to(torch.bfloat16)
+    rho0 = (rho0_scale * torch.randn((B, h, N, d), generator=g)).float()
+    return x, v, rho0
+
+
+@pytest.mark.parametrize("T,N,d,rho0_scale,position", [(64, 256, 256, 0.0, 0), (200, 512, 256, 0.05, 77),
+                                                       (300, 264, 72, 0.05, 5), (520, 128, 512, 0.0, 1000)])
+def test_prefill_chunked_equals_sequential_recurrence(bda, corc, T, N, d, rho0_scale, position):
+    """Oracle = the sequential f32 loop of src/model/bdh.rs:288-302 on the bf16-rounded inputs.
+    Tolerance 2e-2 relative on the max-norm (north_star, bf16 path); Q is rounded to bf16 once
+    and the scores are kept in bf16."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h = 2, 2
+    x, v, rho0 = _prefill_case(T + N, B, h, T, N, d, 0.2, rho0_scale)
+    freqs = corc.build_freqs(N)
+    q = corc.rotate(x.float().numpy(), freqs, orc.ROPE, position)
+    out_ref, rho_ref = corc.recurrent_attention(q, v.float().numpy(), rho0.numpy(), sparse=True)
+    rho = rho0.clone().to(DEV)
+    out = prefill_chunked(x.to(DEV), v.to(DEV), rho, torch.from_numpy(freqs).to(DEV), position,
+                          state_is_zero=(rho0_scale == 0.0))
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), out_ref) < 2e-2
+    assert rel_err(rho.cpu().numpy(), rho_ref) < 2e-2
+    assert not out[:, :, 0].any() or rho0_scale != 0.0  # token 0 reads only the initial state
+
+
+def test_prefill_chunked_then_decode_steps_continue_the_state(bda, corc):
+    """Prefill T tokens on the matrix cores, then decode 3 tokens with bdh_state_step: the
+    readouts must match the all-sequential oracle (2e-2: the prefilled state carries bf16 error)."""
+    from burn_dragon_amd.recurrent import prefill_chunked, recurrent_attention
+
+    B, h, T, N, d = 1, 2, 96, 256, 256
+    x, v, _ = _prefill_case(9, B, h, T + 3, N, d, 0.1, 0.0)
+    freqs = corc.build_freqs(N)
+    q = corc.rotate(x.float().numpy(), freqs, orc.ROPE, 0)
+    out_ref, rho_ref = corc.recurrent_attention(q, v.float().numpy(), np.zeros((B, h, N, d), np.float32), sparse=True)
+    rho = torch.zeros((B, h, N, d), device=DEV)
+    ft = torch.from_numpy(freqs).to(DEV)
+    out_p = prefill_chunked(x[:, :, :T].contiguous().to(DEV), v[:, :T].contiguous().to(DEV), rho, ft, 0, state_is_zero=True)
+    out_d = recurrent_attention(x[:, :, T:].float().contiguous().to(DEV), v[:, T:].float().contiguous().to(DEV), rho, ft,
+                                T, bda.RotaryEmbedding.ROPE)
+    torch.cuda.synchronize()
+    assert rel_err(out_p.cpu().numpy(), out_ref[:, :, :T]) < 2e-2
+    assert rel_err(out_d.cpu().numpy(), out_ref[:, :, T:]) < 2e-2
+    assert rel_err(rho.cpu().numpy(), rho_ref) < 2e-2
+
+
+def test_prefill_chunked_config3_shape_properties(bda, corc):
+    """BASELINE config 3 per-slice shape (T=2048, N=8192, d=256, 5 % density) on a reduced batch
+    (B=1, h=2) so the oracle finishes in seconds.  Checks against the sequential oracle and the
+    size-independent closed forms (first row zero, final state == Q^T V)."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h, T, N, d = 1, 2, 2048, 8192, 256
+    x, v, _ = _prefill_case(11, B, h, T, N, d, 0.05, 0.0)
+    freqs = corc.build_freqs(N)
+    rho = torch.zeros((B, h, N, d), device=DEV)
+    out = prefill_chunked(x.to(DEV), v.to(DEV), rho, torch.from_numpy(freqs).to(DEV), 0, state_is_zero=True)
+    torch.cuda.synchronize()
+    q = corc.rotate(x.float().numpy(), freqs, orc.ROPE, 0)
+    out_ref, rho_ref = corc.recurrent_attention(q, v.float().numpy(), np.zeros((B, h, N, d), np.float32), sparse=True)
+    assert rel_err(out.cpu().numpy(), out_ref) < 2e-2
+    assert rel_err(rho.cpu().numpy(), rho_ref) < 2e-2
+    assert not out[:, :, 0].any()
+    qtv = torch.einsum("bhtn,btd->bhnd", torch.from_numpy(q).to(DEV), v.float().to(DEV))
+    assert rel_err(rho.cpu().numpy(), qtv.cpu().numpy()) < 2e-2
+
+
+def test_prefill_chunked_argument_errors(bda):
+    from burn_dragon_amd import ffi
+
+    ctx = ffi.default_context(0)
+    t = torch.zeros(4096, device=DEV)
+    p = t.data_ptr()
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 12, 8, p, p, p, 0, 1, p, p) == ffi.E_SHAPE  # N % 8
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 16, 8, None, p, p, 0, 1, p, p) == ffi.E_INVAL
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 0, 1, 8, 16, 8, None, None, None, 0, 1, None, None) == ffi.OK

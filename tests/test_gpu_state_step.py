@@ -164,16 +164,25 @@ def test_per_sequence_positions(gpu, corc):
         assert rel_err(out[b : b + 1], o_ref) < 2e-5 and rel_err(rho_new[b : b + 1], r_ref) < 1e-6
 
 
-def test_bf16_state_within_tolerance(gpu, corc):
-    """bf16 storage, f32 accumulate: 2e-2 relative (north_star)."""
+@pytest.mark.parametrize("N,d", [(256, 256), (384, 512), (32, 16)])
+def test_bf16_state_within_tolerance(gpu, corc, N, d):
+    """bf16 storage, f32 accumulate: 2e-2 relative (north_star).  d=256/512 take the wave-per-pair
+    kernel, d=16 the generic one."""
     _, recurrent_attention = gpu
-    B, h, T, N, d = 2, 2, 4, 256, 256
-    x, v, rho = make_inputs(51, B, h, T, N, d, 0.2, rho_scale=0.05)
+    B, h, T = 2, 2, 4
+    x, v, rho = make_inputs(51 + d, B, h, T, N, d, 0.2, rho_scale=0.05)
     rho_b = torch.from_numpy(rho).to(torch.bfloat16).float().numpy()  # the state both sides start from
     freqs = corc.build_freqs(N)
-    out, rho_new, _, _ = run_gpu(recurrent_attention, x, v, rho_b, freqs, 9, orc.ROPE, dtype=torch.bfloat16)
+    out, rho_new, bm, rows = run_gpu(recurrent_attention, x, v, rho_b, freqs, 9, orc.ROPE, dtype=torch.bfloat16)
     out_ref, rho_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.ROPE, 9), v, rho_b)
     assert rel_err(out, out_ref) < 2e-2 and rel_err(rho_new, rho_ref) < 2e-2
+    assert np.array_equal(rows, orc.pair_closed_rows(x))
+    assert np.array_equal(bm, orc.active_bitmask(np.pad(x, ((0, 0), (0, 0), (0, 0), (0, (-N) % 64)))))
+    # one step from an exactly representable state: the only error is the final rounding to bf16
+    x1, v1 = x[:, :, :1], v[:, :1]
+    _, rho_1, _, _ = run_gpu(recurrent_attention, x1, v1, rho_b, freqs, 0, orc.ROPE, dtype=torch.bfloat16)
+    _, rho_1_ref = corc.recurrent_attention(corc.rotate(x1, freqs, orc.ROPE, 0), v1, rho_b)
+    assert np.array_equal(rho_1, torch.from_numpy(rho_1_ref).to(torch.bfloat16).float().numpy())
 
 
 def test_deterministic_across_runs(gpu, corc):
