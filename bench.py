@@ -54,6 +54,63 @@ def cpu_baseline(B, h, N, d, freqs, budget_s=12.0, max_steps=20):
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def bench_prefill(args):
+    """BASELINE config 3: chunked prefill, B=8, T=2048, h=4, N=8192, d=256, bf16 inputs, f32
+    accumulate, 5 % density, positions 0..T, fresh state.  One step = one bdh_prefill_chunked."""
+    import torch
+    from scipy.stats import norm
+
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.kernel.linear_attention import build_freqs
+    from burn_dragon_amd.positional import RotaryEmbedding
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    dev = torch.device("cuda:0")
+    B = 8 if args.batch == 32 else args.batch
+    h, N, d, T = args.heads, args.latent, args.embd, args.time
+    steps = min(args.steps, 20) if args.steps == 1000 else args.steps
+    warmup = min(args.warmup, 3) if args.warmup == 50 else args.warmup
+    g = torch.Generator(device=dev).manual_seed(4)
+    mu = float(norm.ppf(args.density))
+    x = torch.empty((B, h, T, N), device=dev, dtype=torch.bfloat16)
+    for b in range(B):  # generated per batch entry to bound the f32 temporary
+        x[b] = torch.relu(torch.randn((h, T, N), device=dev, generator=g) + mu).to(torch.bfloat16)
+    v = torch.randn((B, T, d), device=dev, generator=g).to(torch.bfloat16)
+    freqs = build_freqs(N, 65536.0, RotaryEmbedding.ROPE).reshape(-1).to(dev)
+    rho = torch.zeros((B, h, N, d), device=dev)
+    for _ in range(warmup):
+        prefill_chunked(x, v, rho, freqs, 0, state_is_zero=True)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        prefill_chunked(x, v, rho, freqs, 0, state_is_zero=True)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = start.elapsed_time(stop)
+    ms = max(gpu_ms, wall * 1e3) / steps
+    flop = float(B * h) * (T * (T - 1.0) * N + T * (T - 1.0) * d + 2.0 * T * N * d)
+    achieved = flop / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "prefill tokens/sec (chunked dense linear attention) + bf16 MFMA utilisation",
+        "value": B * T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"BASELINE config 3: chunked prefill B={B} T={T} h={h} N={N} d={d}, bf16 in / f32 "
+                               f"accumulate, {args.density:.0%} active, RoPE positions 0..T, fresh state",
+                   "algorithmic_flop_per_step": flop},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "whole bdh_prefill_chunked call (k_rope_bf16 + 3 k_gemm launches); algorithmic FLOP "
+                               "= B*h*[T(T-1)N + T(T-1)d + 2TNd]"},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,6 +124,9 @@ def main():
     ap.add_argument("--rho-dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--ring", type=int, default=16, help="number of distinct (x, v) input sets")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
+                    help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA)")
+    ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); use --gpus 1",
@@ -84,6 +144,8 @@ def main():
     from burn_dragon_amd.positional import RotaryEmbedding
 
     dev = torch.device("cuda:0")
+    if args.workload == "prefill":
+        return bench_prefill(args)
     B, h, N, d = args.batch, args.heads, args.latent, args.embd
     ctx = ffi.default_context(0)
     lib = ctx.lib

@@ -12,9 +12,12 @@
 //                       (+ Q rho0 first when the state is not known to be zero)
 //   4. k_gemm<ACC>      rho += Q^T V
 // One GEMM kernel serves all products: C[m,n] = sum_k A[m,k] B[n,k] with 256x256x64 workgroup
-// tiles, 8 wavefronts (2x4) of 128x64 each, v_mfma_f32_32x32x16_bf16, f32 accumulators.  An
-// operand that is k-contiguous in memory is copied to LDS as is; an operand whose rows are the
-// k index (V, rho0, and Q for Q^T V) is transposed while it is written to LDS.
+// tiles, 8 wavefronts (2x4) of 128x64 each, v_mfma_f32_32x32x16_bf16, f32 accumulators.  B is
+// always k-contiguous in memory (V and rho0 are transposed once by a small kernel).  A is either
+// k-contiguous (copied to LDS as is, fragments read with one 16-byte LDS load) or, for Q^T V,
+// k-major (Q [T,N] with the reduction over T): that tile is also copied as is, [k][m], and the
+// fragments are gathered with 2-byte LDS reads; a 64-byte column swizzle on every other group of
+// eight k rows keeps the two half-waves on different banks.
 #include "bdh_internal.h"
 
 namespace {
@@ -78,6 +81,35 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint4 *__restrict__ x, 
 }
 
 // ------------------------------------------------------------------------------------
+// batched transpose to bf16: in [batch][R][C] (f32 or bf16) -> out [batch][C][ldo], ldo >= R,
+// columns R..ldo-1 of the output are zero-filled.  64x64 tiles through LDS.
+// ------------------------------------------------------------------------------------
+template <typename TIn>
+__global__ __launch_bounds__(256) void k_transpose_to_bf16(const TIn *__restrict__ in, unsigned short *__restrict__ out,
+                                                          int R, int C, int ldo) {
+  __shared__ unsigned short tile[64][66];
+  const long batch = blockIdx.z;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const TIn *src = in + batch * (long)R * C;
+  unsigned short *dst = out + batch * (long)C * ldo;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int rr = ty; rr < 64; rr += 4) {
+    const int r = r0 + rr, c = c0 + tx;
+    unsigned short v = 0;
+    if (r < R && c < C) {
+      if constexpr (sizeof(TIn) == 4) v = f32_to_bf16_bits((float)src[(long)r * C + c]);
+      else v = (unsigned short)src[(long)r * C + c];
+    }
+    tile[rr][tx] = v;
+  }
+  __syncthreads();
+  for (int cc = ty; cc < 64; cc += 4) {
+    const int c = c0 + cc, r = r0 + tx;
+    if (c < C && r < ldo) dst[(long)c * ldo + r] = tile[tx][cc];  // rows >= R were staged as zero
+  }
+}
+
+// ------------------------------------------------------------------------------------
 // batched GEMM  C[m,n] (+)= sum_k A[m,k] B[n,k]
 // ------------------------------------------------------------------------------------
 enum { EPI_SCORES = 0, EPI_ACC = 1 };
@@ -97,10 +129,13 @@ struct GemmArgs {
   int n_tiles, n_slices;
 };
 
-template <bool A_KMAJOR, bool B_KMAJOR, bool B_F32, int EPI>
+constexpr int KM_STRIDE = BM + 8;  // bf16 elements per k row of a k-major tile in LDS (528 bytes)
+
+template <bool A_KMAJOR, int EPI>
 __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
   __shared__ __attribute__((aligned(16))) unsigned short s_a[BM * LDS_STRIDE];
   __shared__ __attribute__((aligned(16))) unsigned short s_b[BN * LDS_STRIDE];
+  static_assert(BK * KM_STRIDE <= BM * LDS_STRIDE, "k-major tile must fit");
 
   // XCD-aware mapping: workgroup ids are dealt round-robin to the 8 XCDs, so workgroups with the
   // same (id % 8) share an L2; all tiles of one slice go to one XCD.
@@ -117,8 +152,7 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
       while ((i + 1) * (i + 2) / 2 <= t) ++i;
       tj = t - i * (i + 1) / 2;
       ti = i;
-      // heaviest rows first does not matter for the scores (equal K); keep natural order
-    } else {
+    } else {  // row tiles from the last (largest causal K) down
       ti = g.mt - 1 - t / g.nt;
       tj = t % g.nt;
     }
@@ -129,9 +163,7 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
   const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves, 128 x 64 each
 
   const unsigned short *A = static_cast<const unsigned short *>(g.A) + (long)slice * g.a_batch;
-  const long b_off = (long)(slice / g.b_div) * g.b_batch;
-  const unsigned short *Bh = static_cast<const unsigned short *>(g.B) + b_off;
-  const float *Bf = static_cast<const float *>(g.B) + b_off;
+  const unsigned short *Bh = static_cast<const unsigned short *>(g.B) + (long)(slice / g.b_div) * g.b_batch;
 
   int K = g.K;
   if (g.causal_k) K = min(K, m0 + BM);
@@ -166,43 +198,23 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int chunk = c * 512 + tid;
+      const int row = chunk >> 3, kc = (chunk & 7) * 8;
       uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (!B_KMAJOR) {
-        const int row = chunk >> 3, kc = (chunk & 7) * 8;
-        if (n0 + row < g.N && k0 + kc < K) v = *reinterpret_cast<const uint4 *>(Bh + (long)(n0 + row) * g.ldb + k0 + kc);
-      } else {
-        const int kr = chunk >> 5, nc = (chunk & 31) * 8;
-        if (k0 + kr < K && n0 + nc < g.N) {
-          if (B_F32) {
-            const float4 f0 = *reinterpret_cast<const float4 *>(Bf + (long)(k0 + kr) * g.ldb + n0 + nc);
-            const float4 f1 = *reinterpret_cast<const float4 *>(Bf + (long)(k0 + kr) * g.ldb + n0 + nc + 4);
-            v.x = f32_to_bf16_bits(f0.x) | ((unsigned int)f32_to_bf16_bits(f0.y) << 16);
-            v.y = f32_to_bf16_bits(f0.z) | ((unsigned int)f32_to_bf16_bits(f0.w) << 16);
-            v.z = f32_to_bf16_bits(f1.x) | ((unsigned int)f32_to_bf16_bits(f1.y) << 16);
-            v.w = f32_to_bf16_bits(f1.z) | ((unsigned int)f32_to_bf16_bits(f1.w) << 16);
-          } else {
-            v = *reinterpret_cast<const uint4 *>(Bh + (long)(k0 + kr) * g.ldb + n0 + nc);
-          }
-        }
-      }
+      if (n0 + row < g.N && k0 + kc < K) v = *reinterpret_cast<const uint4 *>(Bh + (long)(n0 + row) * g.ldb + k0 + kc);
       rb[c] = v;
     }
   };
-  auto store_tile = [&](unsigned short *s, const uint4 (&rv)[4], bool kmajor) {
+  auto store_tiles = [&]() {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int chunk = c * 512 + tid;
-      if (!kmajor) {
-        const int row = chunk >> 3, kc = (chunk & 7) * 8;
-        *reinterpret_cast<uint4 *>(s + row * LDS_STRIDE + kc) = rv[c];
+      const int row = chunk >> 3, kc = (chunk & 7) * 8;
+      *reinterpret_cast<uint4 *>(s_b + row * LDS_STRIDE + kc) = rb[c];
+      if (!A_KMAJOR) {
+        *reinterpret_cast<uint4 *>(s_a + row * LDS_STRIDE + kc) = ra[c];
       } else {
-        const int kr = chunk >> 5, rc = (chunk & 31) * 8;
-        const unsigned int w[4] = {rv[c].x, rv[c].y, rv[c].z, rv[c].w};
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          s[(rc + 2 * p) * LDS_STRIDE + kr] = (unsigned short)(w[p] & 0xffffu);
-          s[(rc + 2 * p + 1) * LDS_STRIDE + kr] = (unsigned short)(w[p] >> 16);
-        }
+        const int kr = chunk >> 5, mc = (chunk & 31) * 8;
+        *reinterpret_cast<uint4 *>(s_a + kr * KM_STRIDE + (mc ^ (((kr >> 3) & 1) << 5))) = ra[c];
       }
     }
   };
@@ -211,8 +223,7 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
   load_b(0);
   for (int k0 = 0; k0 < K; k0 += BK) {
     __syncthreads();  // the previous step's fragment reads are done
-    store_tile(s_a, ra, A_KMAJOR);
-    store_tile(s_b, rb, B_KMAJOR);
+    store_tiles();
     __syncthreads();
     if (k0 + BK < K) {  // prefetch the next k tile while the matrix cores work on this one
       load_a(k0 + BK);
@@ -223,8 +234,21 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
       bf16x8 fa[4], fb[2];
       const int kof = kk + (lane >> 5) * 8;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        fa[i] = *reinterpret_cast<const bf16x8 *>(s_a + (wm * 128 + i * 32 + (lane & 31)) * LDS_STRIDE + kof);
+      for (int i = 0; i < 4; ++i) {
+        const int mrow = wm * 128 + i * 32 + (lane & 31);
+        if (!A_KMAJOR) {
+          fa[i] = *reinterpret_cast<const bf16x8 *>(s_a + mrow * LDS_STRIDE + kof);
+        } else {
+          // k = kof .. kof+7 all have bit 3 equal to (lane >> 5): one swizzle for the eight reads
+          const unsigned short *col = s_a + (mrow ^ ((lane >> 5) << 5));
+          unsigned short t[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) t[e] = col[(kof + e) * KM_STRIDE];
+          typedef unsigned short us8 __attribute__((ext_vector_type(8)));
+          us8 pk = {t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7]};
+          fa[i] = __builtin_bit_cast(bf16x8, pk);
+        }
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         fb[j] = *reinterpret_cast<const bf16x8 *>(s_b + (wn * 64 + j * 32 + (lane & 31)) * LDS_STRIDE + kof);
@@ -261,10 +285,10 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
     }
 }
 
-template <bool AK, bool BK_, bool BF, int EPI>
+template <bool AK, int EPI>
 void launch_gemm(hipStream_t st, const GemmArgs &g) {
   const int groups = (g.n_slices + 7) / 8;
-  hipLaunchKernelGGL((k_gemm<AK, BK_, BF, EPI>), dim3(8 * groups * g.n_tiles), dim3(512), 0, st, g);
+  hipLaunchKernelGGL((k_gemm<AK, EPI>), dim3(8 * groups * g.n_tiles), dim3(512), 0, st, g);
 }
 
 }  // namespace
@@ -288,16 +312,31 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
   const int n_score_tiles = mt * (mt + 1) / 2;
   const int n_out_tiles = mt * nt_d, n_rho_tiles = nt_rho * nt_d;
 
-  // workspace: Q bf16 [S,T,N] | scores bf16 [S,T,Tp]
+  // workspace: Q bf16 [S,T,N] | scores bf16 [S,T,Tp] | V^T bf16 [B,d,Tp] | rho0^T bf16 [S,d,N]
   const size_t q_bytes = bdh_align_up((size_t)S * T * N * 2, 256);
   const size_t s_bytes = bdh_align_up((size_t)S * T * Tp * 2, 256);
-  int rc = bdh_ws_reserve(ctx, q_bytes + s_bytes);
+  const size_t vt_bytes = bdh_align_up((size_t)B * d * Tp * 2, 256);
+  const size_t rt_bytes = state_is_zero ? 0 : bdh_align_up((size_t)S * d * N * 2, 256);
+  int rc = bdh_ws_reserve(ctx, q_bytes + s_bytes + vt_bytes + rt_bytes);
   if (rc != BDH_OK) return rc;
   char *ws = static_cast<char *>(ctx->ws);
   unsigned short *Q = reinterpret_cast<unsigned short *>(ws);
   unsigned short *Sc = reinterpret_cast<unsigned short *>(ws + q_bytes);
-  if ((long)S * n_score_tiles > 0x7fffffffL / 16) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles (T=%d)", T);
+  unsigned short *Vt = reinterpret_cast<unsigned short *>(ws + q_bytes + s_bytes);
+  unsigned short *Rt = reinterpret_cast<unsigned short *>(ws + q_bytes + s_bytes + vt_bytes);
+  if ((long)S * n_score_tiles > 0x7fffffffL / 16 || (long)S * n_rho_tiles > 0x7fffffffL / 16)
+    return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles (T=%d N=%d)", T, N);
+  if (B > 65535 || S > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "batch too large for the transpose grid");
 
+  // 0. V^T (and rho0^T): make every B operand k-contiguous
+  hipLaunchKernelGGL(k_transpose_to_bf16<unsigned short>, dim3((d + 63) / 64, (Tp + 63) / 64, B), dim3(256), 0,
+                     ctx->stream, v_bf16, Vt, T, d, Tp);
+  BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<V>");
+  if (!state_is_zero) {
+    hipLaunchKernelGGL(k_transpose_to_bf16<float>, dim3((d + 63) / 64, (N + 63) / 64, S), dim3(256), 0, ctx->stream,
+                       rho, Rt, N, d, N);
+    BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<rho0>");
+  }
   // 1. rotation
   {
     const long work = (long)T * (N / 8);
@@ -314,40 +353,40 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
     g.lda = N; g.ldb = N; g.ldc = Tp;
     g.M = T; g.N = T; g.K = N; g.b_div = 1; g.beta = 0; g.causal_k = 0;
     g.tri = 1; g.mt = mt; g.nt = mt; g.n_tiles = n_score_tiles; g.n_slices = S;
-    launch_gemm<false, false, false, EPI_SCORES>(ctx->stream, g);
+    launch_gemm<false, EPI_SCORES>(ctx->stream, g);
     BDH_LAUNCH_CHECK(ctx, "k_gemm<scores>");
   }
   // 3a. out = Q rho0 (skipped for a fresh state)
   if (!state_is_zero) {
     GemmArgs g{};
-    g.A = Q; g.B = rho; g.C = out;
-    g.a_batch = (long)T * N; g.b_batch = (long)N * d; g.c_batch = (long)T * d;
-    g.lda = N; g.ldb = d; g.ldc = d;
+    g.A = Q; g.B = Rt; g.C = out;
+    g.a_batch = (long)T * N; g.b_batch = (long)d * N; g.c_batch = (long)T * d;
+    g.lda = N; g.ldb = N; g.ldc = d;
     g.M = T; g.N = d; g.K = N; g.b_div = 1; g.beta = 0; g.causal_k = 0;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
-    launch_gemm<false, true, true, EPI_ACC>(ctx->stream, g);
+    launch_gemm<false, EPI_ACC>(ctx->stream, g);
     BDH_LAUNCH_CHECK(ctx, "k_gemm<Q rho0>");
   }
   // 3b. out (+)= scores V
   {
     GemmArgs g{};
-    g.A = Sc; g.B = v_bf16; g.C = out;
-    g.a_batch = (long)T * Tp; g.b_batch = (long)T * d; g.c_batch = (long)T * d;
-    g.lda = Tp; g.ldb = d; g.ldc = d;
+    g.A = Sc; g.B = Vt; g.C = out;
+    g.a_batch = (long)T * Tp; g.b_batch = (long)d * Tp; g.c_batch = (long)T * d;
+    g.lda = Tp; g.ldb = Tp; g.ldc = d;
     g.M = T; g.N = d; g.K = T; g.b_div = h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 1;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
-    launch_gemm<false, true, false, EPI_ACC>(ctx->stream, g);
+    launch_gemm<false, EPI_ACC>(ctx->stream, g);
     BDH_LAUNCH_CHECK(ctx, "k_gemm<S V>");
   }
-  // 4. rho (+)= Q^T V
+  // 4. rho (+)= Q^T V   (A = Q read k-major)
   {
     GemmArgs g{};
-    g.A = Q; g.B = v_bf16; g.C = rho;
-    g.a_batch = (long)T * N; g.b_batch = (long)T * d; g.c_batch = (long)N * d;
-    g.lda = N; g.ldb = d; g.ldc = d;
+    g.A = Q; g.B = Vt; g.C = rho;
+    g.a_batch = (long)T * N; g.b_batch = (long)d * Tp; g.c_batch = (long)N * d;
+    g.lda = N; g.ldb = Tp; g.ldc = d;
     g.M = N; g.N = d; g.K = T; g.b_div = h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 0;
     g.tri = 0; g.mt = nt_rho; g.nt = nt_d; g.n_tiles = n_rho_tiles; g.n_slices = S;
-    launch_gemm<true, true, false, EPI_ACC>(ctx->stream, g);
+    launch_gemm<true, EPI_ACC>(ctx->stream, g);
     BDH_LAUNCH_CHECK(ctx, "k_gemm<Q^T V>");
   }
   return BDH_OK;
