@@ -111,6 +111,57 @@ def bench_prefill(args):
     }))
 
 
+def bench_model(args):
+    """Full-model greedy decode (BDH::forward_with_state per token, argmax on the device).
+    c1 = BASELINE config 1 (V=256, d=256, h=4, N=8192, L=6, B=1, 64-byte prompt, 256 tokens);
+    c4 = config 4 shapes (d=512, h=8, N=16384, L=12, B=32) with a SHORT prompt: the state is
+    established by --prompt tokens, not by the 3584-token prefill the config names."""
+    import torch
+
+    import burn_dragon_amd as bda
+
+    dev = torch.device("cuda:0")
+    if args.model_config == "c1":
+        cfg = bda.BDHConfig(n_layer=6, n_embd=256, n_head=4, mlp_internal_dim_multiplier=128, vocab_size=256)
+        B = 1 if args.batch == 32 else args.batch
+        steps = 256 if args.steps == 1000 else args.steps
+    else:
+        cfg = bda.BDHConfig(n_layer=12, n_embd=512, n_head=8, mlp_internal_dim_multiplier=256, vocab_size=256)
+        B = args.batch
+        steps = 64 if args.steps == 1000 else args.steps
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    rho_dtype = bda.ffi.F32 if args.rho_dtype == "f32" else bda.ffi.BF16
+    model = bda.BDH(cfg, dev, seed=7, rho_dtype=rho_dtype)
+    prompt = torch.randint(0, 256, (B, args.prompt), generator=torch.Generator().manual_seed(1))
+    state = model.init_state()
+    t0 = time.perf_counter()
+    _, nxt = model.forward_with_state(prompt, state, want_next=True)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    warm = min(args.warmup, 8)
+    for _ in range(warm):
+        _, nxt = model.forward_with_state(nxt.reshape(B, 1), state, want_next=True)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        _, nxt = model.forward_with_state(nxt.reshape(B, 1), state, want_next=True)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = max(start.elapsed_time(stop), wall * 1e3) / steps
+    h, d, N, L = cfg.n_head, cfg.n_embd, cfg.latent_per_head(), cfg.n_layer
+    print(json.dumps({
+        "metric": "decode tokens/sec, full model, greedy", "value": B / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.rho_dtype, "data": "synthetic",
+        "config": {"workload": f"full-model greedy decode {args.model_config}: L={L} d={d} h={h} N={N} V=256 B={B}, "
+                               f"random-init weights (about half the neurons active), prompt {args.prompt} tokens",
+                   "prefill_seconds": prefill_s, "state_bytes": L * B * h * N * d * (4 if args.rho_dtype == "f32" else 2)},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -124,8 +175,11 @@ def main():
     ap.add_argument("--rho-dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--ring", type=int, default=16, help="number of distinct (x, v) input sets")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode",
-                    help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA)")
+    ap.add_argument("--workload", choices=["decode", "prefill", "model"], default="decode",
+                    help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA); "
+                         "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4)")
+    ap.add_argument("--model-config", choices=["c1", "c4"], default="c1")
+    ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
     ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -146,6 +200,8 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload == "prefill":
         return bench_prefill(args)
+    if args.workload == "model":
+        return bench_model(args)
     B, h, N, d = args.batch, args.heads, args.latent, args.embd
     ctx = ffi.default_context(0)
     lib = ctx.lib

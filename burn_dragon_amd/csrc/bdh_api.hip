@@ -100,6 +100,16 @@ int bdh_ctx_synchronize(bdh_ctx *ctx) {
 
 const char *bdh_last_error(const bdh_ctx *ctx) { return ctx ? ctx->err : "null context"; }
 
+int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
+  if (!ctx || !name) return BDH_E_INVAL;
+  if (strcmp(name, "state_step.split") == 0) {
+    if (value < -1 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "state_step.split takes -1, 0 or 1");
+    ctx->opt_step_split = value;
+    return BDH_OK;
+  }
+  return bdh_fail(ctx, BDH_E_INVAL, "unknown option '%s'", name);
+}
+
 int bdh_build_freqs(int latent, float theta, int rotary, float *freqs_host) {
   if (latent < 0 || !freqs_host) return BDH_E_INVAL;
   if (rotary != BDH_ROPE && rotary != BDH_ALIBI && rotary != BDH_POPE) return BDH_E_INVAL;

@@ -17,6 +17,7 @@ struct bdh_ctx {
   void *ws = nullptr;
   size_t ws_bytes = 0;
   int n_cu = 0;
+  int opt_step_split = -1;  // -1 choose by grid size, 0 / 1 force the 256- / 64-pair workgroup
   char err[512] = {0};
 };
 

@@ -142,13 +142,13 @@ __global__ __launch_bounds__(256) void k_embed_ln(const int64_t *__restrict__ to
 // mixed[m = b*T+t, k = hh*N+n] = xy[b,hh,t,n].  Rows of E whose xy is zero for every row
 // of the tile are never loaded.
 // ------------------------------------------------------------------------------------
-template <int RT>
+template <int RT, int MAXV>
 __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict__ xy,
                                                          const float *__restrict__ E,
                                                          float *__restrict__ partial, int T, int h, int N,
                                                          int d, int KB, int M) {
   extern __shared__ float s_mem[];  // [RT][KB] xy tile, then reused for the wave reduction
-  constexpr int MAXV = 4;           // d <= 1024: up to 4 float4... columns c = (j*64+lane)*4
+  // MAXV float4 column groups per lane: columns c = (j*64+lane)*4, d <= 256*MAXV
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int kb = blockIdx.x;
   const int m0 = blockIdx.y * RT;
@@ -174,29 +174,47 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) acc[r][j] = make_float4(0.f, 0.f, 0.f, 0.f);
 
-  for (int kk = wave; kk < KB; kk += 4) {
-    const int k = kb * KB + kk;
-    if (k >= K) break;
-    float xs[RT];
-    bool any = false;
+  // each wave takes k = wave, wave+4, ...; four of its E rows are in flight at a time
+  for (int kk0 = wave; kk0 < KB; kk0 += 16) {
+    float xs[4][RT];
+    bool any[4];
+    float4 e[4][MAXV];
 #pragma unroll
-    for (int r = 0; r < RT; ++r) {
-      xs[r] = s_xy[r * KB + kk];
-      any = any || (xs[r] != 0.0f);
-    }
-    if (!any) continue;
-    const float *erow = E + (long)k * d;
-#pragma unroll
-    for (int j = 0; j < MAXV; ++j) {
-      const int c = (j * 64 + lane) * 4;
-      if (j < nv && c < d) {
-        const float4 e = *reinterpret_cast<const float4 *>(erow + c);
+    for (int u = 0; u < 4; ++u) {
+      const int kk = kk0 + 4 * u;
+      const int k = kb * KB + kk;
+      any[u] = false;
+      if (kk < KB && k < K) {
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
-          acc[r][j].x = __builtin_fmaf(xs[r], e.x, acc[r][j].x);
-          acc[r][j].y = __builtin_fmaf(xs[r], e.y, acc[r][j].y);
-          acc[r][j].z = __builtin_fmaf(xs[r], e.z, acc[r][j].z);
-          acc[r][j].w = __builtin_fmaf(xs[r], e.w, acc[r][j].w);
+          xs[u][r] = s_xy[r * KB + kk];
+          any[u] = any[u] || (xs[u][r] != 0.0f);
+        }
+      }
+      if (any[u]) {
+        const float *erow = E + (long)k * d;
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+          const int c = (j * 64 + lane) * 4;
+          if (j < nv && c < d) e[u][j] = *reinterpret_cast<const float4 *>(erow + c);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (any[u]) {
+#pragma unroll
+        for (int j = 0; j < MAXV; ++j) {
+          const int c = (j * 64 + lane) * 4;
+          if (j < nv && c < d) {
+#pragma unroll
+            for (int r = 0; r < RT; ++r) {
+              acc[r][j].x = __builtin_fmaf(xs[u][r], e[u][j].x, acc[r][j].x);
+              acc[r][j].y = __builtin_fmaf(xs[u][r], e[u][j].y, acc[r][j].y);
+              acc[r][j].z = __builtin_fmaf(xs[u][r], e[u][j].z, acc[r][j].z);
+              acc[r][j].w = __builtin_fmaf(xs[u][r], e[u][j].w, acc[r][j].w);
+            }
+          }
         }
       }
     }
@@ -220,80 +238,140 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
 }
 
 // cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))   (src/model/bdh.rs:438-441)
-__global__ __launch_bounds__(256) void k_decoder_finalize(const float *__restrict__ partial, int KBN, int M,
-                                                          int d, float *__restrict__ cur) {
-  __shared__ float s_part[4];
-  const int m = blockIdx.x, tid = threadIdx.x;
+// 1024 threads: four groups each add a quarter of the k-block partials (index order within a
+// group, groups combined in order); the first group then applies the two LayerNorms while the
+// others contribute zeros to the workgroup sums (every thread reaches every barrier).
+__global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restrict__ partial, int KBN, int M,
+                                                           int d, float *__restrict__ cur) {
+  __shared__ float s_grp[4][1024];
+  __shared__ float s_part[16];
+  const int m = blockIdx.x, tid = threadIdx.x & 255, grp = threadIdx.x >> 8;
+  const bool lead = grp == 0;
+  const int per = (KBN + 3) >> 2;
+  const int kb0 = grp * per, kb1 = min(KBN, kb0 + per);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = j * 256 + tid;
+    float v = 0.0f;
+    if (c < d) {
+      int kb = kb0;
+      for (; kb + 16 <= kb1; kb += 16) {
+        float t[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) t[u] = partial[((long)(kb + u) * M + m) * d + c];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v += t[u];
+      }
+      for (; kb < kb1; ++kb) v += partial[((long)kb * M + m) * d + c];
+    }
+    s_grp[grp][c] = v;
+  }
+  auto block_sum = [&](float v) {  // sum over the 1024 threads; all of them get the result
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) t += s_part[w];
+    return t;
+  };
+  __syncthreads();
   float vals[4];
   float s = 0.0f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int c = j * 256 + tid;
     float v = 0.0f;
-    if (c < d) {
-      for (int kb = 0; kb < KBN; ++kb) v += partial[((long)kb * M + m) * d + c];
+    if (lead && c < d) {
+      v = ((s_grp[0][c] + s_grp[1][c]) + s_grp[2][c]) + s_grp[3][c];
       s += v;
     }
     vals[j] = v;
   }
-  float mean = block_sum_256(s, s_part) / (float)d;
+  float mean = block_sum(s) / (float)d;
   float q = 0.0f;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
-    if (j * 256 + tid < d) {
+    if (lead && j * 256 + tid < d) {
       const float t = vals[j] - mean;
       q += t * t;
     }
-  float den = sqrtf(block_sum_256(q, s_part) / (float)d + kLnEps);
+  float den = sqrtf(block_sum(q) / (float)d + kLnEps);
   s = 0.0f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int c = j * 256 + tid;
-    if (c < d) {
+    if (lead && c < d) {
       const float mlp = (vals[j] - mean) / den;
       vals[j] = cur[(long)m * d + c] + mlp;
       s += vals[j];
     }
   }
-  mean = block_sum_256(s, s_part) / (float)d;
+  mean = block_sum(s) / (float)d;
   q = 0.0f;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
-    if (j * 256 + tid < d) {
+    if (lead && j * 256 + tid < d) {
       const float t = vals[j] - mean;
       q += t * t;
     }
-  den = sqrtf(block_sum_256(q, s_part) / (float)d + kLnEps);
+  den = sqrtf(block_sum(q) / (float)d + kLnEps);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int c = j * 256 + tid;
-    if (c < d) cur[(long)m * d + c] = (vals[j] - mean) / den;
+    if (lead && c < d) cur[(long)m * d + c] = (vals[j] - mean) / den;
   }
 }
 
-// logits[m,:] = cur[m,:] . lm_head ; optional argmax of the last token of each sequence
-__global__ __launch_bounds__(256) void k_lm_head(const float *__restrict__ cur, const float *__restrict__ W,
-                                                 int T, int d, int V, float *__restrict__ logits,
-                                                 int64_t *__restrict__ next_tokens) {
-  extern __shared__ float s_cur[];  // [d]
+// logits[m,:] = cur[m,:] . lm_head ; optional argmax of the last token of each sequence.
+// 1024 threads: 256 vocabulary columns x 4 groups over k; the four partial dot products of a
+// logit are added in group order.
+__global__ __launch_bounds__(1024) void k_lm_head(const float *__restrict__ cur, const float *__restrict__ W,
+                                                  int T, int d, int V, float *__restrict__ logits,
+                                                  int64_t *__restrict__ next_tokens) {
+  extern __shared__ float s_dyn[];  // [d] input row, then [4][256] partials
   __shared__ float s_best[4];
   __shared__ int s_arg[4];
-  const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int k = tid; k < d; k += 256) s_cur[k] = cur[(long)m * d + k];
+  float *s_cur = s_dyn;
+  float *s_acc = s_dyn + d;
+  const int m = blockIdx.x, tid = threadIdx.x & 255, grp = threadIdx.x >> 8;
+  const int lane = tid & 63, wave = tid >> 6;
+  for (int k = threadIdx.x; k < d; k += 1024) s_cur[k] = cur[(long)m * d + k];
   __syncthreads();
+  const int per = (d + 3) >> 2;
+  const int k0 = grp * per, k1 = min(d, k0 + per);
   float best = -INFINITY;
   int arg = 0x7fffffff;
-  for (int c = tid; c < V; c += 256) {
+  for (int c0 = 0; c0 < V; c0 += 256) {
+    const int c = c0 + tid;
     float acc = 0.0f;
-    for (int k = 0; k < d; ++k) acc = __builtin_fmaf(s_cur[k], W[(long)k * V + c], acc);
-    logits[(long)m * V + c] = acc;
-    if (acc > best) {  // strided visit in increasing c: keeps the lowest index on ties
-      best = acc;
-      arg = c;
+    if (c < V) {
+      int k = k0;
+      for (; k + 16 <= k1; k += 16) {  // 16 independent loads in flight, then the chain
+        float w[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) w[u] = W[(long)(k + u) * V + c];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc = __builtin_fmaf(s_cur[k + u], w[u], acc);
+      }
+      for (; k < k1; ++k) acc = __builtin_fmaf(s_cur[k], W[(long)k * V + c], acc);
     }
+    s_acc[grp * 256 + tid] = acc;
+    __syncthreads();
+    if (grp == 0 && c < V) {
+      const float v = ((s_acc[tid] + s_acc[256 + tid]) + s_acc[512 + tid]) + s_acc[768 + tid];
+      logits[(long)m * V + c] = v;
+      if (v > best) {  // increasing c: keeps the lowest index on ties
+        best = v;
+        arg = c;
+      }
+    }
+    __syncthreads();
   }
   const int b = m / T, t = m - b * T;
-  if (!next_tokens || t != T - 1) return;
+  const bool want = next_tokens && t == T - 1;  // uniform over the workgroup
+  if (!want) return;
   for (int o = 32; o > 0; o >>= 1) {
     const float ob = __shfl_xor(best, o);
     const int oa = __shfl_xor(arg, o);
@@ -302,12 +380,12 @@ __global__ __launch_bounds__(256) void k_lm_head(const float *__restrict__ cur, 
       arg = oa;
     }
   }
-  if (lane == 0) {
+  if (grp == 0 && lane == 0) {
     s_best[wave] = best;
     s_arg[wave] = arg;
   }
   __syncthreads();
-  if (tid == 0) {
+  if (threadIdx.x == 0) {
     for (int w = 1; w < 4; ++w)
       if (s_best[w] > best || (s_best[w] == best && s_arg[w] < arg)) {
         best = s_best[w];
@@ -380,8 +458,9 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
   const int row_tiles = (M + RT - 1) / RT;
   // k-block size: enough workgroups to fill the chip, few enough partials
+  // about two workgroups per CU: more k-blocks only add partials for the second stage to read
   int KB = 1024;
-  while (KB > 64 && ((K + KB - 1) / KB) * row_tiles < 4L * (ctx->n_cu > 0 ? ctx->n_cu : 256)) KB >>= 1;
+  while (KB > 128 && ((K + KB - 1) / KB) * row_tiles < 2L * (ctx->n_cu > 0 ? ctx->n_cu : 256)) KB >>= 1;
   const int KBN = (int)((K + KB - 1) / KB);
   size_t lds = sizeof(float) * (size_t)RT * KB;
   if (lds < sizeof(float) * 4u * d) lds = sizeof(float) * 4u * d;
@@ -390,14 +469,20 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   if (rc != BDH_OK) return rc;
   float *partial = static_cast<float *>(ctx->ws);
   dim3 grid(KBN, row_tiles);
-  switch (RT) {
-    case 8: hipLaunchKernelGGL((k_decoder_partial<8>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
-    case 4: hipLaunchKernelGGL((k_decoder_partial<4>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
-    case 2: hipLaunchKernelGGL((k_decoder_partial<2>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
-    default: hipLaunchKernelGGL((k_decoder_partial<1>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d, KB, M); break;
+#define BDH_DEC(RT_, MV_)                                                                                   \
+  hipLaunchKernelGGL((k_decoder_partial<RT_, MV_>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, \
+                     N, d, KB, M)
+  const int mv = d <= 256 ? 1 : (d <= 512 ? 2 : 4);
+  if (mv == 1) {
+    if (RT == 8) BDH_DEC(8, 1); else if (RT == 4) BDH_DEC(4, 1); else if (RT == 2) BDH_DEC(2, 1); else BDH_DEC(1, 1);
+  } else if (mv == 2) {
+    if (RT == 8) BDH_DEC(8, 2); else if (RT == 4) BDH_DEC(4, 2); else if (RT == 2) BDH_DEC(2, 2); else BDH_DEC(1, 2);
+  } else {
+    if (RT >= 4) BDH_DEC(4, 4); else if (RT == 2) BDH_DEC(2, 4); else BDH_DEC(1, 4);
   }
+#undef BDH_DEC
   BDH_LAUNCH_CHECK(ctx, "k_decoder_partial");
-  hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(256), 0, ctx->stream, partial, KBN, M, d, cur);
+  hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur);
   BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
   return BDH_OK;
 }
@@ -405,8 +490,8 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
 int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cur, const float *lm_head,
                        float *logits, int64_t *next_tokens) {
   const int M = B * T;
-  hipLaunchKernelGGL(k_lm_head, dim3(M), dim3(256), sizeof(float) * (size_t)d, ctx->stream, cur, lm_head, T, d,
-                     V, logits, next_tokens);
+  hipLaunchKernelGGL(k_lm_head, dim3(M), dim3(1024), sizeof(float) * ((size_t)d + 1024), ctx->stream, cur, lm_head,
+                     T, d, V, logits, next_tokens);
   BDH_LAUNCH_CHECK(ctx, "k_lm_head");
   return BDH_OK;
 }

@@ -75,11 +75,16 @@ struct StepPtrs {
 // ------------------------------------------------------------------------------------
 // fast path: RoPE, f32 state, D in {256, 512}
 // ------------------------------------------------------------------------------------
-template <int D, int WAVES, int U>
+// SPLIT > 1: the workgroup still has WAVES waves but owns only WAVES*64/SPLIT lane pairs; the
+// first WAVES/SPLIT waves compact them and all waves walk the list.  Used when there are few
+// (b,h) slices, so that a small batch still spreads over every CU with enough loads in flight.
+template <int D, int WAVES, int U, int SPLIT>
 __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float *__restrict__ rho) {
-  constexpr int VPL = D / 256;     // float4 per lane per row
-  constexpr int PPB = WAVES * 64;  // lane pairs per workgroup
-  __shared__ int s_cnt[WAVES];
+  constexpr int VPL = D / 256;             // float4 per lane per row
+  constexpr int PPB = WAVES * 64 / SPLIT;  // lane pairs per workgroup
+  constexpr int OW = WAVES / SPLIT;        // waves that own pairs
+  static_assert(OW >= 1 && OW * SPLIT == WAVES, "SPLIT must divide WAVES");
+  __shared__ int s_cnt[OW];
   __shared__ unsigned short s_idx[PPB];
   __shared__ float2 s_q[PPB];
   __shared__ float4 s_red[WAVES][D / 4];
@@ -91,10 +96,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
   const int seg = blockIdx.x - slice * a.S;
   const int b = slice / a.h;
   const int NP = a.N >> 1;
+  const bool owner = wave < OW;
   const int p = seg * PPB + tid;
 
   float2 xv = make_float2(0.0f, 0.0f), fv = make_float2(0.0f, 0.0f);
-  if (p < NP) {
+  if (owner && p < NP) {
     xv = reinterpret_cast<const float2 *>(a.x + (long)slice * a.x_slice_stride)[p];
     fv = reinterpret_cast<const float2 *>(a.freqs)[p];
   }
@@ -105,7 +111,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
   const unsigned long long m_act = __ballot(act);
 
   // element bitmask: two 64-bit words per wave (128 consecutive neurons)
-  if (a.bitmask) {
+  if (a.bitmask && owner) {
     const unsigned long long me = __ballot(ae), mo = __ballot(ao);
     if (lane == 0) {
       const int w0 = (seg * PPB + wave * 64) >> 5;
@@ -137,11 +143,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
   }
 
   // workgroup-wide compaction of the active pairs
-  if (lane == 0) s_cnt[wave] = __popcll(m_act);
+  if (lane == 0 && owner) s_cnt[wave] = __popcll(m_act);
   __syncthreads();
   int offset = 0, total = 0;
 #pragma unroll
-  for (int w = 0; w < WAVES; ++w) {
+  for (int w = 0; w < OW; ++w) {
     const int c = s_cnt[w];
     if (w < wave) offset += c;
     total += c;
@@ -220,7 +226,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
   for (int j = 0; j < VPL; ++j) s_red[wave][j * 64 + lane] = acc[j];
   __syncthreads();
   float *pout = a.partial + (long)blockIdx.x * D;
-  for (int c4 = tid; c4 < D / 4; c4 += PPB) {
+  for (int c4 = tid; c4 < D / 4; c4 += WAVES * 64) {
     float4 s = s_red[0][c4];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) {
@@ -236,11 +242,13 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
 // fast path: RoPE, bf16 state (f32 accumulate), D in {256, 512}.  A lane pair's two rows are
 // 4*D contiguous bytes; each lane owns D/256 16-byte pieces (8 bf16) of that chunk.
 // ------------------------------------------------------------------------------------
-template <int D, int WAVES, int U>
+template <int D, int WAVES, int U, int SPLIT>
 __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsigned short *__restrict__ rho) {
   constexpr int PL = D / 256;      // 16-byte pieces per lane per pair (D=256: 1, D=512: 2)
-  constexpr int PPB = WAVES * 64;
-  __shared__ int s_cnt[WAVES];
+  constexpr int PPB = WAVES * 64 / SPLIT;
+  constexpr int OW = WAVES / SPLIT;
+  static_assert(OW >= 1 && OW * SPLIT == WAVES, "SPLIT must divide WAVES");
+  __shared__ int s_cnt[OW];
   __shared__ unsigned short s_idx[PPB];
   __shared__ float2 s_q[PPB];
   __shared__ float s_red[WAVES][2][D];  // per wave, per row of the pair
@@ -250,10 +258,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsig
   const int seg = blockIdx.x - slice * a.S;
   const int b = slice / a.h;
   const int NP = a.N >> 1;
+  const bool owner = wave < OW;
   const int p = seg * PPB + tid;
 
   float2 xv = make_float2(0.0f, 0.0f), fv = make_float2(0.0f, 0.0f);
-  if (p < NP) {
+  if (owner && p < NP) {
     xv = reinterpret_cast<const float2 *>(a.x + (long)slice * a.x_slice_stride)[p];
     fv = reinterpret_cast<const float2 *>(a.freqs)[p];
   }
@@ -261,7 +270,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsig
   const bool ae = xv.x != 0.0f, ao = xv.y != 0.0f;
   const bool act = ae || ao;
   const unsigned long long m_act = __ballot(act);
-  if (a.bitmask) {
+  if (a.bitmask && owner) {
     const unsigned long long me = __ballot(ae), mo = __ballot(ao);
     if (lane == 0) {
       const int w0 = (seg * PPB + wave * 64) >> 5;
@@ -287,11 +296,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsig
     q.x = a0 + r0;
     q.y = a1 + r1;
   }
-  if (lane == 0) s_cnt[wave] = __popcll(m_act);
+  if (lane == 0 && owner) s_cnt[wave] = __popcll(m_act);
   __syncthreads();
   int offset = 0, total = 0;
 #pragma unroll
-  for (int w = 0; w < WAVES; ++w) {
+  for (int w = 0; w < OW; ++w) {
     const int c = s_cnt[w];
     if (w < wave) offset += c;
     total += c;
@@ -368,7 +377,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsig
   }
   __syncthreads();
   float *pout = a.partial + (long)blockIdx.x * D;
-  for (int c = tid; c < D; c += PPB) {
+  for (int c = tid; c < D; c += WAVES * 64) {
     float s = 0.0f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) s += s_red[w][0][c] + s_red[w][1][c];
@@ -564,9 +573,9 @@ void launch_finalize(hipStream_t st, int slices, const float *partial, const int
                        out_stride, out_ln, rows, rows_stride);
 }
 
-template <int D, int WAVES, int U>
+template <int D, int WAVES, int U, int SPLIT>
 void launch_fast(hipStream_t st, int blocks, const StepPtrs &a, float *rho) {
-  hipLaunchKernelGGL((k_step_rope_f32<D, WAVES, U>), dim3(blocks), dim3(WAVES * 64), 0, st, a, rho);
+  hipLaunchKernelGGL((k_step_rope_f32<D, WAVES, U, SPLIT>), dim3(blocks), dim3(WAVES * 64), 0, st, a, rho);
 }
 
 }  // namespace
@@ -580,8 +589,12 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   if ((long)slices > 0x7fffffffL / 4096) return bdh_fail(ctx, BDH_E_SHAPE, "B*h too large");
 
   const bool fast = p.rotary == BDH_ROPE && (d == 256 || d == 512) && N >= 2;
-  constexpr int WAVES = 4;
-  const int S = fast ? ((N / 2) + WAVES * 64 - 1) / (WAVES * 64) : (Nq + kGenRows - 1) / kGenRows;
+  // few slices (small batch): 64 pairs per workgroup of 8 waves, so the grid still covers the chip
+  const int n_cu = ctx->n_cu > 0 ? ctx->n_cu : 256;
+  const bool split = fast && (ctx->opt_step_split >= 0 ? ctx->opt_step_split == 1
+                                                       : (long)slices * (((N / 2) + 255) / 256) < 2L * n_cu);
+  const int ppb = split ? 64 : 256;
+  const int S = fast ? ((N / 2) + ppb - 1) / ppb : (Nq + kGenRows - 1) / kGenRows;
   if (N == 0 || d == 0) {
     // nothing to read or update: the readout is an empty sum
     if (d > 0) BDH_HIP_CHECK(ctx, hipMemsetAsync(p.out, 0, sizeof(float) * (size_t)slices * T * d, ctx->stream));
@@ -623,18 +636,23 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
     float *out_ln_t = out_ln ? out_ln + (long)t * d : nullptr;
     int32_t *rows_t = p.rows_touched ? p.rows_touched + t : nullptr;
     if (fast) {
+      const int blocks = slices * S;
       if (p.rho_dtype == BDH_F32) {
         float *rho = static_cast<float *>(p.rho);
-        if (d == 256)
-          launch_fast<256, WAVES, 2>(ctx->stream, slices * S, a, rho);
-        else
-          launch_fast<512, WAVES, 2>(ctx->stream, slices * S, a, rho);
+        if (d == 256 && !split) launch_fast<256, 4, 2, 1>(ctx->stream, blocks, a, rho);
+        if (d == 256 && split) launch_fast<256, 8, 4, 8>(ctx->stream, blocks, a, rho);
+        if (d == 512 && !split) launch_fast<512, 4, 2, 1>(ctx->stream, blocks, a, rho);
+        if (d == 512 && split) launch_fast<512, 8, 2, 8>(ctx->stream, blocks, a, rho);
       } else {
         unsigned short *rho = static_cast<unsigned short *>(p.rho);
-        if (d == 256)
-          hipLaunchKernelGGL((k_step_rope_bf16<256, WAVES, 4>), dim3(slices * S), dim3(WAVES * 64), 0, ctx->stream, a, rho);
-        else
-          hipLaunchKernelGGL((k_step_rope_bf16<512, WAVES, 2>), dim3(slices * S), dim3(WAVES * 64), 0, ctx->stream, a, rho);
+        if (d == 256 && !split)
+          hipLaunchKernelGGL((k_step_rope_bf16<256, 4, 4, 1>), dim3(blocks), dim3(256), 0, ctx->stream, a, rho);
+        if (d == 256 && split)
+          hipLaunchKernelGGL((k_step_rope_bf16<256, 8, 4, 8>), dim3(blocks), dim3(512), 0, ctx->stream, a, rho);
+        if (d == 512 && !split)
+          hipLaunchKernelGGL((k_step_rope_bf16<512, 4, 2, 1>), dim3(blocks), dim3(256), 0, ctx->stream, a, rho);
+        if (d == 512 && split)
+          hipLaunchKernelGGL((k_step_rope_bf16<512, 8, 2, 8>), dim3(blocks), dim3(512), 0, ctx->stream, a, rho);
       }
       BDH_LAUNCH_CHECK(ctx, "k_step_rope");
       launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T);

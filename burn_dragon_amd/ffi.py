@@ -21,7 +21,7 @@ F32, BF16 = 0, 1
 # every symbol include/bdh_mi355x.h declares
 EXPORTS = [
     "bdh_version", "bdh_status_string", "bdh_ctx_create", "bdh_ctx_destroy", "bdh_ctx_set_stream",
-    "bdh_ctx_synchronize", "bdh_last_error", "bdh_build_freqs", "bdh_default_alibi_slopes",
+    "bdh_ctx_synchronize", "bdh_last_error", "bdh_ctx_set_option", "bdh_build_freqs", "bdh_default_alibi_slopes",
     "bdh_recurrent_attention", "bdh_state_step", "bdh_relu_lowrank", "bdh_layer_norm",
     "bdh_fused_state_aligned", "bdh_prefill_chunked", "bdh_model_create", "bdh_model_destroy",
     "bdh_model_state_bytes", "bdh_model_forward",
@@ -75,6 +75,7 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_ctx_synchronize.argtypes = [P]
     lib.bdh_last_error.restype = c_char_p
     lib.bdh_last_error.argtypes = [P]
+    lib.bdh_ctx_set_option.argtypes = [P, c_char_p, c_int]
     lib.bdh_build_freqs.argtypes = [c_int, c_float, c_int, P]
     lib.bdh_default_alibi_slopes.argtypes = [c_int, P]
     lib.bdh_recurrent_attention.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, P, P, P,
@@ -130,6 +131,9 @@ class Context:
 
     def set_stream(self, stream: int):
         self.check(self.lib.bdh_ctx_set_stream(self.handle, stream or None))
+
+    def set_option(self, name: str, value: int):
+        self.check(self.lib.bdh_ctx_set_option(self.handle, name.encode(), int(value)))
 
     def synchronize(self):
         self.check(self.lib.bdh_ctx_synchronize(self.handle))

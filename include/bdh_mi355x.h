@@ -61,6 +61,10 @@ int bdh_ctx_destroy(bdh_ctx *ctx);
 int bdh_ctx_set_stream(bdh_ctx *ctx, void *hip_stream);
 int bdh_ctx_synchronize(bdh_ctx *ctx);
 const char *bdh_last_error(const bdh_ctx *ctx);
+/* Launch-shape knobs for tests and tuning; no counterpart in the reference.
+ *   "state_step.split": -1 (default) pick by grid size, 0 = 256 lane pairs per workgroup,
+ *                       1 = 64 lane pairs per workgroup of 8 waves (small batches). */
+int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);
 
 /* ---- host-side tables (computed on the host in the reference as well) --------------- */
 /* src/model/attention.rs:351-373  Attention::build_freqs -> freqs_host[latent] */

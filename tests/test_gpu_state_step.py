@@ -60,9 +60,19 @@ def run_gpu(recurrent_attention, x, v, rho, freqs, position, rotary, slopes=None
     return out.cpu().numpy(), rt.float().cpu().numpy(), bm.cpu().numpy().view(np.uint64), rows.cpu().numpy()
 
 
+@pytest.fixture(params=[0, 1], ids=["pairs256", "pairs64"])
+def split(request, gpu):
+    """Runs a test under both workgroup shapes of the wave-per-pair kernels."""
+    ffi, _ = gpu
+    ctx = ffi.default_context(0)
+    ctx.set_option("state_step.split", request.param)
+    yield request.param
+    ctx.set_option("state_step.split", -1)
+
+
 @pytest.mark.parametrize("d", [256, 512])
 @pytest.mark.parametrize("N,density", [(512, 0.05), (640, 0.5), (130, 1.0), (1024, 0.0), (2048, 0.02)])
-def test_fast_path_decode_step_matches_oracle(gpu, corc, N, d, density):
+def test_fast_path_decode_step_matches_oracle(gpu, corc, split, N, d, density):
     _, recurrent_attention = gpu
     B, h, T = 3, 2, 1
     x, v, rho = make_inputs(100 + N + d, B, h, T, N, d, density)
@@ -81,7 +91,7 @@ def test_fast_path_decode_step_matches_oracle(gpu, corc, N, d, density):
     assert np.array_equal(rho_new[inactive], rho[inactive])
 
 
-def test_update_is_bit_exact_when_rotation_is_exact(gpu, corc):
+def test_update_is_bit_exact_when_rotation_is_exact(gpu, corc, split):
     """At position 0 cos = 1 and sin = 0 exactly, so q == x on both sides and the rank-1 update
     rho + (q*v) (product rounded, then added: src/model/bdh.rs:298) must agree bit for bit."""
     _, recurrent_attention = gpu
@@ -124,7 +134,7 @@ def test_generic_path_small_shapes_all_rotaries(gpu, corc, rotary):
     assert np.array_equal(rows, expect_rows)
 
 
-def test_prefill_loop_equals_sequential_steps_and_causal_closed_form(gpu, corc):
+def test_prefill_loop_equals_sequential_steps_and_causal_closed_form(gpu, corc, split):
     _, recurrent_attention = gpu
     B, h, T, N, d = 2, 2, 6, 256, 256
     x, v, _ = make_inputs(31, B, h, T, N, d, 0.1)
@@ -165,7 +175,7 @@ def test_per_sequence_positions(gpu, corc):
 
 
 @pytest.mark.parametrize("N,d", [(256, 256), (384, 512), (32, 16)])
-def test_bf16_state_within_tolerance(gpu, corc, N, d):
+def test_bf16_state_within_tolerance(gpu, corc, split, N, d):
     """bf16 storage, f32 accumulate: 2e-2 relative (north_star).  d=256/512 take the wave-per-pair
     kernel, d=16 the generic one."""
     _, recurrent_attention = gpu
