@@ -111,6 +111,33 @@ def bench_prefill(args):
     }))
 
 
+def bench_copy(args):
+    """Plain device-to-device copy of a known size (1 GiB read + 1 GiB write per step): the
+    calibration run for the FETCH_SIZE / WRITE_SIZE counters and a streaming reference point."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    n = 1 << 28  # f32 elements = 1 GiB
+    src = torch.empty(n, device=dev).normal_()
+    dst = torch.empty_like(src)
+    steps = 20 if args.steps == 1000 else args.steps
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        dst.copy_(src)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / steps
+    print(json.dumps({"metric": "device copy bandwidth", "value": 2.0 * n * 4 / (ms * 1e-3) / 1e9, "unit": "GB/s",
+                      "n_gpus": 1, "steps": steps, "warmup": 3, "ms_per_step": ms, "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": "plain copy, 1 GiB read + 1 GiB write per step (counter calibration)",
+                                 "bytes_read_per_step": n * 4, "bytes_written_per_step": n * 4}}))
+
+
 def bench_model(args):
     """Full-model greedy decode (BDH::forward_with_state per token, argmax on the device).
     c1 = BASELINE config 1 (V=256, d=256, h=4, N=8192, L=6, B=1, 64-byte prompt, 256 tokens);
@@ -175,7 +202,7 @@ def main():
     ap.add_argument("--rho-dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--ring", type=int, default=16, help="number of distinct (x, v) input sets")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["decode", "prefill", "model"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy"], default="decode",
                     help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA); "
                          "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4)")
     ap.add_argument("--model-config", choices=["c1", "c4"], default="c1")
@@ -202,6 +229,8 @@ def main():
         return bench_prefill(args)
     if args.workload == "model":
         return bench_model(args)
+    if args.workload == "copy":
+        return bench_copy(args)
     B, h, N, d = args.batch, args.heads, args.latent, args.embd
     ctx = ffi.default_context(0)
     lib = ctx.lib
@@ -231,6 +260,7 @@ def main():
     R_mean = float(np.mean(R))
     bytes_per_step = 2.0 * R_mean * d * esz + 4.0 * B * h * N + 4.0 * B * d + 4.0 * B * h * d + 4.0 * N
 
+    default_workload = (B, h, N, d, args.density, args.rho_dtype) == (32, 4, 8192, 256, 0.05, "f32")
     fn, hnd = lib.bdh_state_step, ctx.handle
     call_args = [(hnd, B, h, N, d, ffi.ROPE, xs[i % args.ring].data_ptr(), vs[i % args.ring].data_ptr(),
                   freqs.data_ptr(), int(positions[i]), None, None, rho.data_ptr(), rdt, out.data_ptr(), None, None)
@@ -279,7 +309,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain copy of
+            # known size (profiles/state_step_config2_f32_pmc_traffic.md); measured for the default workload only
+            "traffic": 216.06e6 if default_workload else None,
             "kernel": "k_step_rope_f32 (+ k_step_finalize); duration = HIP-event time of the timed region / steps",
             "launch_us": kernel_us,
         },
