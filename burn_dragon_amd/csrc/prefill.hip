@@ -285,10 +285,145 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
     }
 }
 
+// ------------------------------------------------------------------------------------
+// Fast variant for full tiles (M, N multiples of 256, K a multiple of 64, both operands
+// k-contiguous): the tiles go from global memory straight into LDS (global_load_lds_dwordx4, no
+// VGPR staging, no ds_write), double buffered.  LDS tile layout: blocks of 8 rows x 128 bytes
+// (1 KiB, one wave-wide load each); inside a block the 16-byte slot of (row r, k-chunk c) is
+// r*8 + (c ^ r), which makes the 16-byte fragment reads bank-conflict free without padding.
+// Same accumulation order as k_gemm, so both give identical results.
+// ------------------------------------------------------------------------------------
+typedef __attribute__((address_space(1))) const void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+template <int EPI>
+__global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned short s_dyn[];
+  constexpr int TILE = 256 * 64;  // elements per operand tile (32 KiB)
+  constexpr int BUF = 2 * TILE;
+  const int xcd = blockIdx.x & 7;
+  const int r = blockIdx.x >> 3;
+  const int slice = xcd + 8 * (r / g.n_tiles);
+  if (slice >= g.n_slices) return;
+  int ti, tj;
+  {
+    const int t = r % g.n_tiles;
+    if (g.tri) {
+      int i = (int)((sqrtf(8.0f * (float)t + 1.0f) - 1.0f) * 0.5f);
+      while (i * (i + 1) / 2 > t) --i;
+      while ((i + 1) * (i + 2) / 2 <= t) ++i;
+      tj = t - i * (i + 1) / 2;
+      ti = i;
+    } else {
+      ti = g.mt - 1 - t / g.nt;
+      tj = t % g.nt;
+    }
+  }
+  const int m0 = ti * BM, n0 = tj * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const unsigned short *A = static_cast<const unsigned short *>(g.A) + (long)slice * g.a_batch;
+  const unsigned short *Bh = static_cast<const unsigned short *>(g.B) + (long)(slice / g.b_div) * g.b_batch;
+  int K = g.K;
+  if (g.causal_k) K = min(K, m0 + BM);
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  // source chunk of this lane inside an 8-row block: row lr, k-chunk lc (the XOR swizzle)
+  const int lr = lane >> 3, lc = (lane & 7) ^ lr;
+  const unsigned short *pa[4], *pb[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int bi = c * 8 + wave;  // 32 blocks of 8 rows per operand, 4 per wave
+    pa[c] = A + (long)(m0 + bi * 8 + lr) * g.lda + lc * 8;
+    pb[c] = Bh + (long)(n0 + bi * 8 + lr) * g.ldb + lc * 8;
+  }
+#define BDH_ISSUE_TILE(buf, k0)                                                                              \
+  _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                            \
+    const int bi = c * 8 + wave;                                                                             \
+    __builtin_amdgcn_global_load_lds((gptr_t)(pa[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + bi * 512), 16, 0, 0);        \
+    __builtin_amdgcn_global_load_lds((gptr_t)(pb[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, 0); \
+  }
+  BDH_ISSUE_TILE(0, 0)
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  int cur = 0;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    if (k0 + BK < K) { BDH_ISSUE_TILE(cur ^ 1, k0 + BK) }  // lands while the matrix cores work on this tile
+    const unsigned short *sa = s_dyn + cur * BUF, *sb = sa + TILE;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 16) {
+      bf16x8 fa[4], fb[2];
+      const int C = (kk >> 3) + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int R = wm * 128 + i * 32 + (lane & 31);
+        fa[i] = *reinterpret_cast<const bf16x8 *>(sa + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ (R & 7))) * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int R = wn * 64 + j * 32 + (lane & 31);
+        fb[j] = *reinterpret_cast<const bf16x8 *>(sb + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ (R & 7))) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    cur ^= 1;
+  }
+#undef BDH_ISSUE_TILE
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        const float v = acc[i][j][e];
+        if (EPI == EPI_SCORES) {
+          unsigned short *C = static_cast<unsigned short *>(g.C) + (long)slice * g.c_batch;
+          C[(long)row * g.ldc + col] = col < row ? f32_to_bf16_bits(v) : (unsigned short)0;  // tril(-1)
+        } else {
+          float *C = static_cast<float *>(g.C) + (long)slice * g.c_batch;
+          float *p = C + (long)row * g.ldc + col;
+          *p = g.beta ? *p + v : v;
+        }
+      }
+    }
+}
+
 template <bool AK, int EPI>
-void launch_gemm(hipStream_t st, const GemmArgs &g) {
+hipError_t launch_gemm(hipStream_t st, const GemmArgs &g) {
   const int groups = (g.n_slices + 7) / 8;
+  const bool full = !AK && g.M % BM == 0 && g.N % BN == 0 && g.K % BK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 &&
+                    (EPI != EPI_SCORES || g.ldc == g.N);
+  if constexpr (!AK) {
+    if (full) {
+      constexpr int lds = 4 * 256 * 64 * 2;  // two buffers of two 32 KiB tiles
+      static bool configured = false;
+      if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_direct<EPI>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+      }
+      hipLaunchKernelGGL((k_gemm_direct<EPI>), dim3(8 * groups * g.n_tiles), dim3(512), lds, st, g);
+      return hipSuccess;
+    }
+  }
   hipLaunchKernelGGL((k_gemm<AK, EPI>), dim3(8 * groups * g.n_tiles), dim3(512), 0, st, g);
+  return hipSuccess;
 }
 
 }  // namespace
@@ -353,7 +488,7 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
     g.lda = N; g.ldb = N; g.ldc = Tp;
     g.M = T; g.N = T; g.K = N; g.b_div = 1; g.beta = 0; g.causal_k = 0;
     g.tri = 1; g.mt = mt; g.nt = mt; g.n_tiles = n_score_tiles; g.n_slices = S;
-    launch_gemm<false, EPI_SCORES>(ctx->stream, g);
+    BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_SCORES>(ctx->stream, g)));
     BDH_LAUNCH_CHECK(ctx, "k_gemm<scores>");
   }
   // 3a. out = Q rho0 (skipped for a fresh state)
@@ -364,7 +499,7 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
     g.lda = N; g.ldb = N; g.ldc = d;
     g.M = T; g.N = d; g.K = N; g.b_div = 1; g.beta = 0; g.causal_k = 0;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
-    launch_gemm<false, EPI_ACC>(ctx->stream, g);
+    BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC>(ctx->stream, g)));
     BDH_LAUNCH_CHECK(ctx, "k_gemm<Q rho0>");
   }
   // 3b. out (+)= scores V
@@ -375,7 +510,7 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
     g.lda = Tp; g.ldb = Tp; g.ldc = d;
     g.M = T; g.N = d; g.K = T; g.b_div = h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 1;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
-    launch_gemm<false, EPI_ACC>(ctx->stream, g);
+    BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC>(ctx->stream, g)));
     BDH_LAUNCH_CHECK(ctx, "k_gemm<S V>");
   }
   // 4. rho (+)= Q^T V   (A = Q read k-major)
@@ -386,7 +521,7 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
     g.lda = N; g.ldb = Tp; g.ldc = d;
     g.M = N; g.N = d; g.K = T; g.b_div = h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 0;
     g.tri = 0; g.mt = nt_rho; g.nt = nt_d; g.n_tiles = n_rho_tiles; g.n_slices = S;
-    launch_gemm<true, EPI_ACC>(ctx->stream, g);
+    BDH_HIP_CHECK(ctx, (launch_gemm<true, EPI_ACC>(ctx->stream, g)));
     BDH_LAUNCH_CHECK(ctx, "k_gemm<Q^T V>");
   }
   return BDH_OK;

@@ -99,7 +99,8 @@ def _prefill_case(seed, B, h, T, N, d, density, rho0_scale):
 
 
 @pytest.mark.parametrize("T,N,d,rho0_scale,position", [(64, 256, 256, 0.0, 0), (200, 512, 256, 0.05, 77),
-                                                       (300, 264, 72, 0.05, 5), (520, 128, 512, 0.0, 1000)])
+                                                       (300, 264, 72, 0.05, 5), (520, 128, 512, 0.0, 1000),
+                                                       (512, 192, 256, 0.05, 33), (256, 64, 512, 0.0, 9)])
 def test_prefill_chunked_equals_sequential_recurrence(bda, corc, T, N, d, rho0_scale, position):
     """Oracle = the sequential f32 loop of src/model/bdh.rs:288-302 on the bf16-rounded inputs.
     Tolerance 2e-2 relative on the max-norm (north_star, bf16 path); Q is rounded to bf16 once
