@@ -16,8 +16,8 @@
 // always k-contiguous in memory (V and rho0 are transposed once by a small kernel).  A is either
 // k-contiguous (copied to LDS as is, fragments read with one 16-byte LDS load) or, for Q^T V,
 // k-major (Q [T,N] with the reduction over T): that tile is also copied as is, [k][m], and the
-// fragments are gathered with 2-byte LDS reads; a 64-byte column swizzle on every other group of
-// eight k rows keeps the two half-waves on different banks.
+// fragments are read with the transposing LDS load of gfx950 (ds_read_b64_tr_b16); a 64-byte
+// column swizzle on every other group of eight k rows keeps the two half-waves on different banks.
 #include "bdh_internal.h"
 
 namespace {
@@ -239,13 +239,19 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
         if (!A_KMAJOR) {
           fa[i] = *reinterpret_cast<const bf16x8 *>(s_a + mrow * LDS_STRIDE + kof);
         } else {
-          // k = kof .. kof+7 all have bit 3 equal to (lane >> 5): one swizzle for the eight reads
-          const unsigned short *col = s_a + (mrow ^ ((lane >> 5) << 5));
-          unsigned short t[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) t[e] = col[(kof + e) * KM_STRIDE];
-          typedef unsigned short us8 __attribute__((ext_vector_type(8)));
-          us8 pk = {t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7]};
+          // transposing LDS read (ds_read_b64_tr_b16): a group of 16 lanes reads a 4(k) x 16(m)
+          // block, lane j of the group supplying the address of row j/4, columns (j%4)*4..+3, and
+          // receives column j for the four k rows.  Two reads give the 8 consecutive k of lane
+          // (m = lane%32, k-group = lane/32).  Rows kof..kof+7 share bit 3 = lane>>5: one swizzle.
+          const int j16 = lane & 15;
+          const int mcol = (wm * 128 + i * 32 + ((lane >> 4) & 1) * 16) ^ ((lane >> 5) << 5);
+          const unsigned short *src = s_a + (kof + (j16 >> 2)) * KM_STRIDE + mcol + (j16 & 3) * 4;
+          typedef short s16x4 __attribute__((ext_vector_type(4)));
+          typedef short s16x8 __attribute__((ext_vector_type(8)));
+          typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_t;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(src));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(src + 4 * KM_STRIDE));
+          const s16x8 pk = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           fa[i] = __builtin_bit_cast(bf16x8, pk);
         }
       }
