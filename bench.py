@@ -169,11 +169,15 @@ def bench_model(args):
     for _ in range(warm):
         _, nxt = model.forward_with_state(nxt.reshape(B, 1), state, want_next=True)
     torch.cuda.synchronize()
+    graph = model.capture_decode_step(state, nxt) if args.graph else None
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
-    for _ in range(steps):
-        _, nxt = model.forward_with_state(nxt.reshape(B, 1), state, want_next=True)
+    if graph is not None:
+        graph.replay(steps)
+    else:
+        for _ in range(steps):
+            _, nxt = model.forward_with_state(nxt.reshape(B, 1), state, want_next=True)
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -184,7 +188,8 @@ def bench_model(args):
         "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.rho_dtype, "data": "synthetic",
         "config": {"workload": f"full-model greedy decode {args.model_config}: L={L} d={d} h={h} N={N} V=256 B={B}, "
-                               f"random-init weights (about half the neurons active), prompt {args.prompt} tokens",
+                               f"random-init weights (about half the neurons active), prompt {args.prompt} tokens"
+                               + (", one HIP graph replay per token" if args.graph else ", eager launches"),
                    "prefill_seconds": prefill_s, "state_bytes": L * B * h * N * d * (4 if args.rho_dtype == "f32" else 2)},
     }))
 
@@ -207,6 +212,7 @@ def main():
                          "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4)")
     ap.add_argument("--model-config", choices=["c1", "c4"], default="c1")
     ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
+    ap.add_argument("--graph", action="store_true", help="model: replay one captured HIP graph per token")
     ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")
     args = ap.parse_args()
     if args.gpus != 1:

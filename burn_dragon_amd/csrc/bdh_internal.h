@@ -100,3 +100,5 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
 // logits = cur . lm_head (+ argmax of the last token per sequence) (src/model/bdh.rs:446-449)
 int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cur,
                        const float *lm_head, float *logits, int64_t *next_tokens);
+// positions[b] = min(positions[b] + delta, INT32_MAX): the device-side form of state.position += T
+int bdh_launch_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta);

@@ -80,6 +80,13 @@ int bdh_model_destroy(bdh_model *m) {
   return BDH_OK;
 }
 
+int bdh_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta) {
+  if (!ctx) return BDH_E_INVAL;
+  if (B < 0 || (B > 0 && !positions_dev)) return bdh_fail(ctx, BDH_E_INVAL, "bad positions buffer");
+  if (B == 0) return BDH_OK;
+  return bdh_launch_advance_positions(ctx, positions_dev, B, delta);
+}
+
 size_t bdh_model_state_bytes(const bdh_model *m, int B, int rho_dtype) {
   if (!m || B < 0) return 0;
   const size_t Nq = m->cfg.rotary == BDH_POPE ? 2 * (size_t)m->cfg.latent : (size_t)m->cfg.latent;
@@ -89,6 +96,12 @@ size_t bdh_model_state_bytes(const bdh_model *m, int B, int rho_dtype) {
 
 int bdh_model_forward(bdh_model *m, const int64_t *tokens, int B, int T, void *rho, int rho_dtype,
                       int64_t position, float *logits, int64_t *next_tokens, float *x_tap) {
+  return bdh_model_forward_ex(m, tokens, B, T, rho, rho_dtype, position, nullptr, logits, next_tokens, x_tap);
+}
+
+int bdh_model_forward_ex(bdh_model *m, const int64_t *tokens, int B, int T, void *rho, int rho_dtype,
+                         int64_t position, const int32_t *positions_dev, float *logits, int64_t *next_tokens,
+                         float *x_tap) {
   if (!m) return BDH_E_INVAL;
   bdh_ctx *ctx = m->ctx;
   if (B < 0 || T < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative batch or time");
@@ -122,7 +135,7 @@ int bdh_model_forward(bdh_model *m, const int64_t *tokens, int B, int T, void *r
     rc = bdh_launch_relu_lowrank(ctx, px);
     if (rc != BDH_OK) return rc;
     // :353-359  recurrent attention (value = cur) and LayerNorm of its output
-    StateStepParams ps{B, h, T, N, d, c.rotary, rho_dtype, x_l, cur, m->freqs, position, nullptr,
+    StateStepParams ps{B, h, T, N, d, c.rotary, rho_dtype, x_l, cur, m->freqs, position, positions_dev,
                        c.rotary == BDH_ALIBI ? m->slopes : nullptr,
                        static_cast<char *>(rho) + (size_t)l * rho_layer_bytes, attn, nullptr, nullptr};
     rc = bdh_launch_state_steps_ln(ctx, ps, attn_ln);

@@ -395,6 +395,14 @@ __global__ __launch_bounds__(1024) void k_lm_head(const float *__restrict__ cur,
   }
 }
 
+__global__ void k_advance_positions(int32_t *pos, int B, int delta) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < B) {
+    const long v = (long)pos[b] + delta;
+    pos[b] = v > 0x7fffffffL ? 0x7fffffff : (int32_t)v;  // saturating, as state.position (src/model/bdh.rs:445)
+  }
+}
+
 template <int RT>
 void launch_relu(hipStream_t st, dim3 grid, size_t lds, const ReluLowrankParams &p, const unsigned char *mask,
                  int M) {
@@ -493,5 +501,11 @@ int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cu
   hipLaunchKernelGGL(k_lm_head, dim3(M), dim3(1024), sizeof(float) * ((size_t)d + 1024), ctx->stream, cur, lm_head,
                      T, d, V, logits, next_tokens);
   BDH_LAUNCH_CHECK(ctx, "k_lm_head");
+  return BDH_OK;
+}
+
+int bdh_launch_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta) {
+  hipLaunchKernelGGL(k_advance_positions, dim3((B + 255) / 256), dim3(256), 0, ctx->stream, positions_dev, B, delta);
+  BDH_LAUNCH_CHECK(ctx, "k_advance_positions");
   return BDH_OK;
 }

@@ -1,5 +1,5 @@
-from .bdh import BDH
+from .bdh import BDH, DecodeGraph
 from .config import BDHConfig, FusedKernelConfig
 from .state import LayerState, ModelState
 
-__all__ = ["BDH", "BDHConfig", "FusedKernelConfig", "LayerState", "ModelState"]
+__all__ = ["BDH", "DecodeGraph", "BDHConfig", "FusedKernelConfig", "LayerState", "ModelState"]

@@ -100,6 +100,13 @@ class BDH:
         state.position = min(state.position + T, UINT63_MAX)  # saturating_add, :445
         return (logits, nxt) if want_next else logits
 
+    def capture_decode_step(self, state: ModelState, tokens: torch.Tensor) -> "DecodeGraph":
+        """Captures ONE greedy decode step (forward_with_state on the last sampled token, argmax kept on
+        the device, position advanced on the device) in a HIP graph.  Every replay is one token for
+        every sequence of the batch; nothing crosses to the host between tokens (the reference syncs
+        and copies the logits every token, src/generation.rs:114-124)."""
+        return DecodeGraph(self, state, tokens)
+
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
         """src/model/bdh.rs:91-94."""
         return self.forward_with_state(tokens, self.init_state())
@@ -116,3 +123,46 @@ class BDH:
             out.append(tok)
             _, nxt = self.forward_with_state(tok, state, want_next=True)
         return torch.cat(out, dim=1)
+
+
+class DecodeGraph:
+    """One captured decode step.  `tokens` [B] int64 are the tokens to feed first (e.g. the argmax of the
+    prefill); after each replay() the buffer holds the newly generated tokens and `logits` [B,1,V] the
+    logits they were taken from.  The state must already hold its rho tensors (run the prefill first)."""
+
+    def __init__(self, model: BDH, state: ModelState, tokens: torch.Tensor):
+        assert state.storage is not None, "run the prefill before capturing the decode step"
+        self.model, self.state = model, state
+        B = state.storage.shape[1]
+        dev = model.device
+        self.tokens = tokens.to(dev, torch.int64).reshape(B).clone()
+        self.positions = torch.full((B,), state.position, device=dev, dtype=torch.int32)
+        self.logits = torch.empty((B, 1, model.vocab_size), device=dev, dtype=torch.float32)
+        ctx, lib = model.ctx, model.ctx.lib
+
+        def step():
+            ctx.check(lib.bdh_model_forward_ex(model.handle, self.tokens.data_ptr(), B, 1, state.storage.data_ptr(),
+                                               model.rho_dtype, 0, self.positions.data_ptr(), self.logits.data_ptr(),
+                                               self.tokens.data_ptr(), None))
+            ctx.check(lib.bdh_advance_positions(ctx.handle, self.positions.data_ptr(), B, 1))
+
+        # one eager step on a side stream sizes every scratch buffer (no allocation may happen under capture)
+        keep = (self.tokens.clone(), self.positions.clone(), state.storage.clone())
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            ctx.set_stream(side.cuda_stream)
+            step()
+        side.synchronize()
+        self.tokens.copy_(keep[0]); self.positions.copy_(keep[1]); state.storage.copy_(keep[2])
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=side):
+            ctx.set_stream(torch.cuda.current_stream(dev).cuda_stream)
+            step()
+        ctx.set_stream(torch.cuda.current_stream(dev).cuda_stream)
+
+    def replay(self, n: int = 1) -> None:
+        for _ in range(n):
+            self.graph.replay()
+        self.state.position = min(self.state.position + n, UINT63_MAX)

@@ -225,6 +225,22 @@ int bdh_model_forward(bdh_model *model, const int64_t *tokens, int B, int T, voi
                       int rho_dtype, int64_t position, float *logits, int64_t *next_tokens,
                       float *x_tap);
 
+/*
+ * bdh_model_forward with per-sequence start positions kept in DEVICE memory (int32 [B]); when
+ * positions_dev is not NULL it overrides `position`.  Together with next_tokens feeding the next
+ * call's tokens this makes one decode step a fixed sequence of launches with no host-side
+ * arguments that change from token to token, so a caller can capture it in a HIP graph and replay
+ * it.  (The reference keeps one host-side position, src/model/state.rs:14, and round-trips the
+ * token through the host, src/generation.rs:114-124.)
+ */
+int bdh_model_forward_ex(bdh_model *model, const int64_t *tokens, int B, int T, void *rho,
+                         int rho_dtype, int64_t position, const int32_t *positions_dev,
+                         float *logits, int64_t *next_tokens, float *x_tap);
+
+/* positions_dev[b] = saturating(positions_dev[b] + delta): the device-side form of
+ * `state.position += T` (src/model/bdh.rs:445). */
+int bdh_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta);
+
 #ifdef __cplusplus
 }
 #endif

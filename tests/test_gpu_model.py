@@ -202,3 +202,30 @@ def test_model_create_rejects_bad_configs(bda):
     with pytest.raises(ffi.BdhError) as err:
         bda.BDH(cfg, DEV, seed=1)
     assert err.value.status == ffi.E_SHAPE
+
+
+def test_decode_graph_replays_match_eager_steps(bda):
+    """A captured decode step is replayed several times, with eager work and synchronisations of the
+    same program between the replays, and every replay is checked against the eager path."""
+    cfg = bda.BDHConfig(n_layer=3, n_embd=256, n_head=4, mlp_internal_dim_multiplier=16, vocab_size=64)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    model = bda.BDH(cfg, DEV, seed=21)
+    prompt = torch.randint(0, 64, (2, 5), generator=torch.Generator().manual_seed(2))
+    se, sg = model.init_state(), model.init_state()
+    _, nxt_e = model.forward_with_state(prompt, se, want_next=True)
+    _, nxt_g = model.forward_with_state(prompt, sg, want_next=True)
+    graph = model.capture_decode_step(sg, nxt_g)
+    assert torch.equal(sg.storage, se.storage)  # capture must not disturb the state
+    for step in range(6):
+        logits_e, new_e = model.forward_with_state(nxt_e.reshape(2, 1), se, want_next=True)
+        torch.cuda.synchronize()
+        junk = torch.randn(1 << 16, device=DEV).sum()  # unrelated eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(graph.logits, logits_e), f"replay {step}"
+        assert torch.equal(graph.tokens, new_e)
+        assert torch.equal(sg.storage, se.storage)
+        assert sg.position == se.position == 6 + step
+        assert int(graph.positions[0]) == sg.position
+        nxt_e = new_e
+        del junk
