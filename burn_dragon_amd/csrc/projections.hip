@@ -22,8 +22,8 @@ __device__ __forceinline__ float block_sum_256(float v, float *s_part) {
 // One thread per latent column n (coalesced weight rows), RT input rows per workgroup
 // staged in LDS, one k-sequential fmaf chain per output.
 // ------------------------------------------------------------------------------------
-template <int RT, int UK>
-__global__ __launch_bounds__(256) void k_relu_lowrank(const float *__restrict__ in, int h_in, int T, int d,
+template <int RT, int UK, int NTHR>
+__global__ __launch_bounds__(NTHR) void k_relu_lowrank(const float *__restrict__ in, int h_in, int T, int d,
                                                       const float *__restrict__ w, int h, int N,
                                                       const float *__restrict__ bias, float thr,
                                                       const unsigned char *__restrict__ block_active,
@@ -33,9 +33,9 @@ __global__ __launch_bounds__(256) void k_relu_lowrank(const float *__restrict__ 
   extern __shared__ float s_in[];  // [RT][d]
   const int tid = threadIdx.x;
   const int hh = blockIdx.y;
-  const int n = blockIdx.x * 256 + tid;
+  const int n = blockIdx.x * NTHR + tid;
   const int m0 = blockIdx.z * RT;
-  for (int i = tid; i < RT * d; i += 256) {
+  for (int i = tid; i < RT * d; i += NTHR) {
     const int r = i / d, k = i - r * d;
     const int m = m0 + r;
     float val = 0.0f;
@@ -239,14 +239,12 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
 
 // cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))   (src/model/bdh.rs:438-441)
 // 1024 threads: four groups each add a quarter of the k-block partials (index order within a
-// group, groups combined in order); the first group then applies the two LayerNorms while the
-// others contribute zeros to the workgroup sums (every thread reaches every barrier).
+// group, groups combined in order); after the one barrier the first wavefront applies the two
+// LayerNorms with wave shuffles only.
 __global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restrict__ partial, int KBN, int M,
                                                            int d, float *__restrict__ cur) {
   __shared__ float s_grp[4][1024];
-  __shared__ float s_part[16];
   const int m = blockIdx.x, tid = threadIdx.x & 255, grp = threadIdx.x >> 8;
-  const bool lead = grp == 0;
   const int per = (KBN + 3) >> 2;
   const int kb0 = grp * per, kb1 = min(KBN, kb0 + per);
 #pragma unroll
@@ -266,61 +264,57 @@ __global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restri
     }
     s_grp[grp][c] = v;
   }
-  auto block_sum = [&](float v) {  // sum over the 1024 threads; all of them get the result
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float t = 0.0f;
-#pragma unroll
-    for (int w = 0; w < 16; ++w) t += s_part[w];
-    return t;
-  };
   __syncthreads();
-  float vals[4];
+  if (threadIdx.x >= 64) return;  // no barrier follows: the first wave finishes the row alone
+  const int lane = threadIdx.x;
+  float vals[16];  // column c = j*64 + lane, d <= 1024
   float s = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int c = j * 256 + tid;
+  for (int j = 0; j < 16; ++j) {
+    const int c = j * 64 + lane;
     float v = 0.0f;
-    if (lead && c < d) {
+    if (c < d) {
       v = ((s_grp[0][c] + s_grp[1][c]) + s_grp[2][c]) + s_grp[3][c];
       s += v;
     }
     vals[j] = v;
   }
-  float mean = block_sum(s) / (float)d;
+  auto wave_sum = [](float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+  };
+  float mean = wave_sum(s) / (float)d;
   float q = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    if (lead && j * 256 + tid < d) {
+  for (int j = 0; j < 16; ++j)
+    if (j * 64 + lane < d) {
       const float t = vals[j] - mean;
       q += t * t;
     }
-  float den = sqrtf(block_sum(q) / (float)d + kLnEps);
+  float den = sqrtf(wave_sum(q) / (float)d + kLnEps);
   s = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int c = j * 256 + tid;
-    if (lead && c < d) {
+  for (int j = 0; j < 16; ++j) {
+    const int c = j * 64 + lane;
+    if (c < d) {
       const float mlp = (vals[j] - mean) / den;
       vals[j] = cur[(long)m * d + c] + mlp;
       s += vals[j];
     }
   }
-  mean = block_sum(s) / (float)d;
+  mean = wave_sum(s) / (float)d;
   q = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    if (lead && j * 256 + tid < d) {
+  for (int j = 0; j < 16; ++j)
+    if (j * 64 + lane < d) {
       const float t = vals[j] - mean;
       q += t * t;
     }
-  den = sqrtf(block_sum(q) / (float)d + kLnEps);
+  den = sqrtf(wave_sum(q) / (float)d + kLnEps);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int c = j * 256 + tid;
-    if (lead && c < d) cur[(long)m * d + c] = (vals[j] - mean) / den;
+  for (int j = 0; j < 16; ++j) {
+    const int c = j * 64 + lane;
+    if (c < d) cur[(long)m * d + c] = (vals[j] - mean) / den;
   }
 }
 
@@ -406,8 +400,11 @@ __global__ void k_advance_positions(int32_t *pos, int B, int delta) {
 template <int RT>
 void launch_relu(hipStream_t st, dim3 grid, size_t lds, const ReluLowrankParams &p, const unsigned char *mask,
                  int M) {
-  hipLaunchKernelGGL((k_relu_lowrank<RT, 16>), grid, dim3(256), lds, st, p.in, p.h_in, p.T, p.d, p.weight, p.h,
-                     p.N, p.bias, p.threshold, mask, p.block_size, p.n_blocks, p.gate, p.out, M);
+  constexpr int UK = RT == 1 ? 32 : 16;      // weight rows in flight per thread
+  constexpr int NTHR = RT == 1 ? 128 : 256;  // a single input row: smaller workgroups, one per CU at N*h = 32768
+  grid.x = (p.N + NTHR - 1) / NTHR;
+  hipLaunchKernelGGL((k_relu_lowrank<RT, UK, NTHR>), grid, dim3(NTHR), lds, st, p.in, p.h_in, p.T, p.d, p.weight,
+                     p.h, p.N, p.bias, p.threshold, mask, p.block_size, p.n_blocks, p.gate, p.out, M);
 }
 
 }  // namespace
