@@ -54,6 +54,35 @@ def cpu_baseline(B, h, N, d, freqs, budget_s=12.0, max_steps=20):
     }
 
 
+def cpu_baseline_model(cfg, B, prompt, budget_s=20.0, max_tokens=256):
+    """Config 1 end to end on this host with the restated reference path (dense state passes of
+    src/model/bdh.rs:288-302, the same seeded weights and prompt as the GPU run): the prompt as
+    one call, then greedy decode tokens until the time budget is used."""
+    from oracle import bdh_oracle as orc
+
+    c = orc.COracle()
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    shape = orc.BDHShape(n_layer=cfg.n_layer, n_embd=cfg.n_embd, n_head=cfg.n_head,
+                         mlp_internal_dim_multiplier=cfg.mlp_internal_dim_multiplier, vocab_size=cfg.vocab_size,
+                         rotary=orc.ROPE)
+    w = orc.init_weights(shape, 7)
+    rho = np.zeros((cfg.n_layer, B, cfg.n_head, shape.latent_per_head, cfg.n_embd), np.float32)
+    t0 = time.perf_counter()
+    logits, pos, _, _ = c.forward_with_state(shape, w, prompt, rho, 0, sparse_state=False)
+    t_prompt = time.perf_counter() - t0
+    toks = np.array([[c.greedy_token(logits[b, -1])] for b in range(B)])
+    n, t1 = 0, time.perf_counter()
+    while n < max_tokens and (time.perf_counter() - t1) < budget_s:
+        logits, pos, _, _ = c.forward_with_state(shape, w, toks, rho, pos, sparse_state=False)
+        toks = np.array([[c.greedy_token(logits[b, -1])] for b in range(B)])
+        n += 1
+    dt = time.perf_counter() - t1
+    return {"value": B * n / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"{prompt.shape[1]}-token prompt in {t_prompt:.2f} s, then {n} greedy decode tokens at "
+                      f"{dt / n * 1e3:.1f} ms/token; C restatement of the reference op sequence with dense state passes, "
+                      f"OpenMP; same seeded weights and prompt as the GPU run"}
+
+
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
@@ -161,8 +190,13 @@ def bench_model(args):
     model = bda.BDH(cfg, dev, seed=7, rho_dtype=rho_dtype)
     prompt = torch.randint(0, 256, (B, args.prompt), generator=torch.Generator().manual_seed(1))
     state = model.init_state()
+    chunk = args.prefill_chunk or args.prompt
     t0 = time.perf_counter()
-    _, nxt = model.forward_with_state(prompt, state, want_next=True)
+    for lo in range(0, args.prompt, chunk):  # bounded activation memory; same result as one call
+        _, nxt = model.forward_with_state(prompt[:, lo:lo + chunk], state, want_next=True)
+        if (lo // chunk) % 16 == 15:
+            torch.cuda.synchronize()
+            print(f"prefill {lo + chunk}/{args.prompt} tokens, {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
     warm = min(args.warmup, 8)
@@ -183,6 +217,9 @@ def bench_model(args):
     wall = time.perf_counter() - t0
     ms = max(start.elapsed_time(stop), wall * 1e3) / steps
     h, d, N, L = cfg.n_head, cfg.n_embd, cfg.latent_per_head(), cfg.n_layer
+    extra = {}
+    if args.model_config == "c1" and not args.no_cpu_baseline:
+        extra["cpu_baseline"] = cpu_baseline_model(cfg, B, prompt.numpy())
     print(json.dumps({
         "metric": "decode tokens/sec, full model, greedy", "value": B / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
@@ -190,7 +227,9 @@ def bench_model(args):
         "config": {"workload": f"full-model greedy decode {args.model_config}: L={L} d={d} h={h} N={N} V=256 B={B}, "
                                f"random-init weights (about half the neurons active), prompt {args.prompt} tokens"
                                + (", one HIP graph replay per token" if args.graph else ", eager launches"),
-                   "prefill_seconds": prefill_s, "state_bytes": L * B * h * N * d * (4 if args.rho_dtype == "f32" else 2)},
+                   "prefill_seconds": prefill_s, "prefill_tokens_per_s": B * args.prompt / prefill_s,
+                   "state_bytes": L * B * h * N * d * (4 if args.rho_dtype == "f32" else 2)},
+        **extra,
     }))
 
 
@@ -207,6 +246,8 @@ def main():
     ap.add_argument("--rho-dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--ring", type=int, default=16, help="number of distinct (x, v) input sets")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--prefill-chunk", type=int, default=0,
+                    help="model workload: feed the prompt in calls of this many tokens (0 = one call)")
     ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy"], default="decode",
                     help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA); "
                          "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4)")

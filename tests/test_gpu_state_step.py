@@ -260,3 +260,24 @@ def test_full_size_config2_properties(gpu, corc):
     assert torch.equal(rho[~active_rows], rho_before[~active_rows])
     frac = float(active_rows.float().mean())
     assert 0.09 < frac < 0.105  # 1 - 0.95^2 = 9.75 % of the rows
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
+@pytest.mark.parametrize("density", [0.01, 0.05, 0.20])
+def test_config5_shapes_max_relative_error(gpu, corc, dtype, tol, density):
+    """BASELINE config 5 (the config-4 layer shape h=8, N=16384, d=512) at B=1: the step of every
+    density of the sweep, f32 and bf16 state, against the oracle started from the same (bf16-rounded,
+    where it applies) state.  The printed errors are the max-rel-err column of the sweep table."""
+    _, recurrent_attention = gpu
+    B, h, N, d = 1, 8, 16384, 512
+    x, v, rho = make_inputs(int(density * 100), B, h, 1, N, d, density)
+    if dtype == torch.bfloat16:
+        rho = torch.from_numpy(rho).to(torch.bfloat16).float().numpy()
+    freqs = corc.build_freqs(N)
+    out, rho_new, bm, rows = run_gpu(recurrent_attention, x, v, rho, freqs, 4000, orc.ROPE, dtype=dtype)
+    out_ref, rho_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.ROPE, 4000), v, rho)
+    e_out, e_rho = rel_err(out, out_ref), rel_err(rho_new, rho_ref)
+    print(f"config-5 shape B=1 density {density:.0%} {dtype}: readout rel err {e_out:.2e}, state rel err {e_rho:.2e}")
+    assert e_out < tol and e_rho < tol
+    assert np.array_equal(rows, orc.pair_closed_rows(x))
+    assert np.array_equal(bm, orc.active_bitmask(x))
