@@ -62,6 +62,18 @@ class BDH:
         self.handle = handle
         self.latent_q = 2 * N if rot == RotaryEmbedding.POPE else N
 
+    @classmethod
+    def from_checkpoint_dir(cls, directory: str, device="cuda:0", rho_dtype: int = ffi.F32):
+        """A trained model from a directory holding the reference's model.bin (Burn BinFileRecorder
+        record), config.json and optionally vocab.json — the loading steps of src/bin/infer.rs:170-186.
+        Returns (model, tokenizer or None, block_size)."""
+        from ..record import load_checkpoint_dir
+        from ..tokenizer import CharVocab
+
+        config, weights, vocab_json, block_size = load_checkpoint_dir(directory)
+        tokenizer = CharVocab.from_json_str(vocab_json) if vocab_json is not None else None
+        return cls(config, device, weights=weights, rho_dtype=rho_dtype), tokenizer, block_size
+
     def __del__(self):
         try:
             if getattr(self, "handle", None):

@@ -241,6 +241,18 @@ int bdh_model_forward_ex(bdh_model *model, const int64_t *tokens, int B, int T, 
  * `state.position += T` (src/model/bdh.rs:445). */
 int bdh_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta);
 
+/* Draws the next token of every sequence on the device.  Replaces the temperature division of
+ * sample_next_token (src/generation.rs:117) and sample_from_logits_values (src/generation.rs:26-72),
+ * which copy the logits to the host for every token: values = logits / temperature; with
+ * 0 < top_k < V everything below the k-th largest value is masked to -inf (ties with it survive);
+ * softmax (uniform over V when the sum is 0 or NaN); the index is drawn as rand's WeightedIndex
+ * draws it, from the running sums in index order, with uniforms[b] in [0,1) standing for the
+ * variate the reference takes from thread_rng.  top_k <= 0 means no truncation (`None`).
+ * logits: row b starts at logits + b*row_stride (pass the last-token row of [B,T,V] logits with
+ * row_stride = T*V).  V <= 8192.  next_tokens [B] int64 can be fed back as the next call's tokens. */
+int bdh_sample_top_k(bdh_ctx *ctx, int B, int V, const float *logits, int64_t row_stride,
+                     float temperature, int top_k, const float *uniforms, int64_t *next_tokens);
+
 #ifdef __cplusplus
 }
 #endif

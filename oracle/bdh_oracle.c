@@ -526,6 +526,58 @@ int orc_greedy_token(const float *logits, int V) {
   return best;
 }
 
+/* sample_next_token's temperature division (src/generation.rs:117) followed by
+ * sample_from_logits_values (:26-72), with the random draw made explicit: `u` in
+ * [0,1) stands for the uniform variate WeightedIndex takes from thread_rng.
+ * WeightedIndex (rand 0.8) keeps the running sums of the first V-1 weights, draws
+ * `chosen` uniformly in [0, total) and returns the number of running sums that
+ * are <= chosen.  All sums run in index order in binary32, as the iterator sums
+ * of the reference do.  The k-th largest value is found by a full descending sort
+ * like the reference's (:40-41); ties with it survive the mask (:43-45). */
+static int orc_cmp_desc(const void *a, const void *b) {
+  const float x = *(const float *)a, y = *(const float *)b;
+  return (x < y) - (x > y);
+}
+int orc_sample_from_logits(const float *logits, int V, float temperature, int top_k, float u,
+                           float *probs_out) {
+  float *v = (float *)malloc(sizeof(float) * (size_t)V * 2);
+  float *sorted = v + V;
+  for (int i = 0; i < V; ++i) v[i] = logits[i] / temperature;
+  if (top_k > 0 && top_k < V) {
+    memcpy(sorted, v, sizeof(float) * (size_t)V);
+    qsort(sorted, (size_t)V, sizeof(float), orc_cmp_desc);
+    const float threshold = sorted[top_k - 1];
+    for (int i = 0; i < V; ++i)
+      if (v[i] < threshold) v[i] = -INFINITY;
+  }
+  float m = -INFINITY;
+  for (int i = 0; i < V; ++i) m = fmaxf(m, v[i]);
+  float sum = 0.f;
+  for (int i = 0; i < V; ++i) {
+    v[i] = expf(v[i] - m);
+    sum += v[i];
+  }
+  const int flat = (sum == 0.f) || (sum != sum);
+  float total = 0.f;
+  for (int i = 0; i < V; ++i) {
+    v[i] = flat ? 1.0f / (float)V : v[i] / sum;
+    total += v[i];
+  }
+  if (probs_out) memcpy(probs_out, v, sizeof(float) * (size_t)V);
+  if (u < 0.f) u = 0.f;
+  if (u > 0.99999994f) u = 0.99999994f;
+  const float chosen = u * total;
+  float cum = 0.f;
+  int idx = 0;
+  for (int i = 0; i < V - 1; ++i) {
+    cum += v[i];
+    if (cum <= chosen) idx = i + 1;
+    else break;
+  }
+  free(v);
+  return idx;
+}
+
 /* One dense decode step of the single-layer microbenchmark shape (rotate +
  * recurrent_attention with T = 1), used as the timed CPU baseline. */
 void orc_state_step_dense(const float *x, const float *v, const float *freqs, int64_t position,

@@ -315,6 +315,29 @@ def greedy_token(logits_row) -> int:
     return int(np.argmax(logits_row))
 
 
+def sample_from_logits(logits_row, temperature: float, top_k: Optional[int], u: float, dtype=np.float32):
+    """src/generation.rs:117 and :26-72 with the uniform variate `u` of WeightedIndex explicit.
+    Returns (index, probabilities)."""
+    v = (np.asarray(logits_row, dtype) / dtype(temperature)).astype(dtype)
+    V = v.size
+    if top_k is not None and 0 < top_k < V:
+        threshold = np.sort(v)[::-1][top_k - 1]
+        v = np.where(v < threshold, dtype(-np.inf), v)
+    with np.errstate(invalid="ignore"):
+        p = np.exp(v - np.nanmax(v) if not np.all(np.isnan(v)) else v).astype(dtype)
+    s = dtype(0)
+    for e in p:
+        s = dtype(s + e)
+    p = np.full(V, dtype(1) / dtype(V), dtype) if (s == 0 or np.isnan(s)) else (p / s).astype(dtype)
+    cum = np.zeros(V, dtype)
+    acc = dtype(0)
+    for i, e in enumerate(p):
+        acc = dtype(acc + e)
+        cum[i] = acc
+    chosen = dtype(min(max(u, 0.0), 0.99999994)) * cum[-1]
+    return int(np.searchsorted(cum[:-1], chosen, side="right")), p
+
+
 # --------------------------------------------------------------------------
 # helpers shared by tests: what the compaction must produce
 # --------------------------------------------------------------------------
@@ -382,6 +405,7 @@ class COracle:
         self.lib = ctypes.CDLL(path)
         self.lib.orc_forward_with_state.restype = ctypes.c_int
         self.lib.orc_greedy_token.restype = ctypes.c_int
+        self.lib.orc_sample_from_logits.restype = ctypes.c_int
 
     def build_freqs(self, latent, theta=ROPE_THETA, rotary=ROPE):
         out = np.empty(latent, np.float32)
@@ -500,6 +524,14 @@ class COracle:
     def greedy_token(self, logits_row) -> int:
         row = _f32(logits_row)
         return int(self.lib.orc_greedy_token(_p(row), ctypes.c_int(row.size)))
+
+    def sample_from_logits(self, logits_row, temperature, top_k, u):
+        row = _f32(logits_row)
+        probs = np.empty(row.size, np.float32)
+        idx = self.lib.orc_sample_from_logits(_p(row), ctypes.c_int(row.size), ctypes.c_float(temperature),
+                                              ctypes.c_int(0 if top_k is None else int(top_k)), ctypes.c_float(u),
+                                              _p(probs))
+        return int(idx), probs
 
     def state_step_dense(self, x, v, freqs, position, rho):
         """Single-layer decode step (rotate + dense recurrent_attention, T=1); rho IN PLACE."""

@@ -389,3 +389,69 @@ def test_bitmask_and_pair_rows_helpers():
     assert bm.shape == (2, 2)
     assert bm[0, 0] == 1 and bm[0, 1] == 2 and bm[1, 0] == 0 and bm[1, 1] == np.uint64(1) << np.uint64(63)
     assert orc.pair_closed_rows(x).tolist() == [4, 2]
+
+
+# ---- sampling (src/generation.rs:26-72): pinned by the softmax of a library, an inverse CDF in
+# float64, the argmax special case and the draw frequencies ----
+def test_sampler_probabilities_are_the_softmax_of_the_scaled_logits(corc):
+    from scipy.special import softmax
+
+    rng = np.random.default_rng(0)
+    logits = (3 * rng.standard_normal(69)).astype(np.float32)
+    for temperature in (0.5, 1.0, 1.7):
+        _, p = corc.sample_from_logits(logits, temperature, None, 0.3)
+        assert np.allclose(p, softmax(logits.astype(np.float64) / temperature), rtol=1e-5, atol=1e-9)
+        _, p_np = orc.sample_from_logits(logits, temperature, None, 0.3)
+        assert np.allclose(p, p_np, rtol=1e-6, atol=1e-9)
+
+
+def test_sampler_index_is_the_inverse_cdf(corc):
+    rng = np.random.default_rng(1)
+    logits = rng.standard_normal(50).astype(np.float32)
+    _, p = corc.sample_from_logits(logits, 1.0, None, 0.0)
+    cdf = np.cumsum(p.astype(np.float64))
+    for u in rng.random(300):
+        if np.abs(cdf - u * cdf[-1]).min() < 1e-5:  # too close to a boundary for f32 vs f64 to agree
+            continue
+        want = int(np.searchsorted(cdf[:-1], u * cdf[-1], side="right"))
+        assert corc.sample_from_logits(logits, 1.0, None, float(u))[0] == want
+        assert orc.sample_from_logits(logits, 1.0, None, float(u))[0] == want
+    assert corc.sample_from_logits(logits, 1.0, None, 0.0)[0] == 0
+    assert corc.sample_from_logits(logits, 1.0, None, 1.0)[0] == 49  # clamped below 1: the last index
+
+
+def test_sampler_top_k(corc):
+    rng = np.random.default_rng(2)
+    logits = rng.standard_normal(256).astype(np.float32)
+    for u in (0.0, 0.37, 0.999):  # top_k = 1 is greedy whatever the draw
+        assert corc.sample_from_logits(logits, 0.8, 1, u)[0] == int(np.argmax(logits)) == corc.greedy_token(logits)
+    _, p = corc.sample_from_logits(logits, 1.0, 5, 0.5)
+    assert (p > 0).sum() == 5 and set(np.nonzero(p)[0]) == set(np.argsort(logits)[-5:])
+    tied = logits.copy()
+    tied[[3, 77]] = np.sort(logits)[-5]  # two more entries equal to the 5th largest: all survive (:43-45)
+    _, p = corc.sample_from_logits(tied, 1.0, 5, 0.5)
+    assert (p > 0).sum() == 7
+    for k in (0, 256, 1000):  # no truncation
+        assert (corc.sample_from_logits(logits, 1.0, k, 0.5)[1] > 0).all()
+
+
+def test_sampler_degenerate_rows_fall_back_to_uniform(corc):
+    row = np.full(8, np.nan, np.float32)
+    idx, p = corc.sample_from_logits(row, 1.0, None, 0.51)
+    assert np.allclose(p, 1 / 8) and idx == 4
+    idx, p = corc.sample_from_logits(np.full(8, -np.inf, np.float32), 1.0, None, 0.26)
+    assert np.allclose(p, 1 / 8) and idx == 2
+
+
+def test_sampler_draw_frequencies_follow_the_distribution(corc):
+    from scipy.stats import chisquare
+
+    logits = np.array([0.0, 1.0, 2.0, -1.0, 0.5], np.float32)
+    _, p = corc.sample_from_logits(logits, 1.0, None, 0.0)
+    us = (np.arange(20000) + 0.5) / 20000  # stratified uniforms: frequencies must match p to 1/n
+    counts = np.bincount([corc.sample_from_logits(logits, 1.0, None, float(u))[0] for u in us], minlength=5)
+    assert np.abs(counts / 20000 - p).max() < 2e-4
+    draws = np.random.default_rng(5).random(5000)
+    counts = np.bincount([orc.sample_from_logits(logits, 1.0, None, float(u))[0] for u in draws], minlength=5)
+    p64 = p.astype(np.float64)
+    assert chisquare(counts, p64 / p64.sum() * 5000).pvalue > 1e-3
