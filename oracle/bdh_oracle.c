@@ -22,7 +22,7 @@
  * tolerance-based, and "bit-exact active sets" means bit-exact against THIS order.
  *
  * Pinning status (what independent check fixes each function) is listed in
- * tests/test_oracle_*.py; functions with no such check are marked "parity
+ * tests/test_oracle.py and tests/test_record.py; functions with no such check are marked "parity
  * unpinned" below.
  *
  *   orc_build_freqs            pinned: closed form + second statement in
@@ -41,9 +41,20 @@
  *                              force against tril(-1)(QQ^T)V in float64, chunk
  *                              consistency, first-token and final-rho closed forms
  *   orc_forward_with_state     reference pins shapes/position only
- *                              (tests/model_paths.rs:33-91); values pinned here by
- *                              decode-vs-prefill consistency and agreement with the
- *                              independent numpy restatement
+ *                              (tests/model_paths.rs:33-91); values pinned here by the
+ *                              trained checkpoint the reference ships
+ *                              (www/assets/model/tiny_shakespeare, ALiBi): 1.16 nats
+ *                              per character on Shakespeare text against 4.23 for a
+ *                              uniform guess, and back to >= 3.5 with the wrong
+ *                              positional scheme or swapped encoders
+ *                              (tests/test_record.py); also decode-vs-prefill
+ *                              consistency and agreement with the independent numpy
+ *                              restatement.  The RoPE and PoPE variants share
+ *                              everything but orc_rotate (pinned above) with it.
+ *   orc_sample_from_logits     pinned: library softmax, float64 inverse CDF, argmax
+ *                              for top_k = 1, draw frequencies (tests/test_oracle.py);
+ *                              the reference's own draw uses thread_rng and cannot be
+ *                              replayed
  */
 #include <math.h>
 #include <stddef.h>
