@@ -179,6 +179,43 @@ int bdh_recurrent_attention(bdh_ctx *ctx, int B, int h, int T, int N, int d, int
   return bdh_launch_state_steps(ctx, p);
 }
 
+int bdh_recurrent_attention_lazy_alibi(bdh_ctx *ctx, int B, int h, int T, int N, int d, const float *x,
+                                       const float *v, int64_t clock, const int32_t *clocks_dev,
+                                       const float *alibi_slopes_host, void *rho, int rho_dtype,
+                                       int32_t *stamps, float *out, uint64_t *active_bitmask,
+                                       int32_t *rows_touched) {
+  int rc = validate_state_args(ctx, B, h, T, N, d, BDH_ALIBI, x, v, nullptr, clock, rho, rho_dtype, out);
+  if (rc != BDH_OK) return rc;
+  if (B == 0 || h == 0 || T == 0) return BDH_OK;
+  if (N > 0 && !stamps) return bdh_fail(ctx, BDH_E_INVAL, "null stamps");
+  if (clock + T > 0x7fffffffLL) return bdh_fail(ctx, BDH_E_INVAL, "clock beyond the 31-bit stamp range");
+  float slopes[64];
+  if (alibi_slopes_host)
+    memcpy(slopes, alibi_slopes_host, sizeof(float) * h);
+  else
+    bdh_default_alibi_slopes(h, slopes);
+  StateStepParams p{B, h, T, N, d, BDH_ALIBI, rho_dtype, x, v, nullptr, clock, clocks_dev, slopes, rho, out,
+                    active_bitmask, rows_touched, stamps};
+  return bdh_launch_state_steps(ctx, p);
+}
+
+int bdh_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, int64_t clock, const int32_t *clocks_dev,
+                          const float *alibi_slopes_host, void *rho, int rho_dtype, int32_t *stamps) {
+  if (!ctx) return BDH_E_INVAL;
+  if (B < 0 || h < 0 || N < 0 || d < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
+  if (h > 64) return bdh_fail(ctx, BDH_E_SHAPE, "n_head %d > 64", h);
+  if (rho_dtype != BDH_F32 && rho_dtype != BDH_BF16) return bdh_fail(ctx, BDH_E_INVAL, "bad rho_dtype");
+  if (clock < 0 || clock > 0x7fffffffLL) return bdh_fail(ctx, BDH_E_INVAL, "clock outside the 31-bit stamp range");
+  if (B == 0 || h == 0 || N == 0) return BDH_OK;
+  if (!rho || !stamps) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  float slopes[64];
+  if (alibi_slopes_host)
+    memcpy(slopes, alibi_slopes_host, sizeof(float) * h);
+  else
+    bdh_default_alibi_slopes(h, slopes);
+  return bdh_launch_alibi_materialize(ctx, B, h, N, d, slopes, clock, clocks_dev, rho, rho_dtype, stamps);
+}
+
 int bdh_state_step(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const float *x,
                    const float *v, const float *freqs, int64_t position,
                    const int32_t *positions_dev, const float *alibi_slopes_host, void *rho,

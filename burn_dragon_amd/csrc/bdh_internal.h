@@ -69,12 +69,16 @@ struct StateStepParams {
   float *out;
   uint64_t *bitmask;
   int32_t *rows_touched;
+  int32_t *stamps = nullptr;  // ALiBi only: [B,h,N] decay stamps of a lazily decayed state, or null
 };
 int bdh_launch_state_steps(bdh_ctx *ctx, const StateStepParams &p);
 
 // Variant used inside the fused model step: the readout is LayerNorm-ed on the fly
 // (src/model/bdh.rs:359) when out_ln != nullptr.
 int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
+// rho <- the up-to-date state, stamps <- clock, for a lazily decayed ALiBi state
+int bdh_launch_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, const float *slopes_host, int64_t clock,
+                                 const int32_t *clocks_dev, void *rho, int rho_dtype, int32_t *stamps);
 
 struct ReluLowrankParams {
   int B, h_in, T, d, h, N;

@@ -102,8 +102,18 @@ int bdh_model_forward(bdh_model *m, const int64_t *tokens, int B, int T, void *r
 int bdh_model_forward_ex(bdh_model *m, const int64_t *tokens, int B, int T, void *rho, int rho_dtype,
                          int64_t position, const int32_t *positions_dev, float *logits, int64_t *next_tokens,
                          float *x_tap) {
+  return bdh_model_forward_lazy(m, tokens, B, T, rho, rho_dtype, nullptr, position, positions_dev, logits,
+                                next_tokens, x_tap);
+}
+
+int bdh_model_forward_lazy(bdh_model *m, const int64_t *tokens, int B, int T, void *rho, int rho_dtype,
+                           int32_t *stamps, int64_t position, const int32_t *positions_dev, float *logits,
+                           int64_t *next_tokens, float *x_tap) {
   if (!m) return BDH_E_INVAL;
   bdh_ctx *ctx = m->ctx;
+  if (stamps && m->cfg.rotary != BDH_ALIBI)
+    return bdh_fail(ctx, BDH_E_INVAL, "decay stamps only apply to an ALiBi model");
+  if (stamps && position + T > 0x7fffffffLL) return bdh_fail(ctx, BDH_E_INVAL, "position beyond the stamp range");
   if (B < 0 || T < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative batch or time");
   if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
   if (rho_dtype != BDH_F32 && rho_dtype != BDH_BF16) return bdh_fail(ctx, BDH_E_INVAL, "bad rho_dtype");
@@ -137,7 +147,8 @@ int bdh_model_forward_ex(bdh_model *m, const int64_t *tokens, int B, int T, void
     // :353-359  recurrent attention (value = cur) and LayerNorm of its output
     StateStepParams ps{B, h, T, N, d, c.rotary, rho_dtype, x_l, cur, m->freqs, position, positions_dev,
                        c.rotary == BDH_ALIBI ? m->slopes : nullptr,
-                       static_cast<char *>(rho) + (size_t)l * rho_layer_bytes, attn, nullptr, nullptr};
+                       static_cast<char *>(rho) + (size_t)l * rho_layer_bytes, attn, nullptr, nullptr,
+                       stamps ? stamps + (size_t)l * B * h * N : nullptr};
     rc = bdh_launch_state_steps_ln(ctx, ps, attn_ln);
     if (rc != BDH_OK) return rc;
     // :361-381  xy = x * relu(LN(attn) . encoder_v - thr)

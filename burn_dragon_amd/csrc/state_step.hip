@@ -63,6 +63,7 @@ struct StepPtrs {
   long v_batch_stride;
   const float *freqs;
   float pos_scalar;             // f32(position + t)
+  long pos_int;                 // position + t as an integer (the clock of a lazily decayed state)
   const int32_t *pos_dev;       // optional per-sequence start positions
   int pos_add;                  // t, added to pos_dev[b]
   float *partial;               // [slices, S, d]
@@ -239,6 +240,154 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
 }
 
 // ------------------------------------------------------------------------------------
+// fast path: ALiBi with a lazily decayed f32 state, D in {256, 512}.  Same shape as the RoPE
+// kernel (one workgroup of WAVES waves owns WAVES*128 neurons of one slice, ballot compaction
+// into an LDS list, U rows in flight per wave), but the unit is a single state row: ALiBi does
+// not rotate, so a neuron's row is touched only when that neuron is active.  The thread that
+// owns a neuron also reads its stamp, turns it into the catch-up factor decay^(clock - stamp)
+// and writes the new stamp clock + 1.
+// ------------------------------------------------------------------------------------
+template <int D, int WAVES, int U>
+__global__ __launch_bounds__(WAVES * 64) void k_step_alibi_lazy_f32(StepPtrs a, float *__restrict__ rho,
+                                                                   int32_t *__restrict__ stamps, HeadScalars decay,
+                                                                   HeadScalars log_decay) {
+  constexpr int VPL = D / 256;
+  constexpr int RPB = WAVES * 128;  // state rows (neurons) per workgroup
+  __shared__ int s_cnt[2][WAVES];
+  __shared__ unsigned short s_idx[RPB];
+  __shared__ float2 s_qs[RPB];  // (activation, catch-up factor)
+  __shared__ float4 s_red[WAVES][D / 4];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slice = blockIdx.x / a.S;
+  const int seg = blockIdx.x - slice * a.S;
+  const int b = slice / a.h, hh = slice - b * a.h;
+  const int p = seg * (RPB / 2) + tid;  // this thread owns neurons 2p and 2p+1
+  const long clock = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
+  const float dec = decay.v[hh], ld = log_decay.v[hh];
+
+  float2 xv = make_float2(0.0f, 0.0f);
+  if (2 * p + 1 < a.N) {
+    xv = reinterpret_cast<const float2 *>(a.x + (long)slice * a.x_slice_stride)[p];
+  } else if (2 * p < a.N) {
+    xv.x = a.x[(long)slice * a.x_slice_stride + 2 * p];
+  }
+  const bool ae = xv.x != 0.0f, ao = xv.y != 0.0f;
+  const unsigned long long me = __ballot(ae), mo = __ballot(ao);
+  if (a.bitmask && lane == 0) {
+    const int w0 = (seg * RPB + wave * 128) >> 6;
+    const int NW = (a.N + 63) >> 6;
+    unsigned long long *bm = a.bitmask + (long)slice * a.bitmask_slice_stride;
+    if (w0 < NW) bm[w0] = spread_bits((unsigned int)me) | (spread_bits((unsigned int)mo) << 1);
+    if (w0 + 1 < NW) bm[w0 + 1] = spread_bits((unsigned int)(me >> 32)) | (spread_bits((unsigned int)(mo >> 32)) << 1);
+  }
+  float se = 1.0f, so = 1.0f;
+  {
+    int32_t *st = stamps + (long)slice * a.N;
+    const int32_t next = (int32_t)min(clock + 1, 0x7fffffffL);
+    if (ae) {
+      const long k = clock - (long)st[2 * p];
+      if (k > 0) se = expf((float)k * ld);
+      st[2 * p] = next;
+    }
+    if (ao) {
+      const long k = clock - (long)st[2 * p + 1];
+      if (k > 0) so = expf((float)k * ld);
+      st[2 * p + 1] = next;
+    }
+  }
+  if (lane == 0) {
+    s_cnt[0][wave] = __popcll(me);
+    s_cnt[1][wave] = __popcll(mo);
+  }
+  __syncthreads();
+  int off_e = 0, off_o = 0, total_e = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const int ce = s_cnt[0][w], co = s_cnt[1][w];
+    if (w < wave) {
+      off_e += ce;
+      off_o += co;
+    }
+    total_e += ce;
+    total += ce + co;
+  }
+  const unsigned long long below = (1ull << lane) - 1ull;
+  if (ae) {
+    const int rank = off_e + __popcll(me & below);
+    s_idx[rank] = (unsigned short)(2 * tid);
+    s_qs[rank] = make_float2(xv.x, se);
+  }
+  if (ao) {
+    const int rank = total_e + off_o + __popcll(mo & below);
+    s_idx[rank] = (unsigned short)(2 * tid + 1);
+    s_qs[rank] = make_float2(xv.y, so);
+  }
+  __syncthreads();
+
+  float4 acc[VPL], vv[VPL];
+  {
+    const float4 *vrow = reinterpret_cast<const float4 *>(a.v + (long)b * a.v_batch_stride);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      vv[j] = vrow[j * 64 + lane];
+    }
+  }
+  float *base = rho + ((long)slice * a.N + (long)seg * RPB) * D;
+  for (int i0 = wave; i0 < total; i0 += WAVES * U) {
+    float4 r[U][VPL];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * WAVES;
+      if (i < total) {
+        const float4 *rp = reinterpret_cast<const float4 *>(base + (long)s_idx[i] * D);
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) r[u][j] = rp[j * 64 + lane];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * WAVES;
+      if (i < total) {
+        const float2 qs = s_qs[i];
+        float4 *wp = reinterpret_cast<float4 *>(base + (long)s_idx[i] * D);
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          float4 e = r[u][j];
+          e.x = e.x * qs.y; e.y = e.y * qs.y; e.z = e.z * qs.y; e.w = e.w * qs.y;  // pending decay
+          acc[j].x = __builtin_fmaf(e.x, qs.x, acc[j].x);  // readout with the old row (src/model/bdh.rs:293-295)
+          acc[j].y = __builtin_fmaf(e.y, qs.x, acc[j].y);
+          acc[j].z = __builtin_fmaf(e.z, qs.x, acc[j].z);
+          acc[j].w = __builtin_fmaf(e.w, qs.x, acc[j].w);
+          const float4 vj = vv[j];
+          float t;
+          t = qs.x * vj.x; e.x = (e.x + t) * dec;  // update (:298), then this token's decay (:299-301)
+          t = qs.x * vj.y; e.y = (e.y + t) * dec;
+          t = qs.x * vj.z; e.z = (e.z + t) * dec;
+          t = qs.x * vj.w; e.w = (e.w + t) * dec;
+          wp[j * 64 + lane] = e;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) s_red[wave][j * 64 + lane] = acc[j];
+  __syncthreads();
+  float *pout = a.partial + (long)blockIdx.x * D;
+  for (int c4 = tid; c4 < D / 4; c4 += WAVES * 64) {
+    float4 sum = s_red[0][c4];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      const float4 t = s_red[w][c4];
+      sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+    }
+    reinterpret_cast<float4 *>(pout)[c4] = sum;
+  }
+  if (tid == 0) a.pair_cnt[blockIdx.x] = total;
+}
+
+// ------------------------------------------------------------------------------------
 // fast path: RoPE, bf16 state (f32 accumulate), D in {256, 512}.  A lane pair's two rows are
 // 4*D contiguous bytes; each lane owns D/256 16-byte pieces (8 bf16) of that chunk.
 // ------------------------------------------------------------------------------------
@@ -402,9 +551,35 @@ __device__ __forceinline__ float rho_load<unsigned short>(const unsigned short *
 __device__ __forceinline__ void rho_store(float *p, float v) { *p = v; }
 __device__ __forceinline__ void rho_store(unsigned short *p, float v) { *p = f32_to_bf16(v); }
 
+// One state row (all d columns) of the generic path: readout with the old row, rank-1 update,
+// optional decay.  `scale` brings a lazily decayed row up to date first (1 otherwise).
+template <typename RhoT>
+__device__ __forceinline__ void generic_row(RhoT *row, int d, int ncol, int lane, float qn, const float *vrow,
+                                            float scale, bool lazy, bool has_decay, float dec, float *acc) {
+#pragma unroll
+  for (int j = 0; j < kGenMaxCols; ++j) {
+    const int c = j * 64 + lane;
+    if (j < ncol && c < d) {
+      float rv = rho_load<RhoT>(row + c);
+      if (lazy) rv = rv * scale;
+      acc[j] = __builtin_fmaf(rv, qn, acc[j]);
+      const float outer = qn * vrow[c];
+      rv = rv + outer;
+      if (has_decay) rv = rv * dec;  // src/model/bdh.rs:299-301
+      rho_store(row + c, rv);
+    }
+  }
+}
+
+// stamps != nullptr (ALiBi only): the state is kept lazily decayed.  Row n of a slice holds the
+// value it had when the sequence had absorbed stamps[n] tokens; its current value is that times
+// decay^(clock - stamps[n]).  Only rows with a non-zero activation are read, brought up to date,
+// updated, decayed once (src/model/bdh.rs:299-301) and stamped clock+1; all other rows are left
+// alone, so the step stays as sparse as the activations.
 template <typename RhoT>
 __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restrict__ rho, int d, int Nq,
-                                                      int rotary, int has_decay, HeadScalars decay) {
+                                                      int rotary, int has_decay, HeadScalars decay,
+                                                      HeadScalars log_decay, int32_t *__restrict__ stamps) {
   __shared__ float s_red[4][64 * kGenMaxCols];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int slice = blockIdx.x / a.S;
@@ -420,42 +595,52 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
 #pragma unroll
   for (int j = 0; j < kGenMaxCols; ++j) acc[j] = 0.0f;
 
-  for (int r = wave; r < kGenRows; r += 4) {
-    const int n = seg * kGenRows + r;
-    if (n >= Nq) break;
-    float qn;
-    bool touch;
-    if (rotary == BDH_ROPE) {
-      const float xn = xs[n], xo = xs[n ^ 1];
-      touch = (xn != 0.0f) || (xo != 0.0f);
-      float s, c;
-      sincosf(rope_phase(pos, a.freqs[n]), &s, &c);
-      const float rot = (n & 1) ? xo : -xo;
-      const float t0 = xn * c, t1 = rot * s;
-      qn = t0 + t1;
-    } else if (rotary == BDH_POPE) {
-      const int m = n < a.N ? n : n - a.N;
-      const float mag = softplus1(xs[m]);
-      const float ph = rope_phase(pos, a.freqs[m]);
-      qn = n < a.N ? mag * cosf(ph) : mag * sinf(ph);
-      touch = true;
-    } else {
-      qn = xs[n];
-      touch = (qn != 0.0f);
-    }
-    if (!touch && !has_decay) continue;
-    RhoT *row = rho + ((long)slice * Nq + n) * d;
-#pragma unroll
-    for (int j = 0; j < kGenMaxCols; ++j) {
-      const int c = j * 64 + lane;
-      if (j < ncol && c < d) {
-        float rv = rho_load<RhoT>(row + c);
-        acc[j] = __builtin_fmaf(rv, qn, acc[j]);
-        const float outer = qn * vrow[c];
-        rv = rv + outer;
-        if (has_decay) rv = rv * dec;  // src/model/bdh.rs:299-301
-        rho_store(row + c, rv);
+  if (rotary == BDH_ALIBI) {
+    // q = x (src/model/attention.rs:332-349: ALiBi does not rotate).  Lane l < 16 fetches the
+    // activation of row wave + 4l of this segment; the ballot lists the rows to visit.
+    const bool lazy = stamps != nullptr;
+    const long clock = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
+    const int n_l = seg * kGenRows + wave + 4 * lane;
+    const bool in_range = lane < kGenRows / 4 && n_l < Nq;
+    const float xl = in_range ? xs[n_l] : 0.0f;
+    unsigned long long m = __ballot(lazy ? (xl != 0.0f) : in_range);
+    int32_t *st = lazy ? stamps + (long)slice * Nq : nullptr;
+    while (m) {
+      const int l = __builtin_ctzll(m);
+      m &= m - 1;
+      const float qn = __shfl(xl, l, 64);
+      const int n = seg * kGenRows + wave + 4 * l;
+      float scale = 1.0f;
+      if (lazy) {
+        const long k = clock - (long)st[n];
+        if (k > 0) scale = expf((float)k * log_decay.v[hh]);
       }
+      generic_row<RhoT>(rho + ((long)slice * Nq + n) * d, d, ncol, lane, qn, vrow, scale, lazy, true, dec, acc);
+      if (lazy && lane == 0) st[n] = (int32_t)min(clock + 1, 0x7fffffffL);
+    }
+  } else {
+    for (int r = wave; r < kGenRows; r += 4) {
+      const int n = seg * kGenRows + r;
+      if (n >= Nq) break;
+      float qn;
+      bool touch;
+      if (rotary == BDH_ROPE) {
+        const float xn = xs[n], xo = xs[n ^ 1];
+        touch = (xn != 0.0f) || (xo != 0.0f);
+        float s, c;
+        sincosf(rope_phase(pos, a.freqs[n]), &s, &c);
+        const float rot = (n & 1) ? xo : -xo;
+        const float t0 = xn * c, t1 = rot * s;
+        qn = t0 + t1;
+      } else {
+        const int m = n < a.N ? n : n - a.N;
+        const float mag = softplus1(xs[m]);
+        const float ph = rope_phase(pos, a.freqs[m]);
+        qn = n < a.N ? mag * cosf(ph) : mag * sinf(ph);
+        touch = true;
+      }
+      if (!touch) continue;
+      generic_row<RhoT>(rho + ((long)slice * Nq + n) * d, d, ncol, lane, qn, vrow, 1.0f, false, false, 1.0f, acc);
     }
   }
 #pragma unroll
@@ -471,15 +656,37 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
   }
 }
 
+// Brings every row of a lazily decayed ALiBi state up to date: row *= decay^(clock - stamp),
+// stamp = clock.  Afterwards rho is the state the reference would hold.
+template <typename RhoT>
+__global__ __launch_bounds__(256) void k_alibi_materialize(RhoT *__restrict__ rho, int32_t *__restrict__ stamps, int h,
+                                                           int N, int d, long total_rows, long clock_scalar,
+                                                           const int32_t *__restrict__ clocks_dev,
+                                                           HeadScalars log_decay) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);  // one wave per state row
+  const int lane = threadIdx.x & 63;
+  if (row >= total_rows) return;
+  const long slice = row / N;
+  const int b = (int)(slice / h), hh = (int)(slice - (long)b * h);
+  const long clock = clocks_dev ? (long)clocks_dev[b] : clock_scalar;
+  const long k = clock - (long)stamps[row];
+  if (k > 0) {
+    const float scale = expf((float)k * log_decay.v[hh]);
+    RhoT *p = rho + row * d;
+    for (int c = lane; c < d; c += 64) rho_store(p + c, rho_load<RhoT>(p + c) * scale);
+  }
+  if (lane == 0) stamps[row] = (int32_t)min(clock, 0x7fffffffL);
+}
+
 // bitmask + touched-row count for the generic path: one workgroup per slice
 __global__ __launch_bounds__(256) void k_bitmask_rows(StepPtrs a, int rotary, int Nq, int *__restrict__ rows,
-                                                      long rows_slice_stride) {
-  __shared__ int s_pairs[4];
+                                                      long rows_slice_stride, int lazy) {
+  __shared__ int s_pairs[4], s_elems[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int slice = blockIdx.x;
   const float *xs = a.x + (long)slice * a.x_slice_stride;
   const int NW = (a.N + 63) >> 6;
-  int pairs = 0;
+  int pairs = 0, elems = 0;
   for (int w = wave; w < NW; w += 4) {
     const int n = w * 64 + lane;
     const float xv = n < a.N ? xs[n] : 0.0f;
@@ -487,12 +694,17 @@ __global__ __launch_bounds__(256) void k_bitmask_rows(StepPtrs a, int rotary, in
     if (a.bitmask && lane == 0) a.bitmask[(long)slice * a.bitmask_slice_stride + w] = m;
     const unsigned long long pm = (m | (m >> 1)) & 0x5555555555555555ull;
     pairs += __popcll(pm);
+    elems += __popcll(m);
   }
-  if (lane == 0) s_pairs[wave] = pairs;
+  if (lane == 0) {
+    s_pairs[wave] = pairs;
+    s_elems[wave] = elems;
+  }
   __syncthreads();
   if (tid == 0 && rows) {
     const int np = s_pairs[0] + s_pairs[1] + s_pairs[2] + s_pairs[3];
-    rows[(long)slice * rows_slice_stride] = rotary == BDH_ROPE ? 2 * np : Nq;
+    const int ne = s_elems[0] + s_elems[1] + s_elems[2] + s_elems[3];
+    rows[(long)slice * rows_slice_stride] = rotary == BDH_ROPE ? 2 * np : (lazy ? ne : Nq);
   }
 }
 
@@ -505,7 +717,7 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
                                                        const int *__restrict__ pair_cnt, int S, int d,
                                                        float *__restrict__ out, long out_slice_stride,
                                                        float *__restrict__ out_ln, int *__restrict__ rows,
-                                                       long rows_slice_stride) {
+                                                       long rows_slice_stride, int rows_per_count) {
   const int tid = threadIdx.x;
   const int slice = blockIdx.x;
   const float *p = partial + (long)slice * S * d;
@@ -527,7 +739,7 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
     int np = 0;
 #pragma unroll 16
     for (int g = 0; g < S; ++g) np += pair_cnt[(long)slice * S + g];
-    rows[(long)slice * rows_slice_stride] = 2 * np;
+    rows[(long)slice * rows_slice_stride] = rows_per_count * np;
   }
   if (!LN) return;
   // LayerNorm over d: mean, biased variance, (x-mean)/sqrt(var+eps)
@@ -564,13 +776,13 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
 }
 
 void launch_finalize(hipStream_t st, int slices, const float *partial, const int *pair_cnt, int S, int d, float *out,
-                     long out_stride, float *out_ln, int *rows, long rows_stride) {
+                     long out_stride, float *out_ln, int *rows, long rows_stride, int rows_per_count = 2) {
   if (out_ln)
     hipLaunchKernelGGL(k_step_finalize<true>, dim3(slices), dim3(256), 0, st, partial, pair_cnt, S, d, out, out_stride,
-                       out_ln, rows, rows_stride);
+                       out_ln, rows, rows_stride, rows_per_count);
   else
     hipLaunchKernelGGL(k_step_finalize<false>, dim3(slices), dim3(256), 0, st, partial, pair_cnt, S, d, out,
-                       out_stride, out_ln, rows, rows_stride);
+                       out_stride, out_ln, rows, rows_stride, rows_per_count);
 }
 
 template <int D, int WAVES, int U, int SPLIT>
@@ -594,7 +806,9 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   const bool split = fast && (ctx->opt_step_split >= 0 ? ctx->opt_step_split == 1
                                                        : (long)slices * (((N / 2) + 255) / 256) < 2L * n_cu);
   const int ppb = split ? 64 : 256;
-  const int S = fast ? ((N / 2) + ppb - 1) / ppb : (Nq + kGenRows - 1) / kGenRows;
+  // lazily decayed ALiBi state, f32, d in {256,512}: row-compaction kernel, 512 neurons per workgroup
+  const bool fast_lazy = p.rotary == BDH_ALIBI && p.stamps && p.rho_dtype == BDH_F32 && (d == 256 || d == 512);
+  const int S = fast ? ((N / 2) + ppb - 1) / ppb : fast_lazy ? (N + 511) / 512 : (Nq + kGenRows - 1) / kGenRows;
   if (N == 0 || d == 0) {
     // nothing to read or update: the readout is an empty sum
     if (d > 0) BDH_HIP_CHECK(ctx, hipMemsetAsync(p.out, 0, sizeof(float) * (size_t)slices * T * d, ctx->stream));
@@ -609,10 +823,16 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   float *partial = static_cast<float *>(ctx->ws);
   int *pair_cnt = reinterpret_cast<int *>(static_cast<char *>(ctx->ws) + partial_bytes);
 
-  HeadScalars decay{};
+  HeadScalars decay{}, log_decay{};
   const int has_decay = p.rotary == BDH_ALIBI;
   if (has_decay)
-    for (int i = 0; i < h; ++i) decay.v[i] = expf(-p.slopes_host[i]);  // src/model/attention.rs:181-186
+    for (int i = 0; i < h; ++i) {
+      decay.v[i] = expf(-p.slopes_host[i]);  // src/model/attention.rs:181-186
+      // k single-precision multiplications by decay are decay^k = exp(k * log(decay)), with the
+      // logarithm of the ROUNDED factor so that the lazy form follows the reference's product
+      log_decay.v[i] = (float)log((double)decay.v[i]);
+    }
+  if (p.stamps && p.rotary != BDH_ALIBI) return bdh_fail(ctx, BDH_E_INVAL, "decay stamps only apply to ALiBi");
 
   const int NW = (N + 63) / 64;
   for (int t = 0; t < T; ++t) {
@@ -623,6 +843,7 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
     a.v_batch_stride = (long)T * d;
     a.freqs = p.freqs;
     a.pos_scalar = (float)(p.position + (int64_t)t);
+    a.pos_int = (long)(p.position + (int64_t)t);
     a.pos_dev = p.positions_dev;
     a.pos_add = t;
     a.partial = partial;
@@ -657,23 +878,53 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
       BDH_LAUNCH_CHECK(ctx, "k_step_rope");
       launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
+    } else if (fast_lazy) {
+      float *rho = static_cast<float *>(p.rho);
+      if (d == 256)
+        hipLaunchKernelGGL((k_step_alibi_lazy_f32<256, 4, 4>), dim3(slices * S), dim3(256), 0, ctx->stream, a, rho,
+                           p.stamps, decay, log_decay);
+      else
+        hipLaunchKernelGGL((k_step_alibi_lazy_f32<512, 4, 4>), dim3(slices * S), dim3(256), 0, ctx->stream, a, rho,
+                           p.stamps, decay, log_decay);
+      BDH_LAUNCH_CHECK(ctx, "k_step_alibi_lazy_f32");
+      launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T, 1);
+      BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
     } else {
       if (p.rho_dtype == BDH_F32)
         hipLaunchKernelGGL(k_step_generic<float>, dim3(slices * S), dim3(256), 0, ctx->stream, a,
-                           static_cast<float *>(p.rho), d, Nq, p.rotary, has_decay, decay);
+                           static_cast<float *>(p.rho), d, Nq, p.rotary, has_decay, decay, log_decay, p.stamps);
       else
         hipLaunchKernelGGL(k_step_generic<unsigned short>, dim3(slices * S), dim3(256), 0, ctx->stream, a,
-                           static_cast<unsigned short *>(p.rho), d, Nq, p.rotary, has_decay, decay);
+                           static_cast<unsigned short *>(p.rho), d, Nq, p.rotary, has_decay, decay, log_decay,
+                           p.stamps);
       BDH_LAUNCH_CHECK(ctx, "k_step_generic");
       launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
       if (a.bitmask || rows_t) {
         hipLaunchKernelGGL(k_bitmask_rows, dim3(slices), dim3(256), 0, ctx->stream, a, p.rotary, Nq, rows_t,
-                           (long)T);
+                           (long)T, p.stamps ? 1 : 0);
         BDH_LAUNCH_CHECK(ctx, "k_bitmask_rows");
       }
     }
   }
+  return BDH_OK;
+}
+
+int bdh_launch_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, const float *slopes_host, int64_t clock,
+                                 const int32_t *clocks_dev, void *rho, int rho_dtype, int32_t *stamps) {
+  HeadScalars log_decay{};
+  for (int i = 0; i < h; ++i) log_decay.v[i] = (float)log((double)expf(-slopes_host[i]));
+  const long rows = (long)B * h * N;
+  if (rows == 0 || d == 0) return BDH_OK;
+  const long blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "state has too many rows");
+  if (rho_dtype == BDH_F32)
+    hipLaunchKernelGGL(k_alibi_materialize<float>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                       static_cast<float *>(rho), stamps, h, N, d, rows, (long)clock, clocks_dev, log_decay);
+  else
+    hipLaunchKernelGGL(k_alibi_materialize<unsigned short>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                       static_cast<unsigned short *>(rho), stamps, h, N, d, rows, (long)clock, clocks_dev, log_decay);
+  BDH_LAUNCH_CHECK(ctx, "k_alibi_materialize");
   return BDH_OK;
 }
 

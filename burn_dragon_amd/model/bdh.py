@@ -22,10 +22,14 @@ UINT63_MAX = (1 << 63) - 1
 
 class BDH:
     def __init__(self, config: BDHConfig, device="cuda:0", seed: Optional[int] = None, weights: Optional[dict] = None,
-                 rho_dtype: int = ffi.F32):
+                 rho_dtype: int = ffi.F32, alibi_lazy: bool = False):
         """BDH::new (src/model/bdh.rs:37-84).  `weights` (numpy/torch, the reference's shapes) or a
-        seed for Normal(0, 0.02) projections and a Normal(0, 1) embedding."""
+        seed for Normal(0, 0.02) projections and a Normal(0, 1) embedding.  alibi_lazy (ALiBi models
+        only): keep the state lazily decayed, so a step touches only the rows of the active neurons
+        instead of multiplying the whole state by exp(-slope) (src/model/bdh.rs:299-301);
+        materialize_state() turns it back into the reference's state."""
         self.config = config
+        self.alibi_lazy = bool(alibi_lazy)
         self.device = torch.device(device)
         self.n_layer, self.n_embd, self.n_head = config.n_layer, config.n_embd, config.n_head
         self.vocab_size = config.vocab_size
@@ -61,9 +65,12 @@ class BDH:
                                                      ctypes.byref(handle)))
         self.handle = handle
         self.latent_q = 2 * N if rot == RotaryEmbedding.POPE else N
+        if self.alibi_lazy and rot != RotaryEmbedding.ALIBI:
+            raise ValueError("alibi_lazy needs rotary_embedding = alibi")
+        self._slopes = slopes
 
     @classmethod
-    def from_checkpoint_dir(cls, directory: str, device="cuda:0", rho_dtype: int = ffi.F32):
+    def from_checkpoint_dir(cls, directory: str, device="cuda:0", rho_dtype: int = ffi.F32, alibi_lazy: bool = False):
         """A trained model from a directory holding the reference's model.bin (Burn BinFileRecorder
         record), config.json and optionally vocab.json — the loading steps of src/bin/infer.rs:170-186.
         Returns (model, tokenizer or None, block_size)."""
@@ -72,7 +79,8 @@ class BDH:
 
         config, weights, vocab_json, block_size = load_checkpoint_dir(directory)
         tokenizer = CharVocab.from_json_str(vocab_json) if vocab_json is not None else None
-        return cls(config, device, weights=weights, rho_dtype=rho_dtype), tokenizer, block_size
+        model = cls(config, device, weights=weights, rho_dtype=rho_dtype, alibi_lazy=alibi_lazy)
+        return model, tokenizer, block_size
 
     def __del__(self):
         try:
@@ -94,7 +102,22 @@ class BDH:
             state.storage = torch.zeros(shape, device=self.device, dtype=dt)
             for i, layer in enumerate(state.layers):
                 layer.rho = state.storage[i]
+            state.stamps = None
+        if self.alibi_lazy and state.stamps is None:
+            # a state that arrives without stamps is up to date as of its position
+            state.stamps = torch.full(shape[:-1], min(state.position, 0x7FFFFFFF), device=self.device,
+                                      dtype=torch.int32)
         return state.storage
+
+    def materialize_state(self, state: ModelState) -> None:
+        """Applies the pending decay of a lazily decayed ALiBi state: afterwards state.storage is the
+        state the reference holds after state.position tokens.  No-op for an eager state."""
+        if state.storage is None or state.stamps is None:
+            return
+        from ..recurrent import alibi_materialize
+
+        # layers are folded into the batch: the head index, which selects the slope, is unaffected
+        alibi_materialize(state.storage, state.stamps, state.position, self._slopes, None, self.ctx)
 
     def forward_with_state(self, tokens: torch.Tensor, state: ModelState, want_next: bool = False,
                            x_tap: Optional[torch.Tensor] = None):
@@ -106,9 +129,9 @@ class BDH:
         rho = self._ensure_state(state, B)
         logits = torch.empty((B, T, self.vocab_size), device=self.device, dtype=torch.float32)
         nxt = torch.empty((B,), device=self.device, dtype=torch.int64) if want_next else None
-        self.ctx.check(self.ctx.lib.bdh_model_forward(self.handle, tokens.data_ptr(), B, T, rho.data_ptr(),
-                                                      self.rho_dtype, state.position, logits.data_ptr(),
-                                                      ffi.ptr(nxt), ffi.ptr(x_tap)))
+        self.ctx.check(self.ctx.lib.bdh_model_forward_lazy(self.handle, tokens.data_ptr(), B, T, rho.data_ptr(),
+                                                           self.rho_dtype, ffi.ptr(state.stamps), state.position,
+                                                           None, logits.data_ptr(), ffi.ptr(nxt), ffi.ptr(x_tap)))
         state.position = min(state.position + T, UINT63_MAX)  # saturating_add, :445
         return (logits, nxt) if want_next else logits
 
@@ -153,13 +176,15 @@ class DecodeGraph:
         ctx, lib = model.ctx, model.ctx.lib
 
         def step():
-            ctx.check(lib.bdh_model_forward_ex(model.handle, self.tokens.data_ptr(), B, 1, state.storage.data_ptr(),
-                                               model.rho_dtype, 0, self.positions.data_ptr(), self.logits.data_ptr(),
-                                               self.tokens.data_ptr(), None))
+            ctx.check(lib.bdh_model_forward_lazy(model.handle, self.tokens.data_ptr(), B, 1,
+                                                 state.storage.data_ptr(), model.rho_dtype, ffi.ptr(state.stamps), 0,
+                                                 self.positions.data_ptr(), self.logits.data_ptr(),
+                                                 self.tokens.data_ptr(), None))
             ctx.check(lib.bdh_advance_positions(ctx.handle, self.positions.data_ptr(), B, 1))
 
         # one eager step on a side stream sizes every scratch buffer (no allocation may happen under capture)
-        keep = (self.tokens.clone(), self.positions.clone(), state.storage.clone())
+        keep = (self.tokens.clone(), self.positions.clone(), state.storage.clone(),
+                None if state.stamps is None else state.stamps.clone())
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(side):
@@ -167,6 +192,8 @@ class DecodeGraph:
             step()
         side.synchronize()
         self.tokens.copy_(keep[0]); self.positions.copy_(keep[1]); state.storage.copy_(keep[2])
+        if keep[3] is not None:
+            state.stamps.copy_(keep[3])
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph, stream=side):

@@ -18,6 +18,9 @@ class ModelState:
     position: int = 0
     # all layers share one allocation [L,B,h,Nq,d]; layers[i].rho are views into it
     storage: Optional[torch.Tensor] = None
+    # ALiBi with lazy decay only: [L,B,h,N] int32, the token count at which each state row was last brought
+    # up to date (see BDH(alibi_lazy=True)); None for an eagerly decayed state
+    stamps: Optional[torch.Tensor] = None
 
     @classmethod
     def new(cls, num_layers: int) -> "ModelState":
@@ -27,6 +30,7 @@ class ModelState:
         for layer in self.layers:
             layer.rho = None
         self.storage = None
+        self.stamps = None
         self.position = 0
 
     def len(self) -> int:

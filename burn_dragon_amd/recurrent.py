@@ -44,6 +44,53 @@ def recurrent_attention(query: torch.Tensor, value: torch.Tensor, rho: torch.Ten
     return res[0] if len(res) == 1 else tuple(res)
 
 
+def recurrent_attention_lazy_alibi(query: torch.Tensor, value: torch.Tensor, rho: torch.Tensor,
+                                   stamps: torch.Tensor, clock: int, alibi_slopes=None,
+                                   clocks: Optional[torch.Tensor] = None, want_bitmask: bool = False,
+                                   want_rows: bool = False, ctx: Optional[ffi.Context] = None):
+    """BDH::recurrent_attention for ALiBi (src/model/bdh.rs:258-307 with the decay of :299-301) on a
+    state kept lazily decayed: rho [B,h,N,d] and stamps [B,h,N] int32 are updated in place, only the
+    rows with a non-zero activation are touched.  `clock` = tokens absorbed before this call."""
+    ctx = ctx or ffi.default_context(query.device.index or 0)
+    B, h, T, N = query.shape
+    d = value.shape[-1]
+    assert query.dtype == torch.float32 and query.is_contiguous()
+    value = value.reshape(B, T, d)
+    assert value.dtype == torch.float32 and value.is_contiguous()
+    assert rho.is_contiguous() and tuple(rho.shape) == (B, h, N, d), "rho must be [B,h,N,d]"
+    assert stamps.dtype == torch.int32 and stamps.is_contiguous() and tuple(stamps.shape) == (B, h, N)
+    dt = {torch.float32: ffi.F32, torch.bfloat16: ffi.BF16}[rho.dtype]
+    out = torch.empty((B, h, T, d), device=query.device, dtype=torch.float32)
+    bm = torch.zeros((B, h, T, (N + 63) // 64), device=query.device, dtype=torch.int64) if want_bitmask else None
+    rows = torch.zeros((B, h, T), device=query.device, dtype=torch.int32) if want_rows else None
+    slopes = None if alibi_slopes is None else np.ascontiguousarray(alibi_slopes, np.float32)
+    ctx.check(ctx.lib.bdh_recurrent_attention_lazy_alibi(ctx.handle, B, h, T, N, d, ffi.ptr(query), ffi.ptr(value),
+                                                         int(clock), ffi.ptr(clocks), ffi.ptr(slopes), ffi.ptr(rho), dt,
+                                                         ffi.ptr(stamps), ffi.ptr(out), ffi.ptr(bm), ffi.ptr(rows)))
+    res = [out]
+    if want_bitmask:
+        res.append(bm)
+    if want_rows:
+        res.append(rows)
+    return res[0] if len(res) == 1 else tuple(res)
+
+
+def alibi_materialize(rho: torch.Tensor, stamps: torch.Tensor, clock: int, alibi_slopes=None,
+                      clocks: Optional[torch.Tensor] = None, ctx: Optional[ffi.Context] = None) -> None:
+    """Brings a lazily decayed ALiBi state up to date in place (rho [..., B,h,N,d] with stamps [..., B,h,N];
+    leading dimensions, e.g. layers, are folded into the batch): afterwards rho is what the reference holds."""
+    ctx = ctx or ffi.default_context(rho.device.index or 0)
+    assert rho.is_contiguous() and stamps.is_contiguous() and stamps.dtype == torch.int32
+    h, N, d = rho.shape[-3:]
+    B = rho.numel() // (h * N * d) if rho.numel() else 0
+    assert stamps.numel() == B * h * N
+    assert clocks is None or B == rho.shape[-4], "per-sequence clocks need a plain [B,h,N,d] state"
+    dt = {torch.float32: ffi.F32, torch.bfloat16: ffi.BF16}[rho.dtype]
+    slopes = None if alibi_slopes is None else np.ascontiguousarray(alibi_slopes, np.float32)
+    ctx.check(ctx.lib.bdh_alibi_materialize(ctx.handle, B, h, N, d, int(clock), ffi.ptr(clocks), ffi.ptr(slopes),
+                                            ffi.ptr(rho), dt, ffi.ptr(stamps)))
+
+
 def layer_norm(x: torch.Tensor, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
     """BDH::layer_norm (src/model/bdh.rs:86-89)."""
     ctx = ctx or ffi.default_context(x.device.index or 0)

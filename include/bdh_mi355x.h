@@ -241,6 +241,35 @@ int bdh_model_forward_ex(bdh_model *model, const int64_t *tokens, int B, int T, 
  * `state.position += T` (src/model/bdh.rs:445). */
 int bdh_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta);
 
+/* ALiBi state kept LAZILY decayed.  The reference multiplies the whole state by exp(-slope_h) after
+ * every token (src/model/bdh.rs:299-301), which makes every ALiBi step a dense pass over rho.  Here row n
+ * of a slice stores the value it had when the sequence had absorbed stamps[b,h,n] tokens; its current
+ * value is that times decay_h^(clock - stamp).  A step reads, brings up to date, updates, decays once
+ * and re-stamps only the rows whose activation is non-zero, so its traffic follows the sparsity of x.
+ * `clock` (or clocks_dev[b], int32 per sequence) = tokens the state has absorbed before this call =
+ * ModelState::position.  A zero state with zero stamps is a valid fresh state.  Semantics otherwise as
+ * bdh_recurrent_attention with rotary = BDH_ALIBI (q = x, no rotation); rows_touched counts the active
+ * rows.  Values agree with the eager decay to rounding (decay^k is evaluated as exp(k*log(decay))). */
+int bdh_recurrent_attention_lazy_alibi(bdh_ctx *ctx, int B, int h, int T, int N, int d, const float *x,
+                                       const float *v, int64_t clock, const int32_t *clocks_dev,
+                                       const float *alibi_slopes_host, void *rho, int rho_dtype,
+                                       int32_t *stamps, float *out, uint64_t *active_bitmask,
+                                       int32_t *rows_touched);
+
+/* Brings a lazily decayed state up to date: every row *= decay_h^(clock - stamp), stamps = clock.
+ * Afterwards rho [B,h,N,d] is the state the reference holds after `clock` tokens and can be handed to
+ * the eager entry points (or exported). */
+int bdh_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, int64_t clock,
+                          const int32_t *clocks_dev, const float *alibi_slopes_host, void *rho,
+                          int rho_dtype, int32_t *stamps);
+
+/* bdh_model_forward_ex for an ALiBi model whose state is kept lazily decayed: stamps [L,B,h,N] int32
+ * travels with rho (NULL = eager decay, identical to bdh_model_forward_ex). */
+int bdh_model_forward_lazy(bdh_model *model, const int64_t *tokens, int B, int T, void *rho,
+                           int rho_dtype, int32_t *stamps, int64_t position,
+                           const int32_t *positions_dev, float *logits, int64_t *next_tokens,
+                           float *x_tap);
+
 /* Draws the next token of every sequence on the device.  Replaces the temperature division of
  * sample_next_token (src/generation.rs:117) and sample_from_logits_values (src/generation.rs:26-72),
  * which copy the logits to the host for every token: values = logits / temperature; with

@@ -164,3 +164,40 @@ def test_sampled_token_frequencies_follow_the_softmax(trained):
     from scipy.stats import chisquare
 
     assert chisquare(counts, p * 20000).pvalue > 1e-3
+
+
+def test_trained_checkpoint_with_lazily_decayed_state(trained, corc):
+    """The ALiBi checkpoint with the state kept lazily decayed: same logits as the oracle's eager decay
+    for a prompt and the following greedy steps (eager launches and a replayed HIP graph), and the
+    materialised state equals the oracle's."""
+    import burn_dragon_amd as bda
+
+    _, tok, _, shape, w = trained
+    model, _, _ = bda.BDH.from_checkpoint_dir(CKPT, DEV, alibi_lazy=True)
+    ids = np.array([tok.encode(TEXT[:90])])
+    state = model.init_state()
+    logits, nxt = model.forward_with_state(torch.from_numpy(ids), state, want_next=True)
+    assert state.stamps is not None and tuple(state.stamps.shape) == (4, 1, 4, 128)
+    rho_ref = np.zeros((4, 1, 4, 128, 128), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, ids, rho_ref, 0, sparse_state=False)
+    assert rel_err(logits.cpu().numpy(), logits_ref) < 1e-3
+    graph = None
+    for step in range(12):
+        tok_ref = corc.greedy_token(logits_ref[0, -1])
+        if step == 6:
+            graph = model.capture_decode_step(state, torch.tensor([tok_ref]))
+        if graph is None:
+            logits, nxt = model.forward_with_state(torch.tensor([[tok_ref]]), state, want_next=True)
+        else:
+            graph.tokens.fill_(tok_ref)
+            graph.replay()
+            logits = graph.logits
+        logits_ref, pos, _, _ = corc.forward_with_state(shape, w, np.array([[tok_ref]]), rho_ref, pos, sparse_state=False)
+        assert rel_err(logits.cpu().numpy(), logits_ref) < 1e-3, step
+    assert state.position == pos
+    lazy_rows = float((state.stamps < state.position).float().mean())
+    assert lazy_rows > 0.3  # most rows were NOT touched by the last token: that is the saving
+    model.materialize_state(state)
+    torch.cuda.synchronize()
+    assert (state.stamps == state.position).all()
+    assert rel_err(state.storage.cpu().numpy(), rho_ref) < 1e-3

@@ -281,3 +281,53 @@ def test_config5_shapes_max_relative_error(gpu, corc, dtype, tol, density):
     assert e_out < tol and e_rho < tol
     assert np.array_equal(rows, orc.pair_closed_rows(x))
     assert np.array_equal(bm, orc.active_bitmask(x))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
+@pytest.mark.parametrize("N,d,density", [(128, 128, 0.35), (1024, 256, 0.05), (200, 48, 0.5), (512, 512, 0.0),
+                                         (651, 256, 0.3), (1536, 512, 0.1)])
+def test_lazy_alibi_decay_matches_the_eager_reference_semantics(gpu, corc, dtype, tol, N, d, density):
+    """ALiBi state kept lazily decayed (only active rows touched, decay applied when a row is next
+    used) against the oracle's eager `rho *= exp(-slope)` after every token (src/model/bdh.rs:299-301):
+    every readout along the way, and the state after bdh_alibi_materialize."""
+    _, recurrent_attention = gpu
+    from burn_dragon_amd.recurrent import alibi_materialize, recurrent_attention_lazy_alibi
+
+    B, h, T = 2, 4, 9
+    x, v, rho0 = make_inputs(int(1000 * density) + d, B, h, T, N, d, density, rho_scale=0.05)
+    if dtype == torch.bfloat16:
+        rho0 = torch.from_numpy(rho0).to(torch.bfloat16).float().numpy()
+    slopes = corc.default_alibi_slopes(h)
+    clock0 = 37  # the state arrives up to date as of 37 tokens
+    dev = "cuda:0"
+    rho = torch.from_numpy(rho0).to(dev).to(dtype).contiguous()
+    stamps = torch.full((B, h, N), clock0, device=dev, dtype=torch.int32)
+    xt, vt = torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev)
+    # first five tokens in one call, the rest one by one with per-sequence clocks on the device
+    out_a, bm, rows = recurrent_attention_lazy_alibi(xt[:, :, :5].contiguous(), vt[:, :5].contiguous(), rho, stamps,
+                                                     clock0, None, None, want_bitmask=True, want_rows=True)
+    outs = [out_a]
+    clocks = torch.full((B,), clock0 + 5, device=dev, dtype=torch.int32)
+    for t in range(5, T):
+        outs.append(recurrent_attention_lazy_alibi(xt[:, :, t:t + 1].contiguous(), vt[:, t:t + 1].contiguous(), rho,
+                                                   stamps, 0, None, clocks))
+        clocks += 1
+    untouched = torch.from_numpy(~(x != 0).any(axis=2)).to(dev)  # rows no token activated
+    assert torch.equal(rho[untouched].float(), torch.from_numpy(rho0).to(dev)[untouched])  # never read or written
+    assert (stamps[untouched] == clock0).all()
+    alibi_materialize(rho, stamps, clock0 + T)
+    torch.cuda.synchronize()
+    assert (stamps == clock0 + T).all()
+    out = torch.cat(outs, 2).cpu().numpy()
+    out_ref, rho_ref = corc.recurrent_attention(x, v, rho0, decay=corc.alibi_decay(slopes))
+    assert rel_err(out, out_ref) < tol
+    assert rel_err(rho.float().cpu().numpy(), rho_ref) < tol
+    assert np.array_equal(rows.cpu().numpy(), (x[:, :, :5] != 0).sum(-1))
+    assert np.array_equal(bm.cpu().numpy().view(np.uint64),
+                          orc.active_bitmask(np.pad(x[:, :, :5], ((0, 0), (0, 0), (0, 0), (0, (-N) % 64)))))
+    # the eager entry point on the same inputs gives the same values to rounding
+    rho_e = torch.from_numpy(rho0).to(dev).to(dtype).contiguous()
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    out_e = recurrent_attention(xt, vt, rho_e, torch.zeros(N, device=dev), 0, RotaryEmbedding.ALIBI)
+    assert rel_err(out, out_e.cpu().numpy()) < tol and rel_err(rho.float().cpu().numpy(), rho_e.float().cpu().numpy()) < tol
