@@ -359,7 +359,7 @@ def main():
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain copy of
             # known size (profiles/state_step_config2_f32_pmc_traffic.md); measured for the default workload only
             "traffic": 216.06e6 if default_workload else None,
-            "kernel": "k_step_rope_f32 (+ k_step_finalize); duration = HIP-event time of the timed region / steps",
+            "kernel": f"k_step_rope_{args.rho_dtype} (+ k_step_finalize); duration = HIP-event time of the timed region / steps",
             "launch_us": kernel_us,
         },
     }

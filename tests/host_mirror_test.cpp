@@ -3,12 +3,16 @@
 //   tests/model_paths.rs:66-91        inference_paths_run_across_configs
 //   tests/fused_kernel_tests.rs:35-68 relu_lowrank_fused_matches_reference
 //   tests/fused_kernel_tests.rs:70-120 fused_attention_matches_reference_when_alibi_disabled
+//   src/tokenizer/byte.rs:104-126, char_vocab.rs:281-314  the tokenizer tests
+// and, with the trained checkpoint the reference ships (copied as data to tests/golden/tiny_shakespeare),
+// the record reader, the char tokenizer and the generation loop (argv[1] = that directory).
 // Built by __graft_entry__.build(); run by tests/test_gpu_host_cpp.py.
 #include <cmath>
 #include <cstdio>
 #include <random>
 
 #include "../burn_dragon_amd/host/bdh_host.hpp"
+#include "../burn_dragon_amd/host/bdh_host_io.hpp"
 
 extern "C" {  // oracle/bdh_oracle.c (the checker; never linked into the library)
 typedef struct {
@@ -24,6 +28,8 @@ void orc_relu_lowrank(const float *in, int B, int hin, int T, int d, const float
 void orc_fused_state_aligned(const float *query, const float *value, const float *freqs, const float *slopes, int B, int h,
                              int T, int N, int dv, int block_size, const int32_t *pairs, int n_pairs, int rotary, float *out);
 void orc_build_freqs(int latent, float theta, int rotary, float *out);
+int orc_greedy_token(const float *logits, int V);
+int orc_sample_from_logits(const float *logits, int V, float temperature, int top_k, float u, float *probs_out);
 }
 
 using namespace bdh;
@@ -183,10 +189,137 @@ static void config_and_state_semantics() {
   EXPECT(d2.is_active(2, 1) && !d2.is_active(1, 2) && d2.iter_cols(7, 3).size() == 3);
 }
 
-int main() {
+static void tokenizer_semantics() {
+  using namespace tokenizer;
+  ByteTokenizer t(true);
+  auto enc = t.encode("hello", true, true);
+  EXPECT(enc.front() == *t.bos_id() && enc.back() == *t.eos_id() && t.len() == 259);
+  EXPECT(t.decode(enc) == "hello");
+  auto ids = t.encode("abc", false, false);
+  ids.push_back(*t.eos_id());
+  ids.push_back('d');
+  EXPECT(t.decode(ids) == "abc");
+  CharVocab v = CharVocab::fit({"hello", "world"}, true);
+  EXPECT(v.len() >= 4);
+  auto e2 = v.encode("hello", true, true);
+  EXPECT(e2.front() == *v.bos_id() && e2.back() == *v.eos_id() && v.decode(e2) == "hello");
+  CharVocab small = CharVocab::fit({"ab"}, true);
+  auto t2 = small.encode("ac", false, false);
+  EXPECT(t2.size() == 2 && t2[1] == *small.unk_id() && small.decode(t2) == "a?");
+  bool threw = false;
+  try {
+    (void)CharVocab::fit({"ab"}, false).encode("c", false, false);
+  } catch (const std::out_of_range &) {
+    threw = true;
+  }
+  EXPECT(threw);
+  CharVocab u = CharVocab::from_json_str("{\"chars\": [\"\\u0000\", \"\\u0001\", \"\\u0002\", \"\\u0003\", \"\u00e9\", \"\\n\", \"x\"], "
+                                         "\"bos\": 1, \"eos\": 2, \"pad\": 0, \"unk\": 3}");
+  EXPECT(u.len() == 7 && u.encode("x\u00e9\n", false, false) == (std::vector<uint32_t>{6, 4, 5}));
+  EXPECT(u.decode({1, 6, 4, 5, 2, 6}) == "x\u00e9\n");
+}
+
+static const char *kText =
+    "First Citizen:\nBefore we proceed any further, hear me speak.\n\nAll:\nSpeak, speak.\n\n"
+    "First Citizen:\nYou are all resolved rather to die than to famish?\n\nAll:\nResolved. resolved.\n";
+
+static void trained_checkpoint(const Context &ctx, const std::string &dir) {
+  using namespace tokenizer;
+  record::Loaded rec = record::load_record(dir + "/model.bin");
+  EXPECT(rec.meta.version == "0.19.1" && rec.meta.settings == "FullPrecisionSettings");
+  EXPECT(rec.vocab_size == 69 && rec.n_embd == 128 && rec.n_head == 4 && rec.latent_per_head == 128 &&
+         rec.mlp_internal_dim_multiplier == 4);
+  CharVocab tok = CharVocab::load(dir + "/vocab.json");
+  EXPECT(tok.len() == 69 && *tok.unk_id() == 3);
+  ModelOverrides o;  // config.json of the checkpoint
+  o.n_layer = 4;
+  o.n_embd = 128;
+  o.n_head = 4;
+  o.mlp_internal_dim_multiplier = 4;
+  o.fused_kernels = true;
+  o.rotary_embedding = RotaryEmbedding::Alibi;
+  BDHConfig config = build_model_config(o, 512);
+  config.vocab_size = tok.len();
+  BDH model(ctx, config, rec.weights);
+  const auto ids32 = tok.encode(kText, false, false);
+  EXPECT(tok.decode(ids32) == kText);
+  const std::vector<int64_t> ids(ids32.begin(), ids32.end());
+  ModelState state = model.init_state();
+  const std::vector<float> logits = model.forward_with_state(ids, 1, ids.size(), state).to_host();
+  const size_t V = 69, T = ids.size();
+  std::vector<float> rho(4 * 1 * 4 * 128 * 128, 0.0f), ref(T * V);
+  orc_model m{4, 128, 4, 128, 69, (int)RotaryEmbedding::Alibi, 65536.0f, 0.0f, nullptr, rec.weights.embed.data(),
+              rec.weights.encoder.data(), rec.weights.encoder_v.data(), rec.weights.decoder.data(), rec.weights.lm_head.data()};
+  int64_t pos = 0;
+  EXPECT(orc_forward_with_state(&m, ids.data(), 1, (int)T, rho.data(), &pos, ref.data(), nullptr, nullptr, 0) == 0);
+  EXPECT(rel_err(logits, ref) < 1e-3);
+  double loss = 0;  // mean next-character negative log likelihood; a uniform guess scores ln 69 = 4.23
+  for (size_t t = 0; t + 1 < T; ++t) {
+    double mx = -1e30, z = 0;
+    for (size_t c = 0; c < V; ++c) mx = std::max(mx, (double)logits[t * V + c]);
+    for (size_t c = 0; c < V; ++c) z += std::exp(logits[t * V + c] - mx);
+    loss -= logits[t * V + ids[t + 1]] - mx - std::log(z);
+  }
+  loss /= (double)(T - 1);
+  std::printf("  trained checkpoint: logits rel err %.2e, loss %.3f nats/char\n", rel_err(logits, ref), loss);
+  EXPECT(loss < 1.35);
+
+  // greedy generation (top_k = 1) follows the oracle token by token
+  generation::GenerationSettings gs;
+  gs.max_new_tokens = 32;
+  gs.top_k = 1;
+  std::mt19937 rng(5);
+  const auto p32 = tok.encode("First Citizen:\n", false, false);
+  const std::vector<int64_t> prompt(p32.begin(), p32.end());
+  const auto all = generation::generate_tokens(ctx, model, prompt, gs, rng);
+  EXPECT(all.size() == prompt.size() + 32);
+  std::fill(rho.begin(), rho.end(), 0.0f);
+  pos = 0;
+  std::vector<float> lg(prompt.size() * V);
+  orc_forward_with_state(&m, prompt.data(), 1, (int)prompt.size(), rho.data(), &pos, lg.data(), nullptr, nullptr, 0);
+  std::vector<float> last(lg.end() - V, lg.end());
+  for (size_t i = 0; i < 32 && prompt.size() + i < all.size(); ++i) {
+    const int best = orc_greedy_token(last.data(), (int)V);
+    const int64_t got = all[prompt.size() + i];
+    if (got != best) {
+      std::vector<float> sorted(last);
+      std::sort(sorted.begin(), sorted.end());
+      EXPECT(sorted[V - 1] - sorted[V - 2] < 1e-3f * std::fabs(sorted[V - 1]));
+    }
+    orc_forward_with_state(&m, &got, 1, 1, rho.data(), &pos, last.data(), nullptr, nullptr, 0);
+  }
+  std::vector<uint32_t> out32(all.begin(), all.end());
+  std::printf("  greedy: %s\n", tok.decode(out32).c_str());
+
+  // sampled text is reproducible from the seed and the on-device draw agrees with the oracle's
+  generation::GenerationConfig gc;
+  gc.prompt = "ROMEO:";
+  gc.max_tokens = 24;
+  gc.temperature = 0.8f;
+  gc.top_k = 20;
+  gc.context_strategy = generation::ContextStrategy::sliding(0);
+  std::mt19937 r1(11), r2(11);
+  const std::string a = generation::generate_text(ctx, model, tok, 512, gc, r1);
+  const std::string b = generation::generate_text(ctx, model, tok, 512, gc, r2);
+  EXPECT(a == b && a.rfind("ROMEO:", 0) == 0 && a.size() <= 6 + 24);
+  Tensor row = Tensor::from_host(last, {1, 1, V});
+  int agree = 0;
+  const float us[5] = {0.03f, 0.31f, 0.55f, 0.77f, 0.97f};
+  for (float u : us)
+    agree += generation::sample_from_logits(ctx, row.data(), V, 0.8f, 20, u) ==
+             orc_sample_from_logits(last.data(), (int)V, 0.8f, 20, u, nullptr);
+  EXPECT(agree >= 4);  // a draw within rounding of a CDF boundary may differ
+}
+
+int main(int argc, char **argv) {
   try {
     Context ctx(0);
     config_and_state_semantics();
+    tokenizer_semantics();
+    if (argc > 1) {
+      std::printf("trained_checkpoint\n");
+      trained_checkpoint(ctx, argv[1]);
+    }
     std::printf("inference_paths_run_across_configs\n");
     inference_paths_run_across_configs(ctx);
     std::printf("relu_lowrank_fused_matches_reference\n");

@@ -16,7 +16,7 @@ def test_cpp_host_mirror():
     env = dict(os.environ)
     env["LD_LIBRARY_PATH"] = os.pathsep.join([os.path.join(ROOT, "burn_dragon_amd"), os.path.join(ROOT, "oracle"),
                                               "/opt/rocm/lib", env.get("LD_LIBRARY_PATH", "")])
-    proc = subprocess.run([BIN], capture_output=True, text=True, timeout=120, env=env)
+    proc = subprocess.run([BIN, os.path.join(ROOT, "tests", "golden", "tiny_shakespeare")], capture_output=True, text=True, timeout=120, env=env)
     print(proc.stdout, proc.stderr)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert proc.stdout.strip().endswith("OK")
