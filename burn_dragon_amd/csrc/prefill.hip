@@ -18,6 +18,8 @@
 // k-major (Q [T,N] with the reduction over T): that tile is also copied as is, [k][m], and the
 // fragments are read with the transposing LDS load of gfx950 (ds_read_b64_tr_b16); a 64-byte
 // column swizzle on every other group of eight k rows keeps the two half-waves on different banks.
+#include <atomic>
+
 #include "bdh_internal.h"
 
 namespace {
@@ -417,12 +419,17 @@ hipError_t launch_gemm(hipStream_t st, const GemmArgs &g) {
   if constexpr (!AK) {
     if (full) {
       constexpr int lds = 4 * 256 * 64 * 2;  // two buffers of two 32 KiB tiles
-      static bool configured = false;
-      if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_direct<EPI>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      // the attribute belongs to the (kernel, device) pair: remember the devices already configured
+      static std::atomic<uint64_t> configured{0};
+      int dev = 0;
+      hipError_t e = hipGetDevice(&dev);
+      if (e != hipSuccess) return e;
+      const uint64_t bit = 1ull << (dev & 63);
+      if (!(configured.load(std::memory_order_acquire) & bit)) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_direct<EPI>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        configured = true;
+        configured.fetch_or(bit, std::memory_order_release);
       }
       hipLaunchKernelGGL((k_gemm_direct<EPI>), dim3(8 * groups * g.n_tiles), dim3(512), lds, st, g);
       return hipSuccess;

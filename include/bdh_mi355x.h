@@ -18,6 +18,10 @@
  *     src/model/bdh.rs:314-318, src/model/config.rs:143-153).  bdh_last_error() gives the
  *     text of the last failure on a context.
  *   - A context is not re-entrant; independent contexts may be used from different threads.
+ *   - A context belongs to the device it was created on; the caller keeps that device current
+ *     (hipSetDevice) on the calling thread for every call that takes the context or a model of it.
+ *   - Entry points may grow the context's workspace (hipMalloc) the first time a shape is seen: run a
+ *     step of each shape once before capturing calls in a HIP graph.
  *   - There is no CPU fallback: without a HIP device every compute entry point fails.
  */
 #ifndef BDH_MI355X_H

@@ -1,0 +1,205 @@
+"""Edge cases of the C ABI on the GPU: empty and ragged shapes, the size limits, positions beyond the
+exact-integer range of f32, a bf16-state model, degenerate rows.  Values against the CPU oracle
+(f32 state 1e-3, bf16 state 2e-2, index artefacts bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bdh_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def bda():
+    if not torch.cuda.is_available():
+        pytest.fail("no HIP device: the GPU tests must run on the MI355X box")
+    import burn_dragon_amd
+
+    return burn_dragon_amd
+
+
+def rel_err(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def test_empty_shapes_are_no_ops(bda):
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.kernel import BlockPattern1d
+    from burn_dragon_amd.kernel.relu_lowrank import fused_forward
+    from burn_dragon_amd.recurrent import layer_norm, recurrent_attention
+
+    z = lambda *s: torch.zeros(s, device=DEV)
+    out = recurrent_attention(z(0, 2, 1, 64), z(0, 1, 32), z(0, 2, 64, 32), z(64), 0)
+    assert tuple(out.shape) == (0, 2, 1, 32)
+    out = recurrent_attention(z(2, 2, 0, 64), z(2, 0, 32), z(2, 2, 64, 32), z(64), 0)
+    assert tuple(out.shape) == (2, 2, 0, 32)
+    assert tuple(fused_forward(z(0, 1, 3, 8), z(2, 8, 16), None, 0.0, BlockPattern1d.dense(4)).shape) == (0, 2, 3, 16)
+    assert tuple(layer_norm(z(0, 16)).shape) == (0, 16)
+    cfg = bda.BDHConfig(n_layer=1, n_embd=16, n_head=2, mlp_internal_dim_multiplier=4, vocab_size=8)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    model = bda.BDH(cfg, DEV, seed=1)
+    st = model.init_state()
+    assert tuple(model.forward_with_state(torch.zeros((2, 0), dtype=torch.int64), st).shape) == (2, 0, 8)
+    assert st.position == 0
+    ctx = ffi.default_context(0)
+    assert ctx.lib.bdh_sample_top_k(ctx.handle, 0, 8, None, 8, 1.0, 0, None, None) == ffi.OK
+    assert ctx.lib.bdh_alibi_materialize(ctx.handle, 0, 2, 8, 4, 0, None, None, None, ffi.F32, None) == ffi.OK
+    torch.cuda.synchronize()
+
+
+def test_zero_latent_gives_a_zero_readout(bda):
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    out = recurrent_attention(torch.zeros((2, 2, 1, 0), device=DEV), torch.ones((2, 1, 8), device=DEV),
+                              torch.zeros((2, 2, 0, 8), device=DEV), torch.zeros(0, device=DEV), 3)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (2, 2, 1, 8) and float(out.abs().max()) == 0.0
+
+
+def test_size_limits(bda, corc):
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    rng = np.random.default_rng(0)
+    # d = 1024 is the widest state row; h = 64 the most heads
+    for B, h, N, d in [(1, 1, 64, 1024), (1, 64, 16, 8)]:
+        x = np.maximum(rng.standard_normal((B, h, 1, N)), 0).astype(np.float32)
+        v = rng.standard_normal((B, 1, d)).astype(np.float32)
+        rho = (0.1 * rng.standard_normal((B, h, N, d))).astype(np.float32)
+        freqs = corc.build_freqs(N)
+        rt = torch.from_numpy(rho).to(DEV)
+        out = recurrent_attention(torch.from_numpy(x).to(DEV), torch.from_numpy(v).to(DEV), rt,
+                                  torch.from_numpy(freqs).to(DEV), 5)
+        o_ref, r_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.ROPE, 5), v, rho)
+        assert rel_err(out.cpu().numpy(), o_ref) < 1e-3 and rel_err(rt.cpu().numpy(), r_ref) < 1e-3
+    ctx = ffi.default_context(0)
+    t = torch.zeros(1 << 16, device=DEV)
+    p = t.data_ptr()
+    assert ctx.lib.bdh_state_step(ctx.handle, 1, 1, 4, 1028, ffi.ROPE, p, p, p, 0, None, None, p, ffi.F32, p, None,
+                                  None) == ffi.E_SHAPE
+    assert ctx.lib.bdh_state_step(ctx.handle, 1, 65, 4, 4, ffi.ROPE, p, p, p, 0, None, None, p, ffi.F32, p, None,
+                                  None) == ffi.E_SHAPE
+    assert b"n_head" in ctx.lib.bdh_last_error(ctx.handle)
+
+
+@pytest.mark.parametrize("position", [(1 << 24) + 1, (1 << 31) + 12345, (1 << 40) + 7])
+def test_positions_beyond_the_exact_range_of_f32(bda, corc, position):
+    """The reference converts the position to f32 before multiplying by the frequency
+    (src/model/attention.rs:337-343): beyond 2^24 that rounds, and the device must round the same way."""
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    rng = np.random.default_rng(7)
+    B, h, N, d = 2, 2, 256, 256
+    x = np.maximum(rng.standard_normal((B, h, 1, N)) - 1.0, 0).astype(np.float32)
+    v = rng.standard_normal((B, 1, d)).astype(np.float32)
+    rho = (0.1 * rng.standard_normal((B, h, N, d))).astype(np.float32)
+    freqs = corc.build_freqs(N)
+    rt = torch.from_numpy(rho).to(DEV)
+    out = recurrent_attention(torch.from_numpy(x).to(DEV), torch.from_numpy(v).to(DEV), rt,
+                              torch.from_numpy(freqs).to(DEV), position)
+    o_ref, r_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.ROPE, position), v, rho)
+    assert rel_err(out.cpu().numpy(), o_ref) < 1e-3 and rel_err(rt.cpu().numpy(), r_ref) < 1e-3
+
+
+@pytest.mark.parametrize("B,h_in,T,d,h,N", [(1, 1, 1, 4, 1, 1), (2, 3, 17, 20, 3, 77), (3, 1, 9, 256, 2, 130)])
+def test_relu_lowrank_ragged_shapes_bias_mask_and_gate(bda, corc, B, h_in, T, d, h, N):
+    from burn_dragon_amd.kernel import BlockPattern1d
+    from burn_dragon_amd.kernel.relu_lowrank import fused_forward
+
+    rng = np.random.default_rng(B * 100 + N)
+    inp = rng.standard_normal((B, h_in, T, d)).astype(np.float32)
+    w = rng.standard_normal((h, d, N)).astype(np.float32)
+    bias = rng.standard_normal((h, 1, N)).astype(np.float32)
+    bs = 5
+    nblk = (N + bs - 1) // bs
+    active = sorted(set(rng.integers(0, nblk, size=max(nblk // 2, 1)).tolist()))
+    layout = BlockPattern1d.from_blocks(bs, active)
+    out = fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(w).to(DEV), torch.from_numpy(bias).to(DEV),
+                        0.3, layout)
+    ref = corc.relu_lowrank(inp, w, bias, 0.3, bs, active)
+    assert np.array_equal(out.cpu().numpy(), ref)  # one k-sequential chain per output: bit-exact
+    gate = np.maximum(rng.standard_normal((B, h, T, N)), 0).astype(np.float32)
+    gated = fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(w).to(DEV), None, 0.0,
+                          BlockPattern1d.dense(4), gate=torch.from_numpy(gate).to(DEV))
+    assert np.array_equal(gated.cpu().numpy(), corc.relu_lowrank(inp, w, None, 0.0) * gate)
+
+
+def test_layer_norm_degenerate_rows(bda, corc):
+    from burn_dragon_amd.recurrent import layer_norm
+
+    x = np.zeros((4, 33), np.float32)
+    x[1] = 7.5  # constant row: variance 0 -> (x - mean) / sqrt(eps) = 0
+    x[2, 5] = 1e20
+    x[3] = np.linspace(-1, 1, 33)
+    out = layer_norm(torch.from_numpy(x).to(DEV)).cpu().numpy()
+    assert np.array_equal(out[:2], np.zeros((2, 33), np.float32))
+    ref = corc.layer_norm(x)
+    assert np.array_equal(np.isfinite(out), np.isfinite(ref))
+    assert np.array_equal(out[3], ref[3])
+    one = layer_norm(torch.full((3, 1), 2.0, device=DEV)).cpu().numpy()
+    assert np.array_equal(one, np.zeros((3, 1), np.float32))  # d = 1: every row is constant
+
+
+def test_smallest_model_and_argmax_ties(bda, corc):
+    cfg = bda.BDHConfig(n_layer=1, n_embd=4, n_head=1, mlp_internal_dim_multiplier=1, vocab_size=1)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    model = bda.BDH(cfg, DEV, seed=3)
+    logits, nxt = model.forward_with_state(torch.zeros((1, 1), dtype=torch.int64), model.init_state(), want_next=True)
+    assert tuple(logits.shape) == (1, 1, 1) and int(nxt[0]) == 0
+    # identical lm_head columns give identical logits: the argmax is the lowest index, as the oracle's
+    cfg = bda.BDHConfig(n_layer=1, n_embd=16, n_head=2, mlp_internal_dim_multiplier=4, vocab_size=12)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    shape = orc.BDHShape(n_layer=1, n_embd=16, n_head=2, mlp_internal_dim_multiplier=4, vocab_size=12, rotary=orc.ROPE)
+    w = orc.init_weights(shape, 4)
+    w.lm_head[:, :] = w.lm_head[:, :1]
+    model = bda.BDH(cfg, DEV, weights=vars(w))
+    tokens = np.array([[3, 1, 4]])
+    logits, nxt = model.forward_with_state(torch.from_numpy(tokens), model.init_state(), want_next=True)
+    assert int(nxt[0]) == 0 == corc.greedy_token(logits[0, -1].cpu().numpy())
+
+
+@pytest.mark.parametrize("rotary", ["rope", "alibi", "pope"])
+def test_model_with_bf16_state(bda, corc, rotary):
+    """bf16 storage of rho, f32 accumulate: logits within 2e-2 of the f32 oracle over a prompt and a few
+    decode steps (north_star's tolerance for a bf16 state)."""
+    from burn_dragon_amd import ffi
+
+    cfg = bda.BDHConfig(n_layer=3, n_embd=256, n_head=4, mlp_internal_dim_multiplier=8, vocab_size=64)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse(rotary))
+    rot = {"rope": orc.ROPE, "alibi": orc.ALIBI, "pope": orc.POPE}[rotary]
+    shape = orc.BDHShape(n_layer=3, n_embd=256, n_head=4, mlp_internal_dim_multiplier=8, vocab_size=64, rotary=rot)
+    w = orc.init_weights(shape, 13)
+    model = bda.BDH(cfg, DEV, weights=vars(w), rho_dtype=ffi.BF16)
+    tokens = np.random.default_rng(2).integers(0, 64, size=(2, 12))
+    state = model.init_state()
+    logits = model.forward_with_state(torch.from_numpy(tokens[:, :8]), state)
+    assert state.storage.dtype == torch.bfloat16
+    Nq = 512 * (2 if rotary == "pope" else 1)
+    rho = np.zeros((3, 2, 4, Nq, 256), np.float32)
+    ref, pos, _, _ = corc.forward_with_state(shape, w, tokens[:, :8], rho, 0, sparse_state=False)
+    assert rel_err(logits.cpu().numpy(), ref) < 2e-2
+    for t in range(8, 12):
+        lg = model.forward_with_state(torch.from_numpy(tokens[:, t:t + 1]), state)
+        ref, pos, _, _ = corc.forward_with_state(shape, w, tokens[:, t:t + 1], rho, pos, sparse_state=False)
+        assert rel_err(lg.cpu().numpy(), ref) < 2e-2
+    assert rel_err(state.storage.float().cpu().numpy(), rho) < 2e-2
+
+
+def test_pope_step_at_the_config1_layer_shape(bda, corc):
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    rng = np.random.default_rng(11)
+    B, h, N, d = 1, 4, 8192, 256
+    x = rng.standard_normal((B, h, 1, N)).astype(np.float32)  # PoPE takes softplus(x): every row is active
+    v = rng.standard_normal((B, 1, d)).astype(np.float32)
+    rho = (0.01 * rng.standard_normal((B, h, 2 * N, d))).astype(np.float32)
+    freqs = corc.build_freqs(N, rotary=orc.POPE)
+    rt = torch.from_numpy(rho).to(DEV)
+    out, rows = recurrent_attention(torch.from_numpy(x).to(DEV), torch.from_numpy(v).to(DEV), rt,
+                                    torch.from_numpy(freqs).to(DEV), 777, bda.RotaryEmbedding.POPE, want_rows=True)
+    o_ref, r_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.POPE, 777), v, rho)
+    assert rel_err(out.cpu().numpy(), o_ref) < 1e-3 and rel_err(rt.cpu().numpy(), r_ref) < 1e-3
+    assert (rows.cpu().numpy() == 2 * N).all()
