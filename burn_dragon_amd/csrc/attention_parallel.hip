@@ -4,8 +4,10 @@
 //
 // This is the reference's training-path form; it is kept in f32 and follows the reference's
 // block semantics exactly (including the ALiBi term being added to every entry of an active
-// block).  It is a straightforward row-per-workgroup kernel, not tuned: the large-shape
-// inference form is the bf16 matrix-core path in prefill.hip.
+// block).  Small problems take a row-per-workgroup kernel; from T = 128 on the two products run
+// on the f32 matrix cores (v_mfma_f32_32x32x2_f32): S = mask(Q Q^T) + bias is materialised per
+// slice, a row pass sums |S|, and out = (S V) / (norm + eps).  The bf16 form for inference is in
+// prefill.hip.
 #include <vector>
 
 #include "bdh_internal.h"
@@ -105,6 +107,198 @@ __global__ __launch_bounds__(256) void k_fsa_row(const float *__restrict__ q, co
   }
 }
 
+// ------------------------------------------------------------------------------------
+// f32 matrix-core path
+// ------------------------------------------------------------------------------------
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int FT = 128;   // tile rows and columns
+constexpr int FK = 16;    // k per LDS stage
+constexpr int FLD = 20;   // LDS row stride in floats (80 bytes: 16-byte aligned, spreads the banks)
+
+struct FsaArgs {
+  const float *A;   // [slices][M][lda], k contiguous
+  const float *Bm;  // B_KMAJOR ? [b][K][ldb] (n contiguous) : [slices][N][ldb] (k contiguous)
+  float *C;         // [slices][M][ldc]
+  long a_batch, b_batch, c_batch;
+  int lda, ldb, ldc, M, N, K;
+  int b_div;        // B slice = slice / b_div
+  int n_slices;
+  // scores epilogue
+  int block_size, tb, h, use_alibi, dense;
+  const unsigned char *active;  // [tb*tb] when !dense
+  const float *slopes;          // [h] device
+  // output epilogue
+  const float *norm;            // [slices][M] or null
+};
+
+__device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_ok) {
+  if (n_valid >= 4 && vec_ok) return *reinterpret_cast<const float4 *>(p);
+  float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (n_valid > 0) r.x = p[0];
+  if (n_valid > 1) r.y = p[1];
+  if (n_valid > 2) r.z = p[2];
+  if (n_valid > 3) r.w = p[3];
+  return r;
+}
+
+// EPI 0: scores (mask, ALiBi term, zero outside the pattern); EPI 1: out = acc / (norm + eps)
+template <int EPI, bool B_KMAJOR>
+__global__ __launch_bounds__(256) void k_fsa_gemm_f32(FsaArgs g) {
+  __shared__ __attribute__((aligned(16))) float s_a[FT * FLD];
+  __shared__ __attribute__((aligned(16))) float s_b[FT * FLD];
+  const int slice = blockIdx.z;
+  const int m0 = blockIdx.y * FT, n0 = blockIdx.x * FT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 waves, 64 x 64 each
+  const float *A = g.A + (long)slice * g.a_batch;
+  const float *Bm = g.Bm + (long)(slice / g.b_div) * g.b_batch;
+  float *C = g.C + (long)slice * g.c_batch;
+  const int bs = g.block_size;
+
+  int K = g.K;
+  bool tile_active = true;
+  if (EPI == 0) {
+    // dense pattern: block (rb, cb) is active iff cb <= rb; a tile all of whose blocks lie above
+    // the diagonal only writes zeros
+    if (g.dense && n0 / bs > (min(m0 + FT, g.M) - 1) / bs) tile_active = false;
+  } else if (g.dense) {
+    K = min(K, ((min(m0 + FT, g.M) - 1) / bs + 1) * bs);  // S is zero beyond the row tile's last block
+  }
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  if (tile_active) {
+    const bool a_vec = (g.lda % 4 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0);
+    const bool b_vec = (g.ldb % 4 == 0) && (reinterpret_cast<uintptr_t>(Bm) % 16 == 0);
+    float4 ra[2], rb[2];
+    auto load = [&](int k0) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int chunk = c * 256 + tid;
+        {
+          const int row = chunk >> 2, kc = (chunk & 3) * 4;
+          ra[c] = (m0 + row < g.M) ? fsa_ld4(A + (long)(m0 + row) * g.lda + k0 + kc, K - (k0 + kc), a_vec)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        if (!B_KMAJOR) {
+          const int row = chunk >> 2, kc = (chunk & 3) * 4;
+          rb[c] = (n0 + row < g.N) ? fsa_ld4(Bm + (long)(n0 + row) * g.ldb + k0 + kc, K - (k0 + kc), b_vec)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+          const int kr = chunk >> 5, nc = (chunk & 31) * 4;  // 32 chunks of 4 columns per k row
+          rb[c] = (k0 + kr < K) ? fsa_ld4(Bm + (long)(k0 + kr) * g.ldb + n0 + nc, g.N - (n0 + nc), b_vec)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
+    };
+    auto store = [&]() {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int chunk = c * 256 + tid;
+        {
+          const int row = chunk >> 2, kc = (chunk & 3) * 4;
+          *reinterpret_cast<float4 *>(s_a + row * FLD + kc) = ra[c];
+        }
+        if (!B_KMAJOR) {
+          const int row = chunk >> 2, kc = (chunk & 3) * 4;
+          *reinterpret_cast<float4 *>(s_b + row * FLD + kc) = rb[c];
+        } else {
+          const int kr = chunk >> 5, nc = (chunk & 31) * 4;
+          s_b[(nc + 0) * FLD + kr] = rb[c].x;
+          s_b[(nc + 1) * FLD + kr] = rb[c].y;
+          s_b[(nc + 2) * FLD + kr] = rb[c].z;
+          s_b[(nc + 3) * FLD + kr] = rb[c].w;
+        }
+      }
+    };
+    load(0);
+    for (int k0 = 0; k0 < K; k0 += FK) {
+      __syncthreads();
+      store();
+      __syncthreads();
+      if (k0 + FK < K) load(k0 + FK);
+      // lane (r = lane % 32, half = lane / 32) feeds k = half*8 + j to the j-th of eight 32x32x2 steps
+      const int r = lane & 31, kb = (lane >> 5) * 8;
+      float fa[2][8], fb[2][8];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const float4 lo = *reinterpret_cast<const float4 *>(s_a + (wm * 64 + i * 32 + r) * FLD + kb);
+        const float4 hi = *reinterpret_cast<const float4 *>(s_a + (wm * 64 + i * 32 + r) * FLD + kb + 4);
+        fa[i][0] = lo.x; fa[i][1] = lo.y; fa[i][2] = lo.z; fa[i][3] = lo.w;
+        fa[i][4] = hi.x; fa[i][5] = hi.y; fa[i][6] = hi.z; fa[i][7] = hi.w;
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float4 lo = *reinterpret_cast<const float4 *>(s_b + (wn * 64 + j * 32 + r) * FLD + kb);
+        const float4 hi = *reinterpret_cast<const float4 *>(s_b + (wn * 64 + j * 32 + r) * FLD + kb + 4);
+        fb[j][0] = lo.x; fb[j][1] = lo.y; fb[j][2] = lo.z; fb[j][3] = lo.w;
+        fb[j][4] = hi.x; fb[j][5] = hi.y; fb[j][6] = hi.z; fb[j][7] = hi.w;
+      }
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // accumulator element e of lane l in a 32x32 tile: row = (e/4)*8 + (l/32)*4 + (e%4), col = l%32
+  const float slope = (EPI == 0 && g.use_alibi) ? g.slopes[slice % g.h] : 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * 64 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row >= g.M) continue;
+        if (EPI == 0) {
+          if (col >= g.ldc) continue;
+          float v = 0.0f;
+          if (col < g.N) {
+            const int rbk = row / bs, cbk = col / bs;
+            const bool act = g.dense ? (cbk <= rbk) : (g.active[(long)rbk * g.tb + cbk] != 0);
+            if (act) {
+              v = (rbk == cbk && col >= row) ? 0.0f : acc[i][j][e];  // tril(-1) on diagonal blocks (:88-90)
+              if (g.use_alibi) {  // added to every entry of an active block (:97-100)
+                const float al = slope * ((float)col - (float)row);
+                v = v + al;
+              }
+            }
+          }
+          C[(long)row * g.ldc + col] = v;
+        } else {
+          if (col >= g.N) continue;
+          float v = acc[i][j][e];
+          if (g.norm) v = v / (g.norm[(long)slice * g.M + row] + kRowNormEps);
+          C[(long)row * g.ldc + col] = v;
+        }
+      }
+    }
+}
+
+// norm[row] = sum_s |S[row, s]|: one wave per row
+__global__ __launch_bounds__(256) void k_fsa_row_abs_sum(const float *__restrict__ S, long rows, int T, int ld,
+                                                         float *__restrict__ norm) {
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const float *p = S + row * ld;
+  float a = 0.0f;
+  for (int c = lane; c < T; c += 64) a += fabsf(p[c]);
+  for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o);
+  if (lane == 0) norm[row] = a;
+}
+
 }  // namespace
 
 extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N, int dv, const float *query,
@@ -127,17 +321,24 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
   const bool sparse = block_pairs_host != nullptr;
   if (sparse && tb > 4096) return bdh_fail(ctx, BDH_E_SHAPE, "sparse time pattern with %d blocks", tb);
   const size_t lds = sizeof(float) * ((size_t)Nq + T);
-  if (lds > 150 * 1024) return bdh_fail(ctx, BDH_E_SHAPE, "Nq + T = %ld floats exceed the LDS budget", (long)Nq + T);
-  if (S * T > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "B*h*T too large");
+  int path = ctx->opt_fsa_path;  // -1 choose, 0 row kernel, 1 matrix cores
+  if (path < 0) path = T >= 128 ? 1 : 0;
+  if (path == 0 && lds > 150 * 1024) path = 1;
+  if (S * T > 0x7fffffffL || S > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "B*h*T too large");
 
+  const int Tp = (T + 3) & ~3;  // row stride of the score matrix
   const size_t q_bytes = bdh_align_up(sizeof(float) * (size_t)S * T * Nq, 256);
   const size_t act_bytes = sparse ? bdh_align_up((size_t)tb * tb, 256) : 0;
-  int rc = bdh_ws_reserve(ctx, q_bytes + act_bytes + 512);
+  const size_t sc_bytes = path == 1 ? bdh_align_up(sizeof(float) * (size_t)S * T * Tp, 256) : 0;
+  const size_t nm_bytes = path == 1 ? bdh_align_up(sizeof(float) * (size_t)S * T, 256) : 0;
+  int rc = bdh_ws_reserve(ctx, q_bytes + act_bytes + 512 + sc_bytes + nm_bytes);
   if (rc != BDH_OK) return rc;
   char *ws = static_cast<char *>(ctx->ws);
   float *q = reinterpret_cast<float *>(ws);
   unsigned char *active = sparse ? reinterpret_cast<unsigned char *>(ws + q_bytes) : nullptr;
   float *slopes_dev = reinterpret_cast<float *>(ws + q_bytes + act_bytes);
+  float *scores = reinterpret_cast<float *>(ws + q_bytes + act_bytes + 512);
+  float *norm = reinterpret_cast<float *>(ws + q_bytes + act_bytes + 512 + sc_bytes);
   if (sparse) {
     std::vector<unsigned char> m((size_t)tb * tb, 0);
     for (int p = 0; p < n_pairs; ++p) {
@@ -153,6 +354,32 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
   }
   hipLaunchKernelGGL(k_rotate_f32, dim3((unsigned)(S * T)), dim3(256), 0, ctx->stream, query, freqs, q, T, N, rotary);
   BDH_LAUNCH_CHECK(ctx, "k_rotate_f32");
+  if (path == 1) {
+    FsaArgs g{};
+    g.A = q; g.Bm = q; g.C = scores;
+    g.a_batch = g.b_batch = (long)T * Nq; g.c_batch = (long)T * Tp;
+    g.lda = g.ldb = Nq; g.ldc = Tp; g.M = g.N = T; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
+    g.block_size = block_size; g.tb = tb; g.h = h; g.use_alibi = alibi_slopes_host ? 1 : 0; g.dense = sparse ? 0 : 1;
+    g.active = active; g.slopes = slopes_dev; g.norm = nullptr;
+    const int tiles = (T + FT - 1) / FT;
+    hipLaunchKernelGGL((k_fsa_gemm_f32<0, false>), dim3(tiles, tiles, (unsigned)S), dim3(256), 0, ctx->stream, g);
+    BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<scores>");
+    if (row_normalize) {
+      hipLaunchKernelGGL(k_fsa_row_abs_sum, dim3((unsigned)((S * T + 3) / 4)), dim3(256), 0, ctx->stream, scores,
+                         S * T, T, Tp, norm);
+      BDH_LAUNCH_CHECK(ctx, "k_fsa_row_abs_sum");
+    }
+    FsaArgs o{};
+    o.A = scores; o.Bm = value; o.C = out;
+    o.a_batch = (long)T * Tp; o.b_batch = (long)T * dv; o.c_batch = (long)T * dv;
+    o.lda = Tp; o.ldb = dv; o.ldc = dv; o.M = T; o.N = dv; o.K = T; o.b_div = h; o.n_slices = (int)S;
+    o.block_size = block_size; o.tb = tb; o.h = h; o.dense = sparse ? 0 : 1;
+    o.norm = row_normalize ? norm : nullptr;
+    hipLaunchKernelGGL((k_fsa_gemm_f32<1, true>), dim3((dv + FT - 1) / FT, tiles, (unsigned)S), dim3(256), 0,
+                       ctx->stream, o);
+    BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<out>");
+    return BDH_OK;
+  }
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_fsa_row),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) {

@@ -18,6 +18,7 @@ struct bdh_ctx {
   size_t ws_bytes = 0;
   int n_cu = 0;
   int opt_step_split = -1;  // -1 choose by grid size, 0 / 1 force the 256- / 64-pair workgroup
+  int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
   char err[512] = {0};
 };
 

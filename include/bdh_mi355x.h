@@ -67,7 +67,9 @@ int bdh_ctx_synchronize(bdh_ctx *ctx);
 const char *bdh_last_error(const bdh_ctx *ctx);
 /* Launch-shape knobs for tests and tuning; no counterpart in the reference.
  *   "state_step.split": -1 (default) pick by grid size, 0 = 256 lane pairs per workgroup,
- *                       1 = 64 lane pairs per workgroup of 8 waves (small batches). */
+ *                       1 = 64 lane pairs per workgroup of 8 waves (small batches).
+ *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
+ *                       1 = the two products on the f32 matrix cores (T >= 128 by default). */
 int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);
 
 /* ---- host-side tables (computed on the host in the reference as well) --------------- */

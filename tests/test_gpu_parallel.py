@@ -33,8 +33,19 @@ def rel_err(a, b):
 
 
 # ------------------------------------------------------------ fused_state_aligned
+@pytest.fixture(params=[0, 1], ids=["row-kernel", "matrix-cores"])
+def fsa_path(request, bda):
+    """Runs a test once per implementation of fused_state_aligned (the default picks by T)."""
+    from burn_dragon_amd import ffi
+
+    ctx = ffi.default_context(0)
+    ctx.set_option("fused_state_aligned.path", request.param)
+    yield request.param
+    ctx.set_option("fused_state_aligned.path", -1)
+
+
 @pytest.mark.parametrize("rotary,seed", [("rope", 1337), ("pope", 2024)])
-def test_fused_attention_matches_reference(bda, corc, rotary, seed):
+def test_fused_attention_matches_reference(bda, corc, fsa_path, rotary, seed):
     """tests/fused_kernel_tests.rs:70-170 on the device path: B=1, h=2, T=6, N=8, dv=6,
     BlockPattern2d::dense(3); fused == dense tril(-1) + row-normalise, tolerance 1e-4."""
     from burn_dragon_amd.kernel import linear_attention
@@ -58,7 +69,7 @@ def test_fused_attention_matches_reference(bda, corc, rotary, seed):
     assert_close(fused.cpu().numpy(), ref_c, 1e-4, 1e-4)
 
 
-def test_fused_attention_alibi_sparse_pattern_and_unnormalised(bda, corc):
+def test_fused_attention_alibi_sparse_pattern_and_unnormalised(bda, corc, fsa_path):
     from burn_dragon_amd.kernel import linear_attention
 
     rng = np.random.default_rng(3)
@@ -85,6 +96,38 @@ def test_fused_attention_alibi_sparse_pattern_and_unnormalised(bda, corc):
                                                bda.RotaryEmbedding.ROPE, row_normalize=False)
     out_rec, _ = corc.recurrent_attention(corc.rotate(query, freqs, orc.ROPE, 0), value, np.zeros((B, h, N, dv), np.float32))
     assert_close(got.cpu().numpy(), out_rec, 1e-4, 1e-4)
+
+
+@pytest.mark.parametrize("rotary", ["rope", "alibi", "pope"])
+def test_fused_attention_medium_shapes_on_the_matrix_cores(bda, corc, rotary):
+    """T = 300 (default path: f32 matrix cores), ragged against the 128-wide tiles and the time block of
+    48, N and dv not multiples of 4: against the oracle's blocked form, normalised and not, dense and
+    with a sparse block pattern."""
+    from burn_dragon_amd.kernel import linear_attention
+
+    rng = np.random.default_rng(5)
+    B, h, T, N, dv, bs = 2, 3, 300, 202, 70, 48
+    query = np.maximum(rng.standard_normal((B, h, T, N)) - 0.5, 0).astype(np.float32)
+    value = rng.standard_normal((B, T, dv)).astype(np.float32)
+    rot = {"rope": orc.ROPE, "alibi": orc.ALIBI, "pope": orc.POPE}[rotary]
+    slopes = corc.default_alibi_slopes(h) if rotary == "alibi" else None
+    freqs = corc.build_freqs(N, rotary=rot)
+    qt, vt = torch.from_numpy(query).to(DEV), torch.from_numpy(value[:, None]).to(DEV)
+    st = None if slopes is None else torch.from_numpy(slopes)
+    tb = (T + bs - 1) // bs
+    pairs = {(r, c) for r in range(tb) for c in range(r + 1) if (r + 2 * c) % 3 != 1}
+    for layout, kw in [(bda.BlockPattern2d.dense(bs), {}), (bda.BlockPattern2d.from_pairs(bs, pairs), {"pairs": pairs})]:
+        got = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs), st, layout,
+                                                   bda.RotaryEmbedding.parse(rotary))
+        ref = corc.fused_state_aligned(query, value, freqs, slopes, bs, rot, **kw)
+        assert rel_err(got.cpu().numpy(), ref) < 1e-3
+    got = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs), st, bda.BlockPattern2d.dense(bs),
+                                               bda.RotaryEmbedding.parse(rotary), row_normalize=False)
+    if rotary != "alibi":  # the un-normalised dense form is the recurrent path from a zero state
+        Nq = 2 * N if rotary == "pope" else N
+        out_rec, _ = corc.recurrent_attention(corc.rotate(query, freqs, rot, 0), value,
+                                              np.zeros((B, h, Nq, dv), np.float32))
+        assert rel_err(got.cpu().numpy(), out_rec) < 1e-3
 
 
 # ---------------------------------------------------------------- chunked prefill
