@@ -785,6 +785,11 @@ void launch_finalize(hipStream_t st, int slices, const float *partial, const int
                        out_stride, out_ln, rows, rows_stride, rows_per_count);
 }
 
+__global__ __launch_bounds__(256) void k_fill_zero_u32(uint32_t *__restrict__ p, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
 template <int D, int WAVES, int U, int SPLIT>
 void launch_fast(hipStream_t st, int blocks, const StepPtrs &a, float *rho) {
   hipLaunchKernelGGL((k_step_rope_f32<D, WAVES, U, SPLIT>), dim3(blocks), dim3(WAVES * 64), 0, st, a, rho);
@@ -811,9 +816,19 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   const int S = fast ? ((N / 2) + ppb - 1) / ppb : fast_lazy ? (N + 511) / 512 : (Nq + kGenRows - 1) / kGenRows;
   if (N == 0 || d == 0) {
     // nothing to read or update: the readout is an empty sum
-    if (d > 0) BDH_HIP_CHECK(ctx, hipMemsetAsync(p.out, 0, sizeof(float) * (size_t)slices * T * d, ctx->stream));
+    // cleared by a kernel, not a memset node, so that a caller may capture this call in a HIP graph
     if (out_ln && d > 0) return bdh_fail(ctx, BDH_E_SHAPE, "LayerNorm of an empty readout");
-    if (p.rows_touched) BDH_HIP_CHECK(ctx, hipMemsetAsync(p.rows_touched, 0, sizeof(int32_t) * (size_t)slices * T, ctx->stream));
+    const size_t n_out = (size_t)slices * T * d, n_rows = p.rows_touched ? (size_t)slices * T : 0;
+    if (n_out) {
+      hipLaunchKernelGGL(k_fill_zero_u32, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, ctx->stream,
+                         reinterpret_cast<uint32_t *>(p.out), n_out);
+      BDH_LAUNCH_CHECK(ctx, "k_fill_zero_u32");
+    }
+    if (n_rows) {
+      hipLaunchKernelGGL(k_fill_zero_u32, dim3((unsigned)((n_rows + 255) / 256)), dim3(256), 0, ctx->stream,
+                         reinterpret_cast<uint32_t *>(p.rows_touched), n_rows);
+      BDH_LAUNCH_CHECK(ctx, "k_fill_zero_u32");
+    }
     return BDH_OK;
   }
   const size_t partial_bytes = bdh_align_up(sizeof(float) * (size_t)slices * S * d, 256);
