@@ -167,6 +167,118 @@ def bench_copy(args):
                                  "bytes_read_per_step": n * 4, "bytes_written_per_step": n * 4}}))
 
 
+F32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense f32 matrix, published
+
+
+def bench_alibi(args):
+    """Single-layer ALiBi state step at the decode shape: the reference's eager decay (a dense pass
+    over rho every token, src/model/bdh.rs:299-301) beside the lazily decayed state of this library.
+    `value` is the lazy step; the eager figures ride along in config."""
+    import torch
+    from scipy.stats import norm
+
+    from burn_dragon_amd.positional import RotaryEmbedding
+    from burn_dragon_amd.recurrent import recurrent_attention, recurrent_attention_lazy_alibi
+
+    dev = torch.device("cuda:0")
+    B, h, N, d = args.batch, args.heads, args.latent, args.embd
+    steps = 200 if args.steps == 1000 else args.steps
+    warmup = min(args.warmup, 10)
+    g = torch.Generator(device=dev).manual_seed(1)
+    mu = float(norm.ppf(args.density))
+    ring = min(args.ring, 8)
+    xs = [torch.relu(torch.randn((B, h, 1, N), device=dev, generator=g) + mu) for _ in range(ring)]
+    vs = [torch.randn((B, 1, d), device=dev, generator=g) for _ in range(ring)]
+    rho = 0.01 * torch.randn((B, h, N, d), device=dev, generator=g)
+    stamps = torch.zeros((B, h, N), device=dev, dtype=torch.int32)
+    fz = torch.zeros(N, device=dev)
+    rows = float(sum(int((x != 0).sum()) for x in xs)) / ring
+    times = {}
+    for name in ("eager", "lazy"):
+        n = steps if name == "lazy" else max(steps // 10, 5)
+
+        def step(i):
+            if name == "eager":
+                recurrent_attention(xs[i % ring], vs[i % ring], rho, fz, i, RotaryEmbedding.ALIBI)
+            else:
+                recurrent_attention_lazy_alibi(xs[i % ring], vs[i % ring], rho, stamps, i)
+
+        for i in range(warmup):
+            step(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(n):
+            step(warmup + i)
+        e1.record()
+        torch.cuda.synchronize()
+        times[name] = max(e0.elapsed_time(e1), (time.perf_counter() - t0) * 1e3) / n
+    lazy_bytes = 2.0 * rows * d * 4 + 8.0 * rows + 4.0 * B * h * N + 4.0 * B * d + 4.0 * B * h * d
+    dense_bytes = 2.0 * B * h * N * d * 4
+    ms = times["lazy"]
+    achieved = lazy_bytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "decode tokens/sec at batch B (single-layer ALiBi state step, lazily decayed state)",
+        "value": B / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"ALiBi state step, rho f32 [{B},{h},{N},{d}], {args.density:.0%} active, {ring} input sets",
+                   "active_rows_per_step": rows, "algorithmic_bytes_per_step": lazy_bytes,
+                   "eager_ms_per_step": times["eager"], "eager_dense_bytes_per_step": dense_bytes,
+                   "eager_GBps": dense_bytes / (times["eager"] * 1e-3) / 1e9, "speedup": times["eager"] / ms},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "k_step_alibi_lazy_f32 (+ k_step_finalize)"},
+    }))
+
+
+def bench_parallel(args):
+    """kernel::linear_attention::fused_state_aligned (src/kernel/linear_attention.rs:11-115) in f32 at the
+    config-3 shape: normalised causal linear attention over all tokens at once on the f32 matrix cores."""
+    import torch
+
+    from burn_dragon_amd.kernel import BlockPattern2d
+    from burn_dragon_amd.kernel.linear_attention import build_freqs, fused_state_aligned
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    dev = torch.device("cuda:0")
+    B = 8 if args.batch == 32 else args.batch
+    h, N, d, T = args.heads, args.latent, args.embd, args.time
+    steps = 5 if args.steps == 1000 else args.steps
+    warmup = min(args.warmup, 1)
+    g = torch.Generator(device=dev).manual_seed(3)
+    q = torch.empty((B, h, T, N), device=dev)
+    for b in range(B):
+        q[b] = torch.relu(torch.randn((h, T, N), device=dev, generator=g) - 1.6449)
+    v = torch.randn((B, 1, T, d), device=dev, generator=g)
+    f = build_freqs(N, 65536.0, RotaryEmbedding.ROPE, device=dev)
+    layout = BlockPattern2d.dense(64)
+    for _ in range(warmup):
+        fused_state_aligned(q, v, f, None, layout, RotaryEmbedding.ROPE)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fused_state_aligned(q, v, f, None, layout, RotaryEmbedding.ROPE)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = max(e0.elapsed_time(e1), (time.perf_counter() - t0) * 1e3) / steps
+    flop = float(B * h) * (T * (T - 1.0) * N + T * (T - 1.0) * d)
+    achieved = flop / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "tokens/sec, fused_state_aligned (normalised causal linear attention, f32)",
+        "value": B * T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"fused_state_aligned B={B} h={h} T={T} N={N} dv={d}, RoPE, dense time blocks of 64, "
+                               f"row_normalize, 5% active", "algorithmic_flop_per_step": flop},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": F32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / F32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "whole bdh_fused_state_aligned call (k_rotate_f32, k_fsa_gemm_f32 x2, k_fsa_row_abs_sum); "
+                               "algorithmic FLOP = B*h*[T(T-1)N + T(T-1)d]"},
+    }))
+
+
 def bench_model(args):
     """Full-model greedy decode (BDH::forward_with_state per token, argmax on the device).
     c1 = BASELINE config 1 (V=256, d=256, h=4, N=8192, L=6, B=1, 64-byte prompt, 256 tokens);
@@ -248,9 +360,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--prefill-chunk", type=int, default=0,
                     help="model workload: feed the prompt in calls of this many tokens (0 = one call)")
-    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy", "alibi", "parallel"], default="decode",
                     help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA); "
-                         "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4)")
+                         "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4); "
+                         "alibi = ALiBi state step, lazily decayed state beside the eager dense decay; "
+                         "parallel = fused_state_aligned in f32 at the config-3 shape; copy = counter calibration")
     ap.add_argument("--model-config", choices=["c1", "c4"], default="c1")
     ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
     ap.add_argument("--graph", action="store_true", help="model: replay one captured HIP graph per token")
@@ -278,6 +392,10 @@ def main():
         return bench_model(args)
     if args.workload == "copy":
         return bench_copy(args)
+    if args.workload == "alibi":
+        return bench_alibi(args)
+    if args.workload == "parallel":
+        return bench_parallel(args)
     B, h, N, d = args.batch, args.heads, args.latent, args.embd
     ctx = ffi.default_context(0)
     lib = ctx.lib
