@@ -111,7 +111,6 @@ __global__ __launch_bounds__(256) void k_fsa_row(const float *__restrict__ q, co
 // f32 matrix-core path
 // ------------------------------------------------------------------------------------
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-constexpr int FT = 128;   // tile rows and columns
 constexpr int FK = 16;    // k per LDS stage
 constexpr int FLD = 20;   // LDS row stride in floats (80 bytes: 16-byte aligned, spreads the banks)
 
@@ -141,15 +140,22 @@ __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_
   return r;
 }
 
-// EPI 0: scores (mask, ALiBi term, zero outside the pattern); EPI 1: out = acc / (norm + eps)
-template <int EPI, bool B_KMAJOR>
-__global__ __launch_bounds__(256) void k_fsa_gemm_f32(FsaArgs g) {
-  __shared__ __attribute__((aligned(16))) float s_a[FT * FLD];
-  __shared__ __attribute__((aligned(16))) float s_b[FT * FLD];
+// EPI 0: scores (mask, ALiBi term, zero outside the pattern); EPI 1: out = acc / (norm + eps).
+// Tile BM x BN, NWM x NWN waves, each wave (BM/NWM) x (BN/NWN).  The 128 x 128 tile needs 8 bytes per
+// clock and workgroup from the L2, which three resident workgroups per CU do not get; the
+// 256 x 256 tile halves that per FLOP and is the one that keeps the matrix cores busy.
+template <int EPI, bool B_KMAJOR, int BM, int BN, int NWM, int NWN>
+__global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
+  constexpr int NT = NWM * NWN * 64;
+  constexpr int MI = BM / NWM / 32, NJ = BN / NWN / 32;
+  constexpr int CA = BM * 4 / NT, CB = BN * 4 / NT;  // float4 chunks per thread and stage
+  static_assert(CA >= 1 && CB >= 1 && CA * NT == BM * 4 && CB * NT == BN * 4, "tile does not divide over the threads");
+  __shared__ __attribute__((aligned(16))) float s_a[BM * FLD];
+  __shared__ __attribute__((aligned(16))) float s_b[BN * FLD];
   const int slice = blockIdx.z;
-  const int m0 = blockIdx.y * FT, n0 = blockIdx.x * FT;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 waves, 64 x 64 each
+  const int wm = wave / NWN, wn = wave % NWN;
   const float *A = g.A + (long)slice * g.a_batch;
   const float *Bm = g.Bm + (long)(slice / g.b_div) * g.b_batch;
   float *C = g.C + (long)slice * g.c_batch;
@@ -160,106 +166,114 @@ __global__ __launch_bounds__(256) void k_fsa_gemm_f32(FsaArgs g) {
   if (EPI == 0) {
     // dense pattern: block (rb, cb) is active iff cb <= rb; a tile all of whose blocks lie above
     // the diagonal only writes zeros
-    if (g.dense && n0 / bs > (min(m0 + FT, g.M) - 1) / bs) tile_active = false;
+    if (g.dense && n0 / bs > (min(m0 + BM, g.M) - 1) / bs) tile_active = false;
   } else if (g.dense) {
-    K = min(K, ((min(m0 + FT, g.M) - 1) / bs + 1) * bs);  // S is zero beyond the row tile's last block
+    K = min(K, ((min(m0 + BM, g.M) - 1) / bs + 1) * bs);  // S is zero beyond the row tile's last block
   }
 
-  f32x16 acc[2][2];
+  f32x16 acc[MI][NJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   if (tile_active) {
     const bool a_vec = (g.lda % 4 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0);
     const bool b_vec = (g.ldb % 4 == 0) && (reinterpret_cast<uintptr_t>(Bm) % 16 == 0);
-    float4 ra[2], rb[2];
-    auto load = [&](int k0) {
+    float4 ra[1][CA], rb[1][CB];
+    auto load = [&](float4 *pa, float4 *pb, int k0) {
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const int chunk = c * 256 + tid;
-        {
-          const int row = chunk >> 2, kc = (chunk & 3) * 4;
-          ra[c] = (m0 + row < g.M) ? fsa_ld4(A + (long)(m0 + row) * g.lda + k0 + kc, K - (k0 + kc), a_vec)
-                                   : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+      for (int c = 0; c < CA; ++c) {
+        const int chunk = c * NT + tid;
+        const int row = chunk >> 2, kc = (chunk & 3) * 4;
+        pa[c] = (m0 + row < g.M && k0 < K) ? fsa_ld4(A + (long)(m0 + row) * g.lda + k0 + kc, K - (k0 + kc), a_vec)
+                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int c = 0; c < CB; ++c) {
+        const int chunk = c * NT + tid;
         if (!B_KMAJOR) {
           const int row = chunk >> 2, kc = (chunk & 3) * 4;
-          rb[c] = (n0 + row < g.N) ? fsa_ld4(Bm + (long)(n0 + row) * g.ldb + k0 + kc, K - (k0 + kc), b_vec)
-                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+          pb[c] = (n0 + row < g.N && k0 < K) ? fsa_ld4(Bm + (long)(n0 + row) * g.ldb + k0 + kc, K - (k0 + kc), b_vec)
+                                             : make_float4(0.f, 0.f, 0.f, 0.f);
         } else {
-          const int kr = chunk >> 5, nc = (chunk & 31) * 4;  // 32 chunks of 4 columns per k row
-          rb[c] = (k0 + kr < K) ? fsa_ld4(Bm + (long)(k0 + kr) * g.ldb + n0 + nc, g.N - (n0 + nc), b_vec)
+          const int kr = chunk / (BN / 4), nc = (chunk % (BN / 4)) * 4;  // BN/4 chunks of 4 columns per k row
+          pb[c] = (k0 + kr < K) ? fsa_ld4(Bm + (long)(k0 + kr) * g.ldb + n0 + nc, g.N - (n0 + nc), b_vec)
                                 : make_float4(0.f, 0.f, 0.f, 0.f);
         }
       }
     };
-    auto store = [&]() {
+    auto store = [&](const float4 *pa, const float4 *pb) {
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const int chunk = c * 256 + tid;
-        {
-          const int row = chunk >> 2, kc = (chunk & 3) * 4;
-          *reinterpret_cast<float4 *>(s_a + row * FLD + kc) = ra[c];
-        }
+      for (int c = 0; c < CA; ++c) {
+        const int chunk = c * NT + tid;
+        const int row = chunk >> 2, kc = (chunk & 3) * 4;
+        *reinterpret_cast<float4 *>(s_a + row * FLD + kc) = pa[c];
+      }
+#pragma unroll
+      for (int c = 0; c < CB; ++c) {
+        const int chunk = c * NT + tid;
         if (!B_KMAJOR) {
           const int row = chunk >> 2, kc = (chunk & 3) * 4;
-          *reinterpret_cast<float4 *>(s_b + row * FLD + kc) = rb[c];
+          *reinterpret_cast<float4 *>(s_b + row * FLD + kc) = pb[c];
         } else {
-          const int kr = chunk >> 5, nc = (chunk & 31) * 4;
-          s_b[(nc + 0) * FLD + kr] = rb[c].x;
-          s_b[(nc + 1) * FLD + kr] = rb[c].y;
-          s_b[(nc + 2) * FLD + kr] = rb[c].z;
-          s_b[(nc + 3) * FLD + kr] = rb[c].w;
+          const int kr = chunk / (BN / 4), nc = (chunk % (BN / 4)) * 4;
+          s_b[(nc + 0) * FLD + kr] = pb[c].x;
+          s_b[(nc + 1) * FLD + kr] = pb[c].y;
+          s_b[(nc + 2) * FLD + kr] = pb[c].z;
+          s_b[(nc + 3) * FLD + kr] = pb[c].w;
         }
       }
     };
-    load(0);
-    for (int k0 = 0; k0 < K; k0 += FK) {
-      __syncthreads();
-      store();
-      __syncthreads();
-      if (k0 + FK < K) load(k0 + FK);
-      // lane (r = lane % 32, half = lane / 32) feeds k = half*8 + j to the j-th of eight 32x32x2 steps
+    auto multiply = [&]() {
+      // lane (r = lane % 32, half = lane / 32) feeds k = half*8 + q to the q-th of eight 32x32x2 steps
       const int r = lane & 31, kb = (lane >> 5) * 8;
-      float fa[2][8], fb[2][8];
+      float fa[MI][8], fb[NJ][8];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const float4 lo = *reinterpret_cast<const float4 *>(s_a + (wm * 64 + i * 32 + r) * FLD + kb);
-        const float4 hi = *reinterpret_cast<const float4 *>(s_a + (wm * 64 + i * 32 + r) * FLD + kb + 4);
+      for (int i = 0; i < MI; ++i) {
+        const float *p = s_a + (wm * (BM / NWM) + i * 32 + r) * FLD + kb;
+        const float4 lo = *reinterpret_cast<const float4 *>(p), hi = *reinterpret_cast<const float4 *>(p + 4);
         fa[i][0] = lo.x; fa[i][1] = lo.y; fa[i][2] = lo.z; fa[i][3] = lo.w;
         fa[i][4] = hi.x; fa[i][5] = hi.y; fa[i][6] = hi.z; fa[i][7] = hi.w;
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const float4 lo = *reinterpret_cast<const float4 *>(s_b + (wn * 64 + j * 32 + r) * FLD + kb);
-        const float4 hi = *reinterpret_cast<const float4 *>(s_b + (wn * 64 + j * 32 + r) * FLD + kb + 4);
+      for (int j = 0; j < NJ; ++j) {
+        const float *p = s_b + (wn * (BN / NWN) + j * 32 + r) * FLD + kb;
+        const float4 lo = *reinterpret_cast<const float4 *>(p), hi = *reinterpret_cast<const float4 *>(p + 4);
         fb[j][0] = lo.x; fb[j][1] = lo.y; fb[j][2] = lo.z; fb[j][3] = lo.w;
         fb[j][4] = hi.x; fb[j][5] = hi.y; fb[j][6] = hi.z; fb[j][7] = hi.w;
       }
 #pragma unroll
       for (int q = 0; q < 8; ++q)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int j = 0; j < NJ; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc[i][j], 0, 0, 0);
+    };
+    // one register stage: a second one (loads two k-steps ahead) measured no faster
+    load(ra[0], rb[0], 0);
+    for (int k0 = 0; k0 < K; k0 += FK) {
+      __syncthreads();  // the previous step's fragment reads are done
+      store(ra[0], rb[0]);
+      __syncthreads();
+      load(ra[0], rb[0], k0 + FK);  // an out-of-range stage loads nothing
+      multiply();
     }
   }
 
   // accumulator element e of lane l in a 32x32 tile: row = (e/4)*8 + (l/32)*4 + (e%4), col = l%32
   const float slope = (EPI == 0 && g.use_alibi) ? g.slopes[slice % g.h] : 0.0f;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < NJ; ++j) {
+      const int col = n0 + wn * (BN / NWN) + j * 32 + (lane & 31);
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * 64 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        const int row = m0 + wm * (BM / NWM) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
         if (row >= g.M) continue;
         if (EPI == 0) {
           if (col >= g.ldc) continue;
@@ -361,8 +375,17 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     g.lda = g.ldb = Nq; g.ldc = Tp; g.M = g.N = T; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
     g.block_size = block_size; g.tb = tb; g.h = h; g.use_alibi = alibi_slopes_host ? 1 : 0; g.dense = sparse ? 0 : 1;
     g.active = active; g.slopes = slopes_dev; g.norm = nullptr;
-    const int tiles = (T + FT - 1) / FT;
-    hipLaunchKernelGGL((k_fsa_gemm_f32<0, false>), dim3(tiles, tiles, (unsigned)S), dim3(256), 0, ctx->stream, g);
+    // big tiles once there are enough of them to cover the chip; small ones for short sequences
+    const bool big = (long)S * ((T + 255) / 256) * ((T + 255) / 256) >= 256;
+    if (big) {
+      const int tiles = (T + 255) / 256;
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 256, 256, 2, 4>), dim3(tiles, tiles, (unsigned)S), dim3(512), 0,
+                         ctx->stream, g);
+    } else {
+      const int tiles = (T + 127) / 128;
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 128, 128, 2, 2>), dim3(tiles, tiles, (unsigned)S), dim3(256), 0,
+                         ctx->stream, g);
+    }
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<scores>");
     if (row_normalize) {
       hipLaunchKernelGGL(k_fsa_row_abs_sum, dim3((unsigned)((S * T + 3) / 4)), dim3(256), 0, ctx->stream, scores,
@@ -375,8 +398,8 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     o.lda = Tp; o.ldb = dv; o.ldc = dv; o.M = T; o.N = dv; o.K = T; o.b_div = h; o.n_slices = (int)S;
     o.block_size = block_size; o.tb = tb; o.h = h; o.dense = sparse ? 0 : 1;
     o.norm = row_normalize ? norm : nullptr;
-    hipLaunchKernelGGL((k_fsa_gemm_f32<1, true>), dim3((dv + FT - 1) / FT, tiles, (unsigned)S), dim3(256), 0,
-                       ctx->stream, o);
+    hipLaunchKernelGGL((k_fsa_gemm_f32<1, true, 128, 128, 2, 2>), dim3((dv + 127) / 128, (T + 127) / 128, (unsigned)S),
+                       dim3(256), 0, ctx->stream, o);
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<out>");
     return BDH_OK;
   }

@@ -130,6 +130,26 @@ def test_fused_attention_medium_shapes_on_the_matrix_cores(bda, corc, rotary):
         assert rel_err(got.cpu().numpy(), out_rec) < 1e-3
 
 
+def test_fused_attention_long_sequences_take_the_large_tiles(bda, corc):
+    """T = 1100 with 16 slices: the 256 x 256 tiles of the matrix-core path, ragged against them and
+    against the time block of 100; ALiBi (the term lands on whole blocks) and RoPE."""
+    from burn_dragon_amd.kernel import linear_attention
+
+    rng = np.random.default_rng(9)
+    B, h, T, N, dv, bs = 4, 4, 1100, 66, 40, 100
+    query = np.maximum(rng.standard_normal((B, h, T, N)) - 0.5, 0).astype(np.float32)
+    value = rng.standard_normal((B, T, dv)).astype(np.float32)
+    qt, vt = torch.from_numpy(query).to(DEV), torch.from_numpy(value[:, None]).to(DEV)
+    for rotary, rot in (("rope", orc.ROPE), ("alibi", orc.ALIBI)):
+        slopes = corc.default_alibi_slopes(h) if rotary == "alibi" else None
+        freqs = corc.build_freqs(N, rotary=rot)
+        got = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs),
+                                                   None if slopes is None else torch.from_numpy(slopes),
+                                                   bda.BlockPattern2d.dense(bs), bda.RotaryEmbedding.parse(rotary))
+        ref = corc.fused_state_aligned(query, value, freqs, slopes, bs, rot)
+        assert rel_err(got.cpu().numpy(), ref) < 1e-3
+
+
 # ---------------------------------------------------------------- chunked prefill
 def _prefill_case(seed, B, h, T, N, d, density, rho0_scale):
     from scipy.stats import norm
