@@ -44,13 +44,37 @@ def cpu_baseline(B, h, N, d, freqs, budget_s=12.0, max_steps=20):
         orc.state_step_dense(x, v, freqs, 100 + steps, rho)
         steps += 1
     dt = time.perf_counter() - t0
+    one = None
+    try:  # the same step on one thread (Burn's ndarray backend threads only its GEMMs)
+        import ctypes
+
+        gomp = ctypes.CDLL("libgomp.so.1")
+        gomp.omp_set_num_threads(1)
+        t1 = time.perf_counter()
+        n1 = 0
+        while n1 < 3 and (time.perf_counter() - t1) < 6.0:
+            orc.state_step_dense(x, v, freqs, 200 + n1, rho)
+            n1 += 1
+        one = B * n1 / (time.perf_counter() - t1)
+        gomp.omp_set_num_threads(threads)
+    except OSError:
+        pass
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "")
+    except OSError:
+        pass
     return {
         "value": B * steps / dt,
         "unit": "tokens/s",
         "cores": min(threads, B * h),
         "kind": "port",
         "sample": f"{steps} dense steps of the same config-2 shape (rho f32 [{B},{h},{N},{d}]), "
-                  f"C restatement of the reference op sequence, OpenMP over (b,h) slices, {dt / steps * 1e3:.1f} ms/step",
+                  f"C restatement of the reference op sequence (not a Burn binary), OpenMP over (b,h) slices, "
+                  f"{dt / steps * 1e3:.1f} ms/step"
+                  + (f"; on one thread {one:.0f} tokens/s" if one else "") + (f"; host CPU: {model}" if model else ""),
+        "value_one_thread": one,
     }
 
 
