@@ -16,6 +16,8 @@
 // kernel adds the partials in a fixed order (deterministic, no atomics).
 #include <hip/hip_bf16.h>
 
+#include <algorithm>
+
 #include "bdh_internal.h"
 
 namespace {
@@ -71,6 +73,10 @@ struct StepPtrs {
   unsigned long long *bitmask;  // token t of slice 0, or null
   long bitmask_slice_stride;
   int h, N, S;
+  // k_step_rope_f32 only: the launch walks nt consecutive tokens (each workgroup owns its state rows, so
+  // it can take the tokens one after the other without leaving the kernel); per-token element strides
+  int nt = 1;
+  long x_t_stride = 0, v_t_stride = 0, partial_t_stride = 0, cnt_t_stride = 0, bm_t_stride = 0;
 };
 
 // ------------------------------------------------------------------------------------
@@ -79,7 +85,7 @@ struct StepPtrs {
 // SPLIT > 1: the workgroup still has WAVES waves but owns only WAVES*64/SPLIT lane pairs; the
 // first WAVES/SPLIT waves compact them and all waves walk the list.  Used when there are few
 // (b,h) slices, so that a small batch still spreads over every CU with enough loads in flight.
-template <int D, int WAVES, int U, int SPLIT>
+template <int D, int WAVES, int U, int SPLIT, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float *__restrict__ rho) {
   constexpr int VPL = D / 256;             // float4 per lane per row
   constexpr int PPB = WAVES * 64 / SPLIT;  // lane pairs per workgroup
@@ -99,13 +105,18 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
   const int NP = a.N >> 1;
   const bool owner = wave < OW;
   const int p = seg * PPB + tid;
+  float2 fv = make_float2(0.0f, 0.0f);
 
-  float2 xv = make_float2(0.0f, 0.0f), fv = make_float2(0.0f, 0.0f);
-  if (owner && p < NP) {
-    xv = reinterpret_cast<const float2 *>(a.x + (long)slice * a.x_slice_stride)[p];
-    fv = reinterpret_cast<const float2 *>(a.freqs)[p];
+  // Tokens of this launch, in order.  A workgroup touches only its own state rows and its barriers
+  // order the row stores of one token before the row loads of the next.
+  const int nt = MULTI ? a.nt : 1;  // the single-token kernel keeps its straight-line code
+  for (int t = 0; t < nt; ++t) {
+  float2 xv = make_float2(0.0f, 0.0f);
+  if (owner && p < NP) {  // one block, so that both loads are in flight together
+    xv = reinterpret_cast<const float2 *>(a.x + t * a.x_t_stride + (long)slice * a.x_slice_stride)[p];
+    if (t == 0) fv = reinterpret_cast<const float2 *>(a.freqs)[p];
   }
-  const float pos = a.pos_dev ? (float)((long)a.pos_dev[b] + a.pos_add) : a.pos_scalar;
+  const float pos = (float)((a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int) + t);
 
   const bool ae = xv.x != 0.0f, ao = xv.y != 0.0f;
   const bool act = ae || ao;
@@ -117,7 +128,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
     if (lane == 0) {
       const int w0 = (seg * PPB + wave * 64) >> 5;
       const int NW = (a.N + 63) >> 6;
-      unsigned long long *bm = a.bitmask + (long)slice * a.bitmask_slice_stride;
+      unsigned long long *bm = a.bitmask + t * a.bm_t_stride + (long)slice * a.bitmask_slice_stride;
       if (w0 < NW) bm[w0] = spread_bits((unsigned int)me) | (spread_bits((unsigned int)mo) << 1);
       if (w0 + 1 < NW)
         bm[w0 + 1] = spread_bits((unsigned int)(me >> 32)) | (spread_bits((unsigned int)(mo >> 32)) << 1);
@@ -163,7 +174,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
   float4 acc[VPL];
   float4 vv[VPL];
   {
-    const float4 *vrow = reinterpret_cast<const float4 *>(a.v + (long)b * a.v_batch_stride);
+    const float4 *vrow = reinterpret_cast<const float4 *>(a.v + t * a.v_t_stride + (long)b * a.v_batch_stride);
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -226,7 +237,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
 #pragma unroll
   for (int j = 0; j < VPL; ++j) s_red[wave][j * 64 + lane] = acc[j];
   __syncthreads();
-  float *pout = a.partial + (long)blockIdx.x * D;
+  float *pout = a.partial + t * a.partial_t_stride + (long)blockIdx.x * D;
   for (int c4 = tid; c4 < D / 4; c4 += WAVES * 64) {
     float4 s = s_red[0][c4];
 #pragma unroll
@@ -236,7 +247,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_f32(StepPtrs a, float 
     }
     reinterpret_cast<float4 *>(pout)[c4] = s;
   }
-  if (tid == 0) a.pair_cnt[blockIdx.x] = total;
+  if (tid == 0) a.pair_cnt[t * a.cnt_t_stride + blockIdx.x] = total;
+  }  // tokens
 }
 
 // ------------------------------------------------------------------------------------
@@ -717,9 +729,17 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
                                                        const int *__restrict__ pair_cnt, int S, int d,
                                                        float *__restrict__ out, long out_slice_stride,
                                                        float *__restrict__ out_ln, int *__restrict__ rows,
-                                                       long rows_slice_stride, int rows_per_count) {
+                                                       long rows_slice_stride, int rows_per_count,
+                                                       long partial_t_stride, long cnt_t_stride) {
   const int tid = threadIdx.x;
   const int slice = blockIdx.x;
+  // blockIdx.y = token of a multi-token launch: partials and counts advance by their per-token
+  // strides, the outputs by one row of d (tokens are adjacent in out [slices, T, d] and rows [slices, T])
+  partial += blockIdx.y * partial_t_stride;
+  if (pair_cnt) pair_cnt += blockIdx.y * cnt_t_stride;
+  out += (long)blockIdx.y * d;
+  if (LN) out_ln += (long)blockIdx.y * d;
+  if (rows) rows += blockIdx.y;
   const float *p = partial + (long)slice * S * d;
   float vals[4];  // d <= 1024
   float lsum = 0.0f;
@@ -776,13 +796,14 @@ __global__ __launch_bounds__(256) void k_step_finalize(const float *__restrict__
 }
 
 void launch_finalize(hipStream_t st, int slices, const float *partial, const int *pair_cnt, int S, int d, float *out,
-                     long out_stride, float *out_ln, int *rows, long rows_stride, int rows_per_count = 2) {
+                     long out_stride, float *out_ln, int *rows, long rows_stride, int rows_per_count = 2, int nt = 1,
+                     long partial_t_stride = 0, long cnt_t_stride = 0) {
   if (out_ln)
-    hipLaunchKernelGGL(k_step_finalize<true>, dim3(slices), dim3(256), 0, st, partial, pair_cnt, S, d, out, out_stride,
-                       out_ln, rows, rows_stride, rows_per_count);
+    hipLaunchKernelGGL(k_step_finalize<true>, dim3(slices, nt), dim3(256), 0, st, partial, pair_cnt, S, d, out,
+                       out_stride, out_ln, rows, rows_stride, rows_per_count, partial_t_stride, cnt_t_stride);
   else
-    hipLaunchKernelGGL(k_step_finalize<false>, dim3(slices), dim3(256), 0, st, partial, pair_cnt, S, d, out,
-                       out_stride, out_ln, rows, rows_stride, rows_per_count);
+    hipLaunchKernelGGL(k_step_finalize<false>, dim3(slices, nt), dim3(256), 0, st, partial, pair_cnt, S, d, out,
+                       out_stride, out_ln, rows, rows_stride, rows_per_count, partial_t_stride, cnt_t_stride);
 }
 
 __global__ __launch_bounds__(256) void k_fill_zero_u32(uint32_t *__restrict__ p, size_t n) {
@@ -792,7 +813,10 @@ __global__ __launch_bounds__(256) void k_fill_zero_u32(uint32_t *__restrict__ p,
 
 template <int D, int WAVES, int U, int SPLIT>
 void launch_fast(hipStream_t st, int blocks, const StepPtrs &a, float *rho) {
-  hipLaunchKernelGGL((k_step_rope_f32<D, WAVES, U, SPLIT>), dim3(blocks), dim3(WAVES * 64), 0, st, a, rho);
+  if (a.nt > 1)
+    hipLaunchKernelGGL((k_step_rope_f32<D, WAVES, U, SPLIT, true>), dim3(blocks), dim3(WAVES * 64), 0, st, a, rho);
+  else
+    hipLaunchKernelGGL((k_step_rope_f32<D, WAVES, U, SPLIT, false>), dim3(blocks), dim3(WAVES * 64), 0, st, a, rho);
 }
 
 }  // namespace
@@ -812,7 +836,8 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
                                                        : (long)slices * (((N / 2) + 255) / 256) < 2L * n_cu);
   const int ppb = split ? 64 : 256;
   // lazily decayed ALiBi state, f32, d in {256,512}: row-compaction kernel, 512 neurons per workgroup
-  const bool fast_lazy = p.rotary == BDH_ALIBI && p.stamps && p.rho_dtype == BDH_F32 && (d == 256 || d == 512);
+  const bool fast_lazy = p.rotary == BDH_ALIBI && p.stamps && p.rho_dtype == BDH_F32 && (d == 256 || d == 512) &&
+                         (N % 2 == 0);  // the kernel reads x two neurons at a time
   const int S = fast ? ((N / 2) + ppb - 1) / ppb : fast_lazy ? (N + 511) / 512 : (Nq + kGenRows - 1) / kGenRows;
   if (N == 0 || d == 0) {
     // nothing to read or update: the readout is an empty sum
@@ -831,8 +856,14 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
     }
     return BDH_OK;
   }
-  const size_t partial_bytes = bdh_align_up(sizeof(float) * (size_t)slices * S * d, 256);
-  const size_t cnt_bytes = bdh_align_up(sizeof(int) * (size_t)slices * S, 256);
+  // tokens per launch: only the f32 RoPE kernel walks several, as many as 64 MiB of partials allow
+  const size_t partial_one = bdh_align_up(sizeof(float) * (size_t)slices * S * d, 256);
+  const size_t cnt_one = bdh_align_up(sizeof(int) * (size_t)slices * S, 256);
+  int group = 1;
+  if (fast && p.rho_dtype == BDH_F32 && T > 1)
+    group = (int)std::max<size_t>(1, std::min<size_t>((size_t)T, (size_t(64) << 20) / partial_one));
+  const size_t partial_bytes = partial_one * group;
+  const size_t cnt_bytes = cnt_one * group;
   int rc = bdh_ws_reserve(ctx, partial_bytes + cnt_bytes);
   if (rc != BDH_OK) return rc;
   float *partial = static_cast<float *>(ctx->ws);
@@ -850,8 +881,15 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   if (p.stamps && p.rotary != BDH_ALIBI) return bdh_fail(ctx, BDH_E_INVAL, "decay stamps only apply to ALiBi");
 
   const int NW = (N + 63) / 64;
-  for (int t = 0; t < T; ++t) {
+  for (int t = 0; t < T; t += group) {
+    const int nt = std::min(group, T - t);
     StepPtrs a{};
+    a.nt = nt;
+    a.x_t_stride = N;
+    a.v_t_stride = d;
+    a.partial_t_stride = (long)(partial_one / sizeof(float));
+    a.cnt_t_stride = (long)(cnt_one / sizeof(int));
+    a.bm_t_stride = NW;
     a.x = p.x + (long)t * N;
     a.x_slice_stride = (long)T * N;
     a.v = p.v + (long)t * d;
@@ -891,7 +929,8 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
           hipLaunchKernelGGL((k_step_rope_bf16<512, 8, 2, 8>), dim3(blocks), dim3(512), 0, ctx->stream, a, rho);
       }
       BDH_LAUNCH_CHECK(ctx, "k_step_rope");
-      launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T);
+      launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T, 2, nt,
+                      a.partial_t_stride, a.cnt_t_stride);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
     } else if (fast_lazy) {
       float *rho = static_cast<float *>(p.rho);
