@@ -122,6 +122,7 @@ struct FsaArgs {
   int lda, ldb, ldc, M, N, K;
   int b_div;        // B slice = slice / b_div
   int n_slices;
+  int mt, nt;       // tile grid (rows, columns) of one slice
   // scores epilogue
   int block_size, tb, h, use_alibi, dense;
   const unsigned char *active;  // [tb*tb] when !dense
@@ -152,8 +153,15 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
   static_assert(CA >= 1 && CB >= 1 && CA * NT == BM * 4 && CB * NT == BN * 4, "tile does not divide over the threads");
   __shared__ __attribute__((aligned(16))) float s_a[BM * FLD];
   __shared__ __attribute__((aligned(16))) float s_b[BN * FLD];
-  const int slice = blockIdx.z;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  // XCD-aware mapping: workgroup ids are dealt round-robin to the 8 XCDs, so ids with the same
+  // (id % 8) share an L2; all tiles of one slice go to one XCD and reuse its operand rows there.
+  const int xcd = blockIdx.x & 7;
+  const int rr = blockIdx.x >> 3;
+  const int tiles = g.mt * g.nt;
+  const int slice = xcd + 8 * (rr / tiles);
+  if (slice >= g.n_slices) return;
+  const int tile = rr % tiles;
+  const int m0 = (tile / g.nt) * BM, n0 = (tile % g.nt) * BN;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / NWN, wn = wave % NWN;
   const float *A = g.A + (long)slice * g.a_batch;
@@ -338,7 +346,7 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
   int path = ctx->opt_fsa_path;  // -1 choose, 0 row kernel, 1 matrix cores
   if (path < 0) path = T >= 128 ? 1 : 0;
   if (path == 0 && lds > 150 * 1024) path = 1;
-  if (S * T > 0x7fffffffL || S > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "B*h*T too large");
+  if (S * T > 0x7fffffffL || (S + 7) / 8 * 8 * (long)(((T + 127) / 128) * ((T + 127) / 128)) > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "B*h*T too large");
 
   const int Tp = (T + 3) & ~3;  // row stride of the score matrix
   const size_t q_bytes = bdh_align_up(sizeof(float) * (size_t)S * T * Nq, 256);
@@ -377,13 +385,14 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     g.active = active; g.slopes = slopes_dev; g.norm = nullptr;
     // big tiles once there are enough of them to cover the chip; small ones for short sequences
     const bool big = (long)S * ((T + 255) / 256) * ((T + 255) / 256) >= 256;
+    const unsigned groups = (unsigned)((S + 7) / 8);
     if (big) {
-      const int tiles = (T + 255) / 256;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 256, 256, 2, 4>), dim3(tiles, tiles, (unsigned)S), dim3(512), 0,
+      g.mt = g.nt = (T + 255) / 256;
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 256, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512), 0,
                          ctx->stream, g);
     } else {
-      const int tiles = (T + 127) / 128;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 128, 128, 2, 2>), dim3(tiles, tiles, (unsigned)S), dim3(256), 0,
+      g.mt = g.nt = (T + 127) / 128;
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
                          ctx->stream, g);
     }
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<scores>");
@@ -398,8 +407,10 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     o.lda = Tp; o.ldb = dv; o.ldc = dv; o.M = T; o.N = dv; o.K = T; o.b_div = h; o.n_slices = (int)S;
     o.block_size = block_size; o.tb = tb; o.h = h; o.dense = sparse ? 0 : 1;
     o.norm = row_normalize ? norm : nullptr;
-    hipLaunchKernelGGL((k_fsa_gemm_f32<1, true, 128, 128, 2, 2>), dim3((dv + 127) / 128, (T + 127) / 128, (unsigned)S),
-                       dim3(256), 0, ctx->stream, o);
+    o.mt = (T + 127) / 128;
+    o.nt = (dv + 127) / 128;
+    hipLaunchKernelGGL((k_fsa_gemm_f32<1, true, 128, 128, 2, 2>), dim3(8 * groups * o.mt * o.nt), dim3(256), 0,
+                       ctx->stream, o);
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<out>");
     return BDH_OK;
   }
