@@ -352,11 +352,14 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
     pa[c] = A + (long)(m0 + bi * 8 + lr) * g.lda + lc * 8;
     pb[c] = Bh + (long)(n0 + bi * 8 + lr) * g.ldb + lc * 8;
   }
+  // scores: A and B are the same matrix, so a tile on the diagonal needs its rows only once
+  const bool same_ab = EPI == EPI_SCORES && g.tri && ti == tj && g.A == g.B && g.b_div == 1;
 #define BDH_ISSUE_TILE(buf, k0)                                                                              \
   _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                            \
     const int bi = c * 8 + wave;                                                                             \
     __builtin_amdgcn_global_load_lds((gptr_t)(pa[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + bi * 512), 16, 0, 0);        \
-    __builtin_amdgcn_global_load_lds((gptr_t)(pb[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, 0); \
+    if (!same_ab)                                                                                            \
+      __builtin_amdgcn_global_load_lds((gptr_t)(pb[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, 0); \
   }
   BDH_ISSUE_TILE(0, 0)
   __builtin_amdgcn_s_waitcnt(0);
@@ -364,7 +367,7 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
   int cur = 0;
   for (int k0 = 0; k0 < K; k0 += BK) {
     if (k0 + BK < K) { BDH_ISSUE_TILE(cur ^ 1, k0 + BK) }  // lands while the matrix cores work on this tile
-    const unsigned short *sa = s_dyn + cur * BUF, *sb = sa + TILE;
+    const unsigned short *sa = s_dyn + cur * BUF, *sb = same_ab ? sa : sa + TILE;
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 16) {
       bf16x8 fa[4], fb[2];
