@@ -93,3 +93,26 @@ def test_sampler_index_is_in_range_and_monotone_in_the_variate(corc, seed, V, k,
     assert abs(float(p.sum()) - 1) < 1e-4 and all(p[i] > 0 for i in idx)
     if 0 < k < V:
         assert (p > 0).sum() >= k  # ties with the k-th largest survive
+
+
+@FAST
+@given(data=st.data())
+def test_damaged_record_framing_fails_cleanly(data):
+    """Random byte edits in the framing of a small record: the reader returns or raises RecordError,
+    never another exception (no index errors, no huge allocations)."""
+    rng = np.random.default_rng(0)
+    w = {"embed": rng.standard_normal((5, 4)), "encoder": rng.standard_normal((2, 4, 6)),
+         "encoder_v": rng.standard_normal((2, 4, 6)), "decoder": rng.standard_normal((12, 4)),
+         "lm_head": rng.standard_normal((4, 5))}
+    buf = bytearray(record.serialize_record({k: a.astype(np.float32) for k, a in w.items()}))
+    n_edits = data.draw(st.integers(1, 4))
+    for _ in range(n_edits):
+        pos = data.draw(st.integers(0, len(buf) - 1))
+        buf[pos] = data.draw(st.integers(0, 255))
+    if data.draw(st.booleans()):
+        del buf[data.draw(st.integers(0, len(buf) - 1)):]
+    try:
+        _, params = record.parse_record(bytes(buf))
+        record.weights_from_params(params)
+    except record.RecordError:
+        pass
