@@ -60,25 +60,33 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint4 *__restrict__ x, 
     const float ph = (raw - floorf(raw)) * kTwoPi;
     sincosf(ph, &sn[e], &cs[e]);
   }
-  for (int s = 0; s < S; ++s) {
-    const long off = ((long)s * T + t) * groups + g;
-    const uint4 in = x[off];
-    uint4 out = make_uint4(0u, 0u, 0u, 0u);
-    if (in.x | in.y | in.z | in.w) {
-      const unsigned int w[4] = {in.x, in.y, in.z, in.w};
-      unsigned int o[4];
+  auto rotate = [&](const uint4 in) -> uint4 {
+    if (!(in.x | in.y | in.z | in.w)) return make_uint4(0u, 0u, 0u, 0u);
+    const unsigned int w[4] = {in.x, in.y, in.z, in.w};
+    unsigned int o[4];
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        const float xe = bf16_bits_to_f32((unsigned short)(w[p] & 0xffffu));
-        const float xo = bf16_bits_to_f32((unsigned short)(w[p] >> 16));
-        // q[2j] = x[2j] cos + (-x[2j+1]) sin ; q[2j+1] = x[2j+1] cos + x[2j] sin  (attention.rs:305-321)
-        const float a0 = xe * cs[2 * p], r0 = (-xo) * sn[2 * p];
-        const float a1 = xo * cs[2 * p + 1], r1 = xe * sn[2 * p + 1];
-        o[p] = (unsigned int)f32_to_bf16_bits(a0 + r0) | ((unsigned int)f32_to_bf16_bits(a1 + r1) << 16);
-      }
-      out = make_uint4(o[0], o[1], o[2], o[3]);
+    for (int p = 0; p < 4; ++p) {
+      const float xe = bf16_bits_to_f32((unsigned short)(w[p] & 0xffffu));
+      const float xo = bf16_bits_to_f32((unsigned short)(w[p] >> 16));
+      // q[2j] = x[2j] cos + (-x[2j+1]) sin ; q[2j+1] = x[2j+1] cos + x[2j] sin  (attention.rs:305-321)
+      const float a0 = xe * cs[2 * p], r0 = (-xo) * sn[2 * p];
+      const float a1 = xo * cs[2 * p + 1], r1 = xe * sn[2 * p + 1];
+      o[p] = (unsigned int)f32_to_bf16_bits(a0 + r0) | ((unsigned int)f32_to_bf16_bits(a1 + r1) << 16);
     }
-    q[off] = out;
+    return make_uint4(o[0], o[1], o[2], o[3]);
+  };
+  // eight slices at a time: the loads are issued together, so eight requests per thread are in flight
+  int s = 0;
+  for (; s + 8 <= S; s += 8) {
+    uint4 in[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) in[u] = x[((long)(s + u) * T + t) * groups + g];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) q[((long)(s + u) * T + t) * groups + g] = rotate(in[u]);
+  }
+  for (; s < S; ++s) {
+    const long off = ((long)s * T + t) * groups + g;
+    q[off] = rotate(x[off]);
   }
 }
 
