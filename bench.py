@@ -393,6 +393,8 @@ def main():
     ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
     ap.add_argument("--graph", action="store_true", help="model: replay one captured HIP graph per token")
     ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library launch-shape option set on the context before the run (repeatable)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); use --gpus 1",
@@ -410,6 +412,9 @@ def main():
     from burn_dragon_amd.positional import RotaryEmbedding
 
     dev = torch.device("cuda:0")
+    for item in args.option:
+        name, _, value = item.partition("=")
+        ffi.default_context(0).set_option(name, int(value))
     if args.workload == "prefill":
         return bench_prefill(args)
     if args.workload == "model":
