@@ -221,6 +221,27 @@ int bdh_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, int64_t cloc
   return bdh_launch_alibi_materialize(ctx, B, h, N, d, slopes, clock, clocks_dev, rho, rho_dtype, stamps);
 }
 
+int bdh_rho_energy(bdh_ctx *ctx, int B, int h, int N, int d, const void *rho, int rho_dtype,
+                   const int32_t *stamps, int64_t clock, const int32_t *clocks_dev,
+                   const float *alibi_slopes_host, float *out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (B < 0 || h < 0 || N < 0 || d < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
+  if (h > 64) return bdh_fail(ctx, BDH_E_SHAPE, "n_head %d > 64", h);
+  if (rho_dtype != BDH_F32 && rho_dtype != BDH_BF16) return bdh_fail(ctx, BDH_E_INVAL, "bad rho_dtype");
+  if (stamps && (clock < 0 || clock > 0x7fffffffLL))
+    return bdh_fail(ctx, BDH_E_INVAL, "clock outside the 31-bit stamp range");
+  if (h == 0 || N == 0) return BDH_OK;
+  if (!out || (!rho && B > 0 && d > 0)) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  float slopes[64] = {0};
+  if (stamps) {
+    if (alibi_slopes_host)
+      memcpy(slopes, alibi_slopes_host, sizeof(float) * h);
+    else
+      bdh_default_alibi_slopes(h, slopes);
+  }
+  return bdh_launch_rho_energy(ctx, B, h, N, d, rho, rho_dtype, stamps, slopes, clock, clocks_dev, 0, out);
+}
+
 int bdh_state_step(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const float *x,
                    const float *v, const float *freqs, int64_t position,
                    const int32_t *positions_dev, const float *alibi_slopes_host, void *rho,

@@ -107,3 +107,13 @@ int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cu
                        const float *lm_head, float *logits, int64_t *next_tokens);
 // positions[b] = min(positions[b] + delta, INT32_MAX): the device-side form of state.position += T
 int bdh_launch_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta);
+
+// viz_taps.hip: out[h,N] = batch mean of the per-row mean |rho| (src/model/bdh.rs:411-419); with stamps the
+// state is read through its pending ALiBi decay at clock (or clocks_dev[b] + clock_add)
+int bdh_launch_rho_energy(bdh_ctx *ctx, int B, int h, int N, int d, const void *rho, int rho_dtype,
+                          const int32_t *stamps, const float *slopes_host, int64_t clock, const int32_t *clocks_dev,
+                          int clock_add, float *out);
+// dst[hh, 0..cols) = src[hh * head_stride + offset + (0..cols)]
+int bdh_launch_gather_head_rows(bdh_ctx *ctx, const float *src, int h, long head_stride, long offset, int cols,
+                                float *dst);
+int bdh_launch_fill_zero_f32(bdh_ctx *ctx, float *p, long n);

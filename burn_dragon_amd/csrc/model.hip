@@ -109,6 +109,13 @@ int bdh_model_forward_ex(bdh_model *m, const int64_t *tokens, int B, int T, void
 int bdh_model_forward_lazy(bdh_model *m, const int64_t *tokens, int B, int T, void *rho, int rho_dtype,
                            int32_t *stamps, int64_t position, const int32_t *positions_dev, float *logits,
                            int64_t *next_tokens, float *x_tap) {
+  return bdh_model_forward_viz(m, tokens, B, T, rho, rho_dtype, stamps, position, positions_dev, logits, next_tokens,
+                               x_tap, nullptr);
+}
+
+int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, void *rho, int rho_dtype,
+                          int32_t *stamps, int64_t position, const int32_t *positions_dev, float *logits,
+                          int64_t *next_tokens, float *x_tap, float *viz) {
   if (!m) return BDH_E_INVAL;
   bdh_ctx *ctx = m->ctx;
   if (stamps && m->cfg.rotary != BDH_ALIBI)
@@ -125,15 +132,17 @@ int bdh_model_forward_lazy(bdh_model *m, const int64_t *tokens, int B, int T, vo
   const size_t Nq = c.rotary == BDH_POPE ? 2 * (size_t)N : (size_t)N;
   const size_t M = (size_t)B * T;
 
-  // activation scratch: cur [M,d] | x [B,h,T,N] | xy [B,h,T,N] | attn [B,h,T,d] | attn_ln [B,h,T,d]
+  // activation scratch: cur [M,d] | x [B,h,T,N] | xy [B,h,T,N] | attn [B,h,T,d] | attn_ln [B,h,T,d] | last [h,d]
   const size_t n_cur = bdh_align_up(M * d, 64), n_x = bdh_align_up(M * h * N, 64), n_a = bdh_align_up(M * h * d, 64);
-  int rc = ensure_act(m, sizeof(float) * (n_cur + 2 * n_x + 2 * n_a));
+  const size_t n_last = viz ? bdh_align_up((size_t)h * d, 64) : 0;
+  int rc = ensure_act(m, sizeof(float) * (n_cur + 2 * n_x + 2 * n_a + n_last));
   if (rc != BDH_OK) return rc;
   float *cur = static_cast<float *>(m->act);
   float *x = cur + n_cur;
   float *xy = x + n_x;
   float *attn = xy + n_x;
   float *attn_ln = attn + n_a;
+  float *last = attn_ln + n_a;
 
   rc = bdh_launch_embed_ln(ctx, tokens, (int64_t)M, d, V, m->w.embed, cur);  // :319-322
   if (rc != BDH_OK) return rc;
@@ -155,6 +164,28 @@ int bdh_model_forward_lazy(bdh_model *m, const int64_t *tokens, int B, int T, vo
     ReluLowrankParams py{B, h, T, d, h, N, attn_ln, m->w.encoder_v, nullptr, c.relu_threshold, 1, nullptr, 0, x_l, xy};
     rc = bdh_launch_relu_lowrank(ctx, py);
     if (rc != BDH_OK) return rc;
+    if (viz) {  // :386-434: first sequence, last token; the state is already this call's updated one
+      float *vz = viz + (size_t)l * 4 * h * N;
+      const long hs = (long)T * N, off = (long)(T - 1) * N;
+      rc = bdh_launch_gather_head_rows(ctx, x_l, h, hs, off, N, vz);
+      if (rc != BDH_OK) return rc;
+      // y alone is never stored (the gate is fused into the D_y kernel): one more D_y pass over the h rows
+      rc = bdh_launch_gather_head_rows(ctx, attn_ln, h, (long)T * d, (long)(T - 1) * d, d, last);
+      if (rc != BDH_OK) return rc;
+      ReluLowrankParams pv{1, h, 1, d, h, N, last, m->w.encoder_v, nullptr, c.relu_threshold, 1, nullptr, 0, nullptr,
+                           vz + (size_t)h * N};
+      rc = bdh_launch_relu_lowrank(ctx, pv);
+      if (rc != BDH_OK) return rc;
+      rc = bdh_launch_gather_head_rows(ctx, xy, h, hs, off, N, vz + (size_t)2 * h * N);
+      if (rc != BDH_OK) return rc;
+      if (Nq == (size_t)N)
+        rc = bdh_launch_rho_energy(ctx, B, h, N, d, static_cast<char *>(rho) + (size_t)l * rho_layer_bytes, rho_dtype,
+                                   stamps ? stamps + (size_t)l * B * h * N : nullptr, m->slopes, position + T,
+                                   positions_dev, T, vz + (size_t)3 * h * N);
+      else  // PoPE: the state has 2N rows, the reference stores a zero map (:413-424)
+        rc = bdh_launch_fill_zero_f32(ctx, vz + (size_t)3 * h * N, (long)h * N);
+      if (rc != BDH_OK) return rc;
+    }
     // :383,436-441  cur = LN(cur + LN(mixed . decoder))
     rc = bdh_launch_decoder_residual(ctx, B, T, h, N, d, xy, m->w.decoder, cur);
     if (rc != BDH_OK) return rc;

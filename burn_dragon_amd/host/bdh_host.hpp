@@ -299,8 +299,19 @@ inline BDHConfig build_model_config(const ModelOverrides &o, size_t training_blo
 }
 
 // ---- model::state ---------------------------------------------------------------------
+// src/model/state.rs:17-24 (the reference's "viz" feature): [h,N] maps on the host
+struct LayerVizState {
+  std::vector<float> x_last, y_last, xy_last, rho_last;
+};
+
 struct LayerState {
   std::optional<Tensor> rho;  // [B,h,Nq,d]
+  std::optional<LayerVizState> viz;
+  std::optional<LayerVizState> take_viz() {  // src/model/state.rs:76-80
+    std::optional<LayerVizState> out;
+    out.swap(viz);
+    return out;
+  }
 };
 
 struct ModelState {
@@ -317,6 +328,14 @@ struct ModelState {
   size_t len() const { return position; }
   bool is_empty() const { return position == 0; }
   void trim(size_t) {}  // a no-op in the reference (src/model/state.rs:55-57)
+  std::vector<std::optional<LayerVizState>> take_viz() {  // src/model/state.rs:59-65
+    std::vector<std::optional<LayerVizState>> out;
+    for (auto &l : layers) out.push_back(l.take_viz());
+    return out;
+  }
+  void clear_viz() {  // src/model/state.rs:67-72
+    for (auto &l : layers) l.viz.reset();
+  }
 };
 
 // ---- model::BDH -------------------------------------------------------------------------
@@ -346,8 +365,9 @@ class BDH {
   ModelState init_state() const { return ModelState(config_.n_layer); }
 
   // tokens [B,T] (host, row-major) -> logits [B,T,V]
+  // viz = true also fills every layer's LayerVizState (src/model/bdh.rs:386-434)
   Tensor forward_with_state(const std::vector<int64_t> &tokens, size_t batch, size_t time, ModelState &state,
-                            std::vector<int64_t> *next_tokens = nullptr) {
+                            std::vector<int64_t> *next_tokens = nullptr, bool viz = false) {
     if (state.layers.size() != config_.n_layer) throw std::logic_error("model state layers mismatch");
     if (tokens.size() != batch * time) throw std::logic_error("tokens do not match [batch, time]");
     const size_t h = config_.n_head, d = config_.n_embd, N = config_.latent_per_head();
@@ -361,8 +381,21 @@ class BDH {
     int rc = BDH_OK;
     if (!tokens.empty()) {
       hip_check(hipMemcpy(tok_dev, tokens.data(), sizeof(int64_t) * tokens.size(), hipMemcpyHostToDevice), "hipMemcpy");
-      rc = bdh_model_forward(model_, tok_dev, (int)batch, (int)time, state.storage->data(), BDH_F32,
-                             (int64_t)state.position, logits.data(), next_tokens ? next_dev : nullptr, nullptr);
+      std::optional<Tensor> maps;
+      if (viz) maps.emplace(std::vector<size_t>{config_.n_layer, 4, h, N});
+      rc = bdh_model_forward_viz(model_, tok_dev, (int)batch, (int)time, state.storage->data(), BDH_F32, nullptr,
+                                 (int64_t)state.position, nullptr, logits.data(), next_tokens ? next_dev : nullptr,
+                                 nullptr, maps ? maps->data() : nullptr);
+      if (rc == BDH_OK && maps) {
+        ctx_.synchronize();
+        const std::vector<float> host = maps->to_host();
+        const size_t hn = h * N;
+        for (size_t l = 0; l < config_.n_layer; ++l) {
+          const float *p = host.data() + l * 4 * hn;
+          state.layers[l].viz = LayerVizState{{p, p + hn}, {p + hn, p + 2 * hn}, {p + 2 * hn, p + 3 * hn},
+                                              {p + 3 * hn, p + 4 * hn}};
+        }
+      }
     }
     if (rc == BDH_OK && next_tokens && batch > 0 && time > 0) {
       next_tokens->resize(batch);

@@ -1,5 +1,5 @@
 from .bdh import BDH, DecodeGraph
 from .config import BDHConfig, FusedKernelConfig
-from .state import LayerState, ModelState
+from .state import LayerState, LayerVizState, ModelState
 
-__all__ = ["BDH", "DecodeGraph", "BDHConfig", "FusedKernelConfig", "LayerState", "ModelState"]
+__all__ = ["BDH", "DecodeGraph", "BDHConfig", "FusedKernelConfig", "LayerState", "LayerVizState", "ModelState"]

@@ -15,7 +15,7 @@ import torch
 from .. import ffi
 from ..positional import RotaryEmbedding
 from .config import BDHConfig
-from .state import LayerState, ModelState
+from .state import LayerState, LayerVizState, ModelState
 
 UINT63_MAX = (1 << 63) - 1
 
@@ -120,18 +120,26 @@ class BDH:
         alibi_materialize(state.storage, state.stamps, state.position, self._slopes, None, self.ctx)
 
     def forward_with_state(self, tokens: torch.Tensor, state: ModelState, want_next: bool = False,
-                           x_tap: Optional[torch.Tensor] = None):
+                           x_tap: Optional[torch.Tensor] = None, viz: bool = False):
         """src/model/bdh.rs:309-450.  tokens [B,T] int64 -> logits [B,T,V] (and the greedy next
-        token per sequence, kept on the device, when want_next)."""
+        token per sequence, kept on the device, when want_next).  viz=True also fills every
+        layer's LayerVizState as the reference does when built with its "viz" feature (:386-434)."""
         assert len(state.layers) == self.n_layer, "model state layers mismatch"  # :314-318
         tokens = tokens.to(self.device, torch.int64).contiguous()
         B, T = tokens.shape
         rho = self._ensure_state(state, B)
         logits = torch.empty((B, T, self.vocab_size), device=self.device, dtype=torch.float32)
         nxt = torch.empty((B,), device=self.device, dtype=torch.int64) if want_next else None
-        self.ctx.check(self.ctx.lib.bdh_model_forward_lazy(self.handle, tokens.data_ptr(), B, T, rho.data_ptr(),
-                                                           self.rho_dtype, ffi.ptr(state.stamps), state.position,
-                                                           None, logits.data_ptr(), ffi.ptr(nxt), ffi.ptr(x_tap)))
+        maps = None
+        if viz and T > 0:
+            maps = torch.empty((self.n_layer, 4, self.n_head, self.latent), device=self.device, dtype=torch.float32)
+        self.ctx.check(self.ctx.lib.bdh_model_forward_viz(self.handle, tokens.data_ptr(), B, T, rho.data_ptr(),
+                                                          self.rho_dtype, ffi.ptr(state.stamps), state.position,
+                                                          None, logits.data_ptr(), ffi.ptr(nxt), ffi.ptr(x_tap),
+                                                          ffi.ptr(maps)))
+        if maps is not None:
+            for layer, m in zip(state.layers, maps):
+                layer.viz = LayerVizState(x_last=m[0], y_last=m[1], xy_last=m[2], rho_last=m[3])
         state.position = min(state.position + T, UINT63_MAX)  # saturating_add, :445
         return (logits, nxt) if want_next else logits
 

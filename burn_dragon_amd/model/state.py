@@ -8,8 +8,25 @@ import torch
 
 
 @dataclass
+class LayerVizState:
+    """src/model/state.rs:17-24 (the reference's "viz" feature): [h,N] maps of the first sequence's last
+    token, and the energy map of the layer's state."""
+
+    x_last: torch.Tensor
+    y_last: torch.Tensor
+    xy_last: torch.Tensor
+    rho_last: torch.Tensor
+
+
+@dataclass
 class LayerState:
     rho: Optional[torch.Tensor] = None  # [B,h,Nq,d]
+    viz: Optional[LayerVizState] = None  # filled by BDH.forward_with_state(..., viz=True)
+
+    def take_viz(self) -> Optional[LayerVizState]:
+        """src/model/state.rs:76-80."""
+        viz, self.viz = self.viz, None
+        return viz
 
 
 @dataclass
@@ -41,6 +58,15 @@ class ModelState:
 
     def is_empty(self) -> bool:
         return self.position == 0
+
+    def take_viz(self) -> List[Optional[LayerVizState]]:
+        """src/model/state.rs:59-65."""
+        return [layer.take_viz() for layer in self.layers]
+
+    def clear_viz(self) -> None:
+        """src/model/state.rs:67-72."""
+        for layer in self.layers:
+            layer.viz = None
 
     def trim(self, max_len: int) -> None:
         """A no-op, as in the reference (src/model/state.rs:55-57)."""

@@ -91,6 +91,23 @@ def alibi_materialize(rho: torch.Tensor, stamps: torch.Tensor, clock: int, alibi
                                             ffi.ptr(rho), dt, ffi.ptr(stamps)))
 
 
+def rho_energy(rho: torch.Tensor, stamps: Optional[torch.Tensor] = None, clock: int = 0, alibi_slopes=None,
+               clocks: Optional[torch.Tensor] = None, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
+    """The energy map of a state, `rho_last` of LayerVizState (src/model/bdh.rs:411-419): rho [B,h,N,d]
+    -> [h,N], the batch mean of each row's mean |rho|.  With stamps [B,h,N] a lazily decayed ALiBi state is
+    read through its pending decay at `clock` (or the per-sequence device `clocks`)."""
+    ctx = ctx or ffi.default_context(rho.device.index or 0)
+    assert rho.dim() == 4 and rho.is_contiguous()
+    B, h, N, d = rho.shape
+    assert stamps is None or (stamps.is_contiguous() and stamps.dtype == torch.int32 and stamps.numel() == B * h * N)
+    dt = {torch.float32: ffi.F32, torch.bfloat16: ffi.BF16}[rho.dtype]
+    slopes = None if alibi_slopes is None else np.ascontiguousarray(alibi_slopes, np.float32)
+    out = torch.empty((h, N), device=rho.device, dtype=torch.float32)
+    ctx.check(ctx.lib.bdh_rho_energy(ctx.handle, B, h, N, d, ffi.ptr(rho), dt, ffi.ptr(stamps), int(clock),
+                                     ffi.ptr(clocks), ffi.ptr(slopes), ffi.ptr(out)))
+    return out
+
+
 def layer_norm(x: torch.Tensor, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
     """BDH::layer_norm (src/model/bdh.rs:86-89)."""
     ctx = ctx or ffi.default_context(x.device.index or 0)

@@ -276,6 +276,26 @@ int bdh_model_forward_lazy(bdh_model *model, const int64_t *tokens, int B, int T
                            const int32_t *positions_dev, float *logits, int64_t *next_tokens,
                            float *x_tap);
 
+/* The energy map of a state: out[h,N] = (sum over b of (sum over c of |rho[b,h,n,c]|) / d) / B, the
+ * `rho_last` of LayerVizState (src/model/bdh.rs:411-419, built under the reference's "viz" feature).
+ * rho [B,h,N,d] f32 or bf16.  stamps [B,h,N] (optional, ALiBi only) marks a lazily decayed state, read
+ * at `clock` (or clocks_dev[b], device int32 [B]) through its pending decay; alibi_slopes_host [h] as in
+ * bdh_recurrent_attention (NULL = default slopes), ignored without stamps. */
+int bdh_rho_energy(bdh_ctx *ctx, int B, int h, int N, int d, const void *rho, int rho_dtype,
+                   const int32_t *stamps, int64_t clock, const int32_t *clocks_dev,
+                   const float *alibi_slopes_host, float *out);
+
+/* bdh_model_forward_lazy that also fills the per-layer LayerVizState of the reference
+ * (src/model/state.rs:17-24, src/model/bdh.rs:386-434): viz [L,4,h,N] f32 receives, for every layer,
+ * x_last, y_last, xy_last (first sequence, last token of this call) and rho_last (bdh_rho_energy of the
+ * layer's updated state; all zeros for PoPE, whose state has 2N rows).  viz = NULL is exactly
+ * bdh_model_forward_lazy.  Costs one extra D_y pass over h rows and one dense read of the state per
+ * layer, so it is meant for the visualisation loop, not for throughput runs. */
+int bdh_model_forward_viz(bdh_model *model, const int64_t *tokens, int B, int T, void *rho,
+                          int rho_dtype, int32_t *stamps, int64_t position,
+                          const int32_t *positions_dev, float *logits, int64_t *next_tokens,
+                          float *x_tap, float *viz);
+
 /* Draws the next token of every sequence on the device.  Replaces the temperature division of
  * sample_next_token (src/generation.rs:117) and sample_from_logits_values (src/generation.rs:26-72),
  * which copy the logits to the host for every token: values = logits / temperature; with

@@ -55,6 +55,11 @@
  *                              for top_k = 1, draw frequencies (tests/test_oracle.py);
  *                              the reference's own draw uses thread_rng and cannot be
  *                              replayed
+ *   orc_rho_energy,            pinned: numpy float64 mean(|rho|) over d and the batch;
+ *   orc_forward_with_state_viz the other three taps are slices of x, y and x*y of the
+ *                              pinned forward pass, checked against the numpy
+ *                              restatement; PoPE gives a zero energy map (state rows
+ *                              2N != N, src/model/bdh.rs:413-424)
  */
 #include <math.h>
 #include <stddef.h>
@@ -437,9 +442,25 @@ typedef struct {
   const float *embed, *encoder, *encoder_v, *decoder, *lm_head;
 } orc_model;
 
-int orc_forward_with_state(const orc_model *m, const int64_t *tokens, int B, int T, float *rho,
-                           int64_t *position, float *logits, float *x_tap, float *attn_tap,
-                           int sparse_state) {
+/* src/model/bdh.rs:411-419: rho_energy[h,n] = mean over the batch of (sum_c |rho[b,h,n,c]|) / d.
+ * Sums run in index order; the batch mean is sum_dim(0) followed by div_scalar(batch). */
+void orc_rho_energy(const float *rho, int B, int h, int N, int d, float *out) {
+  for (int hh = 0; hh < h; ++hh)
+    for (int n = 0; n < N; ++n) {
+      float acc = 0.0f;
+      for (int b = 0; b < B; ++b) {
+        const float *row = rho + (((size_t)b * h + hh) * N + n) * (size_t)d;
+        float s = 0.0f;
+        for (int c = 0; c < d; ++c) s = s + fabsf(row[c]);
+        acc = acc + s / (float)d;
+      }
+      out[(size_t)hh * N + n] = acc / (float)B;
+    }
+}
+
+static int orc_forward_impl(const orc_model *m, const int64_t *tokens, int B, int T, float *rho,
+                            int64_t *position, float *logits, float *x_tap, float *attn_tap,
+                            int sparse_state, float *viz) {
   const int d = m->n_embd, h = m->n_head, N = m->latent, V = m->vocab, L = m->n_layer;
   const int Nq = m->rotary == ORC_POPE ? 2 * N : N;
   const size_t rows = (size_t)B * T;
@@ -504,6 +525,21 @@ int orc_forward_with_state(const orc_model *m, const int64_t *tokens, int B, int
           float *mr = mixed + ((size_t)b * T + t) * (size_t)h * N + (size_t)hh * N;
           for (int n = 0; n < N; ++n) mr[n] = xr[n] * yr[n];
         }
+    /* :386-434 (feature "viz"): x, y, x*y of the first sequence's last token, and the energy of
+     * the updated state (zeros when the state is not [B,h,N,d], i.e. for PoPE's 2N rows) */
+    if (viz && T > 0) {
+      float *vz = viz + (size_t)l * 4 * h * N;
+      for (int hh = 0; hh < h; ++hh) {
+        const size_t src = ((size_t)hh * T + (T - 1)) * N; /* b = 0 */
+        memcpy(vz + (size_t)hh * N, x + src, sizeof(float) * N);
+        memcpy(vz + (size_t)(h + hh) * N, y + src, sizeof(float) * N);
+        for (int n = 0; n < N; ++n) vz[(size_t)(2 * h + hh) * N + n] = x[src + n] * y[src + n];
+      }
+      if (Nq == N)
+        orc_rho_energy(rho_l, B, h, N, d, vz + (size_t)3 * h * N);
+      else
+        memset(vz + (size_t)3 * h * N, 0, sizeof(float) * (size_t)h * N);
+    }
     /* :438 mlp = mixed . decoder */
 #pragma omp parallel for
     for (int64_t r = 0; r < (int64_t)rows; ++r)
@@ -524,6 +560,19 @@ int orc_forward_with_state(const orc_model *m, const int64_t *tokens, int B, int
   free(freqs); free(slopes); free(decay); free(cur); free(tmp); free(x); free(y); free(q);
   free(attn); free(attn_ln); free(mixed); free(mlp);
   return 0;
+}
+
+int orc_forward_with_state(const orc_model *m, const int64_t *tokens, int B, int T, float *rho,
+                           int64_t *position, float *logits, float *x_tap, float *attn_tap,
+                           int sparse_state) {
+  return orc_forward_impl(m, tokens, B, T, rho, position, logits, x_tap, attn_tap, sparse_state, NULL);
+}
+
+/* forward_with_state built with the reference's "viz" feature: viz [L,4,h,N] receives, per layer,
+ * x_last, y_last, xy_last and rho_last of LayerVizState (src/model/state.rs:17-24). */
+int orc_forward_with_state_viz(const orc_model *m, const int64_t *tokens, int B, int T, float *rho,
+                               int64_t *position, float *logits, int sparse_state, float *viz) {
+  return orc_forward_impl(m, tokens, B, T, rho, position, logits, NULL, NULL, sparse_state, viz);
 }
 
 /* src/generation.rs:26-72 with top_k = Some(1): everything below the maximum is

@@ -303,11 +303,22 @@ def forward_with_state(shape: BDHShape, w: BDHWeights, tokens, state: ModelState
         attn = layer_norm(attn)  # :359
         y = relu_lowrank(attn, w.encoder_v, None, shape.relu_threshold)  # :361-375
         xy = x * y  # :380
+        if taps is not None and T > 0:  # :386-434, feature "viz"
+            taps.setdefault("viz", []).append(dict(
+                x_last=x[0, :, T - 1], y_last=y[0, :, T - 1], xy_last=xy[0, :, T - 1],
+                rho_last=rho_energy(rho) if Nq == N else np.zeros((h, N), dtype)))
         mixed = np.swapaxes(xy, 1, 2).reshape(B * T, h * N)  # :383, :436
         mlp = layer_norm(np.matmul(mixed, w.decoder).reshape(B, 1, T, d))  # :438-440
         cur = layer_norm(cur + mlp)  # :441
     state.position = state.position + T  # :445
     return np.matmul(cur.reshape(B * T, d), w.lm_head).reshape(B, T, shape.vocab_size)  # :446-449
+
+
+def rho_energy(rho):
+    """src/model/bdh.rs:411-419: [B,h,N,d] -> [h,N], mean over the batch of the per-row mean |rho|."""
+    B, _, _, d = rho.shape
+    per_row = np.abs(rho).sum(axis=3, dtype=rho.dtype) / rho.dtype.type(d)
+    return per_row.sum(axis=0, dtype=rho.dtype) / rho.dtype.type(B)
 
 
 def greedy_token(logits_row) -> int:
@@ -404,6 +415,7 @@ class COracle:
             path = build_c_oracle()
         self.lib = ctypes.CDLL(path)
         self.lib.orc_forward_with_state.restype = ctypes.c_int
+        self.lib.orc_forward_with_state_viz.restype = ctypes.c_int
         self.lib.orc_greedy_token.restype = ctypes.c_int
         self.lib.orc_sample_from_logits.restype = ctypes.c_int
 
@@ -520,6 +532,35 @@ class COracle:
         if rc != 0:
             raise ValueError("token id out of range")
         return logits, pos.value, x_tap, attn_tap
+
+    def rho_energy(self, rho):
+        rho = _f32(rho)
+        B, h, N, d = rho.shape
+        out = np.empty((h, N), np.float32)
+        self.lib.orc_rho_energy(_p(rho), B, h, N, d, _p(out))
+        return out
+
+    def forward_with_state_viz(self, shape: BDHShape, w: BDHWeights, tokens, rho: np.ndarray, position: int,
+                               sparse_state: bool = True):
+        """forward_with_state plus the LayerVizState taps: returns (logits, new position, viz [L,4,h,N])
+        with viz[l] = (x_last, y_last, xy_last, rho_last).  rho is updated in place."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int64)
+        B, T = tokens.shape
+        h, d, N, V, L = shape.n_head, shape.n_embd, shape.latent_per_head, shape.vocab_size, shape.n_layer
+        Nq = 2 * N if shape.rotary == POPE else N
+        assert rho.dtype == np.float32 and rho.flags.c_contiguous and rho.shape == (L, B, h, Nq, d)
+        keep = [_f32(w.embed), _f32(w.encoder), _f32(w.encoder_v), _f32(w.decoder), _f32(w.lm_head)]
+        sl = None if shape.alibi_slopes is None else _f32(shape.alibi_slopes)
+        m = _OrcModel(L, d, h, N, V, shape.rotary, shape.rope_theta, shape.relu_threshold,
+                      None if sl is None else sl.ctypes.data, *[a.ctypes.data for a in keep])
+        logits = np.empty((B, T, V), np.float32)
+        viz = np.zeros((L, 4, h, N), np.float32)
+        pos = ctypes.c_int64(position)
+        rc = self.lib.orc_forward_with_state_viz(ctypes.byref(m), _p(tokens), B, T, _p(rho), ctypes.byref(pos),
+                                                 _p(logits), ctypes.c_int(int(sparse_state)), _p(viz))
+        if rc != 0:
+            raise ValueError("token id out of range")
+        return logits, pos.value, viz
 
     def greedy_token(self, logits_row) -> int:
         row = _f32(logits_row)

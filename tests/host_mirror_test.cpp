@@ -23,6 +23,8 @@ typedef struct {
 } orc_model;
 int orc_forward_with_state(const orc_model *m, const int64_t *tokens, int B, int T, float *rho, int64_t *position,
                            float *logits, float *x_tap, float *attn_tap, int sparse_state);
+int orc_forward_with_state_viz(const orc_model *m, const int64_t *tokens, int B, int T, float *rho, int64_t *position,
+                               float *logits, int sparse_state, float *viz);
 void orc_relu_lowrank(const float *in, int B, int hin, int T, int d, const float *w, int h, int N, const float *bias,
                       float thr, int block_size, const uint8_t *active_blocks, int n_blocks, float *out);
 void orc_fused_state_aligned(const float *query, const float *value, const float *freqs, const float *slopes, int B, int h,
@@ -110,6 +112,24 @@ static void inference_paths_run_across_configs(const Context &ctx) {
     std::printf("  %-5s fused=%d logits rel err %.2e\n", as_str(rotary), (int)fused, e);
     EXPECT(e < 1e-3);
     EXPECT(rel_err(state.storage->to_host(), rho) < 1e-3);
+    // one more token with the LayerVizState by-products (src/model/bdh.rs:386-434)
+    const std::vector<int64_t> more{9, 10};
+    std::vector<float> ref2(2 * 1 * V), viz(2 * 4 * h * N);
+    model.forward_with_state(more, 2, 1, state, nullptr, true);
+    EXPECT(orc_forward_with_state_viz(&m, more.data(), 2, 1, rho.data(), &pos, ref2.data(), 0, viz.data()) == 0);
+    auto maps = state.take_viz();
+    EXPECT(maps.size() == 2 && maps[0] && maps[1] && !state.layers[0].viz);
+    for (size_t l = 0; l < 2 && maps[l]; ++l) {
+      const float *p = viz.data() + l * 4 * h * N;
+      const std::vector<float> x(p, p + h * N), y(p + h * N, p + 2 * h * N), xy(p + 2 * h * N, p + 3 * h * N),
+          energy(p + 3 * h * N, p + 4 * h * N);
+      EXPECT(rel_err(maps[l]->x_last, x) < 1e-3 && rel_err(maps[l]->y_last, y) < 1e-3);
+      EXPECT(rel_err(maps[l]->xy_last, xy) < 1e-3);
+      if (rotary == RotaryEmbedding::Pope)
+        EXPECT(std::all_of(maps[l]->rho_last.begin(), maps[l]->rho_last.end(), [](float v) { return v == 0.0f; }));
+      else
+        EXPECT(rel_err(maps[l]->rho_last, energy) < 1e-3);
+    }
   }
 }
 

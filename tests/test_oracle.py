@@ -357,6 +357,54 @@ def test_forward_decode_equals_prefill(corc, rotary):
     assert 0.35 < frac < 0.65
 
 
+def test_rho_energy_is_the_batch_mean_of_row_mean_abs(corc):
+    """src/model/bdh.rs:411-419 against a float64 library statement."""
+    rng = np.random.default_rng(41)
+    rho = rng.standard_normal((3, 2, 10, 24)).astype(np.float32)
+    want = np.abs(rho.astype(np.float64)).mean(axis=3).mean(axis=0)
+    np.testing.assert_allclose(corc.rho_energy(rho), want, rtol=2e-6)
+    np.testing.assert_allclose(orc.rho_energy(rho), want, rtol=2e-6)
+    # one hot row: energy = |value| / d / B at that neuron only
+    one = np.zeros((2, 1, 4, 8), np.float32)
+    one[1, 0, 2, 5] = -3.0
+    e = corc.rho_energy(one)
+    assert e[0, 2] == np.float32(3.0 / 8 / 2) and np.count_nonzero(e) == 1
+
+
+@pytest.mark.parametrize("rotary", [ROPE, POPE, ALIBI])
+def test_forward_viz_taps(corc, rotary):
+    """LayerVizState (src/model/bdh.rs:386-434): last token of the first sequence, energy of the updated
+    state; the C and numpy restatements agree and the taps are consistent with the plain forward."""
+    shape = _small_shape(rotary)
+    w = orc.init_weights(shape, seed=6)
+    tokens = np.array([[5, 1, 9, 30, 2], [0, 31, 7, 7, 12]])
+    N, h, d, L = shape.latent_per_head, 2, 16, 2
+    Nq = 2 * N if rotary == POPE else N
+    rho = np.zeros((L, 2, h, Nq, d), np.float32)
+    logits, pos, viz = corc.forward_with_state_viz(shape, w, tokens, rho, 0, sparse_state=False)
+    rho_plain = np.zeros_like(rho)
+    logits_plain, _, x_tap, _ = corc.forward_with_state(shape, w, tokens, rho_plain, 0, taps=True, sparse_state=False)
+    np.testing.assert_array_equal(logits, logits_plain)
+    np.testing.assert_array_equal(rho, rho_plain)
+    assert pos == 5 and viz.shape == (L, 4, h, N)
+    st = orc.ModelState(L)
+    taps = {}
+    orc.forward_with_state(shape, w, tokens, st, taps)
+    for l in range(L):
+        np.testing.assert_array_equal(viz[l, 0], x_tap[l, 0, :, -1])  # x_last = x[b=0, :, T-1]
+        np.testing.assert_array_equal(viz[l, 2], viz[l, 0] * viz[l, 1])  # xy = x * y
+        assert (viz[l, 1] >= 0).all() and (viz[l, 1] > 0).any()
+        nv = taps["viz"][l]
+        np.testing.assert_allclose(viz[l, 0], nv["x_last"], atol=2e-5, rtol=1e-3)
+        np.testing.assert_allclose(viz[l, 1], nv["y_last"], atol=2e-5, rtol=1e-3)
+        np.testing.assert_allclose(viz[l, 2], nv["xy_last"], atol=2e-6, rtol=1e-3)
+        np.testing.assert_allclose(viz[l, 3], nv["rho_last"], atol=1e-7, rtol=1e-3)
+        if rotary == POPE:
+            assert not viz[l, 3].any()  # state rows 2N != N: the reference stores zeros
+        else:
+            np.testing.assert_allclose(viz[l, 3], np.abs(rho[l].astype(np.float64)).mean(3).mean(0), rtol=1e-5)
+
+
 def test_forward_rejects_bad_token(corc):
     shape = _small_shape(ROPE)
     w = orc.init_weights(shape, seed=4)
