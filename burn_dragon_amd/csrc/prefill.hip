@@ -139,7 +139,9 @@ struct GemmArgs {
   int n_tiles, n_slices;
 };
 
-constexpr int KM_STRIDE = BM + 8;  // bf16 elements per k row of a k-major tile in LDS (528 bytes)
+// bf16 elements per k row of a k-major tile in LDS: 576 bytes = 64 mod 256, so the four k rows of 64 bytes
+// that 32 lanes of a transposing read touch fall on disjoint quarters of the 64 banks
+constexpr int KM_STRIDE = BM + 32;
 
 template <bool A_KMAJOR, int EPI>
 __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
@@ -305,8 +307,9 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
 // Fast variant for full tiles (M, N multiples of 256, K a multiple of 64, both operands
 // k-contiguous): the tiles go from global memory straight into LDS (global_load_lds_dwordx4, no
 // VGPR staging, no ds_write), double buffered.  LDS tile layout: blocks of 8 rows x 128 bytes
-// (1 KiB, one wave-wide load each); inside a block the 16-byte slot of (row r, k-chunk c) is
-// r*8 + (c ^ r), which makes the 16-byte fragment reads bank-conflict free without padding.
+// (1 KiB, one wave-wide load each); inside a block the 16-byte slot of (row R, k-chunk c) is
+// (R%8)*8 + (c ^ ((R/2)%8)): the LDS has 64 banks and serves a 16-byte read 16 lanes at a time, and
+// 16 consecutive rows at one k-chunk then cover all 64 banks once (no conflicts, no padding).
 // Same accumulation order as k_gemm, so both give identical results.
 // ------------------------------------------------------------------------------------
 typedef __attribute__((address_space(1))) const void *gptr_t;
@@ -352,7 +355,7 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // source chunk of this lane inside an 8-row block: row lr, k-chunk lc (the XOR swizzle)
-  const int lr = lane >> 3, lc = (lane & 7) ^ lr;
+  const int lr = lane >> 3, lc = (lane & 7) ^ ((lr >> 1) | ((wave & 1) << 2));
   const unsigned short *pa[4], *pb[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
@@ -383,12 +386,12 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int R = wm * 128 + i * 32 + (lane & 31);
-        fa[i] = *reinterpret_cast<const bf16x8 *>(sa + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ (R & 7))) * 8);
+        fa[i] = *reinterpret_cast<const bf16x8 *>(sa + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ ((R >> 1) & 7))) * 8);
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int R = wn * 64 + j * 32 + (lane & 31);
-        fb[j] = *reinterpret_cast<const bf16x8 *>(sb + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ (R & 7))) * 8);
+        fb[j] = *reinterpret_cast<const bf16x8 *>(sb + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ ((R >> 1) & 7))) * 8);
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
