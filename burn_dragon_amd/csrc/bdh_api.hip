@@ -232,6 +232,7 @@ int bdh_rho_energy(bdh_ctx *ctx, int B, int h, int N, int d, const void *rho, in
     return bdh_fail(ctx, BDH_E_INVAL, "clock outside the 31-bit stamp range");
   if (h == 0 || N == 0) return BDH_OK;
   if (!out || (!rho && B > 0 && d > 0)) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  if (!bdh_aligned(rho, 16)) return bdh_fail(ctx, BDH_E_ALIGN, "rho needs 16-byte alignment");
   float slopes[64] = {0};
   if (stamps) {
     if (alibi_slopes_host)

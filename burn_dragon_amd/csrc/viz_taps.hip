@@ -14,6 +14,17 @@ __device__ __forceinline__ float viz_load(const unsigned short *p) {
   return __uint_as_float(static_cast<unsigned int>(*p) << 16);
 }
 
+__device__ __forceinline__ float viz_abs_sum4(const float *p) {
+  const float4 v = *reinterpret_cast<const float4 *>(p);
+  return (fabsf(v.x) + fabsf(v.y)) + (fabsf(v.z) + fabsf(v.w));
+}
+__device__ __forceinline__ float viz_abs_sum4(const unsigned short *p) {
+  const uint2 v = *reinterpret_cast<const uint2 *>(p);
+  const float a = __uint_as_float((v.x << 16) & 0x7fffffffu), b = __uint_as_float(v.x & 0x7fff0000u);
+  const float c = __uint_as_float((v.y << 16) & 0x7fffffffu), e = __uint_as_float(v.y & 0x7fff0000u);
+  return (a + b) + (c + e);
+}
+
 // out[hh,n] = (sum_b (sum_c |rho[b,hh,n,c]|) / d) / B   (src/model/bdh.rs:411-419)
 // One wave per (head, neuron): the B rows of d elements are read coalesced, one after the other.
 // A lazily decayed ALiBi state (stamps != null) is read as the state it stands for: row (b,hh,n)
@@ -29,11 +40,16 @@ __global__ __launch_bounds__(256) void k_rho_energy(const RhoT *__restrict__ rho
   const int hh = (int)(row / N);
   const int n = (int)(row - (long)hh * N);
   float acc = 0.0f;
+  const bool vec = (d & 3) == 0;  // rows are 16-byte (f32) / 8-byte (bf16) aligned: four elements per load
   for (int b = 0; b < B; ++b) {
     const long r = ((long)b * h + hh) * N + n;
     const RhoT *p = rho + r * d;
     float s = 0.0f;
-    for (int c = lane; c < d; c += 64) s += fabsf(viz_load(p + c));
+    if (vec) {
+      for (int c = lane * 4; c < d; c += 256) s += viz_abs_sum4(p + c);
+    } else {
+      for (int c = lane; c < d; c += 64) s += fabsf(viz_load(p + c));
+    }
     for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
     if (stamps) {
       const long clock = clocks_dev ? (long)clocks_dev[b] + clock_add : clock_scalar;
