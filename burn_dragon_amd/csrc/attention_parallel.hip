@@ -8,6 +8,7 @@
 // on the f32 matrix cores (v_mfma_f32_32x32x2_f32): S = mask(Q Q^T) + bias is materialised per
 // slice, a row pass sums |S|, and out = (S V) / (norm + eps).  The bf16 form for inference is in
 // prefill.hip.
+#include <algorithm>
 #include <vector>
 
 #include "bdh_internal.h"
@@ -44,6 +45,50 @@ __global__ __launch_bounds__(256) void k_rotate_f32(const float *__restrict__ x,
       qr[n] = m * c;
       qr[N + n] = m * s;
     }
+  }
+}
+
+// q [S,Tc,Nq] from rows t0..t0+Tc of x [S][T][N] (x points at row t0 of slice 0), token t of the chunk at
+// position pos0 + t, or pos_dev[b] + pos_add + t with per-sequence positions.  The arithmetic is that of
+// the decode step kernels (src/model/attention.rs:305-330), so the rotated values are the same bits.
+__global__ __launch_bounds__(256) void k_rotate_chunk_f32(const float *__restrict__ x, long x_slice_stride,
+                                                          const float *__restrict__ freqs, float *__restrict__ q,
+                                                          int Tc, int N, int rotary, long pos0,
+                                                          const int32_t *__restrict__ pos_dev, int pos_add, int h) {
+  const long row = blockIdx.x;  // slice * Tc + t
+  const long slice = row / Tc;
+  const int t = (int)(row - slice * Tc);
+  const float pos = (float)((pos_dev ? (long)pos_dev[slice / h] + pos_add : pos0) + t);
+  const float *xr = x + slice * x_slice_stride + (long)t * N;
+  const int Nq = rotary == BDH_POPE ? 2 * N : N;
+  float *qr = q + row * Nq;
+  if (rotary == BDH_ROPE) {  // N is even: one lane per pair
+    for (int pr = threadIdx.x; pr < (N >> 1); pr += 256) {
+      const float2 xv = reinterpret_cast<const float2 *>(xr)[pr];
+      float2 o = make_float2(0.0f, 0.0f);
+      if (xv.x != 0.0f || xv.y != 0.0f) {
+        const float2 fv = reinterpret_cast<const float2 *>(freqs)[pr];
+        const float raw0 = pos * fv.x, raw1 = pos * fv.y;
+        float s0, c0, s1, c1;
+        sincosf((raw0 - floorf(raw0)) * kTwoPi, &s0, &c0);
+        sincosf((raw1 - floorf(raw1)) * kTwoPi, &s1, &c1);
+        const float a0 = xv.x * c0, r0 = (-xv.y) * s0;
+        const float a1 = xv.y * c1, r1 = xv.x * s1;
+        o.x = a0 + r0;
+        o.y = a1 + r1;
+      }
+      reinterpret_cast<float2 *>(qr)[pr] = o;
+    }
+    return;
+  }
+  for (int n = threadIdx.x; n < N; n += 256) {
+    const float raw = pos * freqs[n];
+    const float ph = (raw - floorf(raw)) * kTwoPi;
+    float sn, cs;
+    sincosf(ph, &sn, &cs);
+    const float m = logf(expf(xr[n] * 1.0f) + 1.0f) / 1.0f;  // softplus(x, 1)
+    qr[n] = m * cs;
+    qr[N + n] = m * sn;
   }
 }
 
@@ -115,7 +160,7 @@ constexpr int FK = 16;    // k per LDS stage
 constexpr int FLD = 20;   // LDS row stride in floats (80 bytes: 16-byte aligned, spreads the banks)
 
 struct FsaArgs {
-  const float *A;   // [slices][M][lda], k contiguous
+  const float *A;   // A_KMAJOR ? [slices][K][lda] (m contiguous) : [slices][M][lda] (k contiguous)
   const float *Bm;  // B_KMAJOR ? [b][K][ldb] (n contiguous) : [slices][N][ldb] (k contiguous)
   float *C;         // [slices][M][ldc]
   long a_batch, b_batch, c_batch;
@@ -129,6 +174,7 @@ struct FsaArgs {
   const float *slopes;          // [h] device
   // output epilogue
   const float *norm;            // [slices][M] or null
+  int beta;                     // EPI 2: C += acc instead of C = acc
 };
 
 __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_ok) {
@@ -141,13 +187,20 @@ __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_
   return r;
 }
 
-// EPI 0: scores (mask, ALiBi term, zero outside the pattern); EPI 1: out = acc / (norm + eps).
+// EPI 0: scores (mask, ALiBi term, zero outside the pattern); EPI 1: out = acc / (norm + eps);
+// EPI 2: C = acc or C += acc.
+// A k-major operand (its reduction index is the slow one in memory) is staged as it lies, [k][m] with a
+// row stride of tile + 4 floats: float4 stores, and fragment reads of one float per lane in which the
+// 32 lanes of a half-wave take consecutive addresses and the two halves (k and k + 8) fall on the two
+// halves of the 64 banks.
 // Tile BM x BN, NWM x NWN waves, each wave (BM/NWM) x (BN/NWN).  The 128 x 128 tile needs 8 bytes per
 // clock and workgroup from the L2, which three resident workgroups per CU do not get; the
 // 256 x 256 tile halves that per FLOP and is the one that keeps the matrix cores busy.
-template <int EPI, bool B_KMAJOR, int BM, int BN, int NWM, int NWN>
+template <int EPI, bool A_KMAJOR, bool B_KMAJOR, int BM, int BN, int NWM, int NWN>
 __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
   constexpr int NT = NWM * NWN * 64;
+  constexpr int KLA = BM + 4, KLB = BN + 4;  // row strides of the k-major LDS layouts
+  static_assert(FK * KLA <= BM * FLD && FK * KLB <= BN * FLD, "k-major tile must fit");
   constexpr int MI = BM / NWM / 32, NJ = BN / NWN / 32;
   constexpr int CA = BM * 4 / NT, CB = BN * 4 / NT;  // float4 chunks per thread and stage
   static_assert(CA >= 1 && CB >= 1 && CA * NT == BM * 4 && CB * NT == BN * 4, "tile does not divide over the threads");
@@ -178,6 +231,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
   } else if (g.dense) {
     K = min(K, ((min(m0 + BM, g.M) - 1) / bs + 1) * bs);  // S is zero beyond the row tile's last block
   }
+  if (K <= 0) tile_active = false;
 
   f32x16 acc[MI][NJ];
 #pragma unroll
@@ -195,9 +249,15 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
 #pragma unroll
       for (int c = 0; c < CA; ++c) {
         const int chunk = c * NT + tid;
-        const int row = chunk >> 2, kc = (chunk & 3) * 4;
-        pa[c] = (m0 + row < g.M && k0 < K) ? fsa_ld4(A + (long)(m0 + row) * g.lda + k0 + kc, K - (k0 + kc), a_vec)
-                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!A_KMAJOR) {
+          const int row = chunk >> 2, kc = (chunk & 3) * 4;
+          pa[c] = (m0 + row < g.M && k0 < K) ? fsa_ld4(A + (long)(m0 + row) * g.lda + k0 + kc, K - (k0 + kc), a_vec)
+                                             : make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+          const int kr = chunk / (BM / 4), mc = (chunk % (BM / 4)) * 4;  // BM/4 chunks of 4 rows per k row
+          pa[c] = (k0 + kr < K) ? fsa_ld4(A + (long)(k0 + kr) * g.lda + m0 + mc, g.M - (m0 + mc), a_vec)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
       }
 #pragma unroll
       for (int c = 0; c < CB; ++c) {
@@ -217,8 +277,13 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
 #pragma unroll
       for (int c = 0; c < CA; ++c) {
         const int chunk = c * NT + tid;
-        const int row = chunk >> 2, kc = (chunk & 3) * 4;
-        *reinterpret_cast<float4 *>(s_a + row * FLD + kc) = pa[c];
+        if (!A_KMAJOR) {
+          const int row = chunk >> 2, kc = (chunk & 3) * 4;
+          *reinterpret_cast<float4 *>(s_a + row * FLD + kc) = pa[c];
+        } else {
+          const int kr = chunk / (BM / 4), mc = (chunk % (BM / 4)) * 4;
+          *reinterpret_cast<float4 *>(s_a + kr * KLA + mc) = pa[c];
+        }
       }
 #pragma unroll
       for (int c = 0; c < CB; ++c) {
@@ -228,10 +293,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
           *reinterpret_cast<float4 *>(s_b + row * FLD + kc) = pb[c];
         } else {
           const int kr = chunk / (BN / 4), nc = (chunk % (BN / 4)) * 4;
-          s_b[(nc + 0) * FLD + kr] = pb[c].x;
-          s_b[(nc + 1) * FLD + kr] = pb[c].y;
-          s_b[(nc + 2) * FLD + kr] = pb[c].z;
-          s_b[(nc + 3) * FLD + kr] = pb[c].w;
+          *reinterpret_cast<float4 *>(s_b + kr * KLB + nc) = pb[c];
         }
       }
     };
@@ -241,6 +303,12 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
       float fa[MI][8], fb[NJ][8];
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
+        if (A_KMAJOR) {
+          const float *p = s_a + kb * KLA + wm * (BM / NWM) + i * 32 + r;
+#pragma unroll
+          for (int q = 0; q < 8; ++q) fa[i][q] = p[q * KLA];
+          continue;
+        }
         const float *p = s_a + (wm * (BM / NWM) + i * 32 + r) * FLD + kb;
         const float4 lo = *reinterpret_cast<const float4 *>(p), hi = *reinterpret_cast<const float4 *>(p + 4);
         fa[i][0] = lo.x; fa[i][1] = lo.y; fa[i][2] = lo.z; fa[i][3] = lo.w;
@@ -248,6 +316,12 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
       }
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
+        if (B_KMAJOR) {
+          const float *p = s_b + kb * KLB + wn * (BN / NWN) + j * 32 + r;
+#pragma unroll
+          for (int q = 0; q < 8; ++q) fb[j][q] = p[q * KLB];
+          continue;
+        }
         const float *p = s_b + (wn * (BN / NWN) + j * 32 + r) * FLD + kb;
         const float4 lo = *reinterpret_cast<const float4 *>(p), hi = *reinterpret_cast<const float4 *>(p + 4);
         fb[j][0] = lo.x; fb[j][1] = lo.y; fb[j][2] = lo.z; fb[j][3] = lo.w;
@@ -298,11 +372,15 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
             }
           }
           C[(long)row * g.ldc + col] = v;
-        } else {
+        } else if (EPI == 1) {
           if (col >= g.N) continue;
           float v = acc[i][j][e];
           if (g.norm) v = v / (g.norm[(long)slice * g.M + row] + kRowNormEps);
           C[(long)row * g.ldc + col] = v;
+        } else {
+          if (col >= g.N) continue;
+          float *p = C + (long)row * g.ldc + col;
+          *p = g.beta ? *p + acc[i][j][e] : acc[i][j][e];
         }
       }
     }
@@ -388,11 +466,11 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     const unsigned groups = (unsigned)((S + 7) / 8);
     if (big) {
       g.mt = g.nt = (T + 255) / 256;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 256, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512), 0,
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 256, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512), 0,
                          ctx->stream, g);
     } else {
       g.mt = g.nt = (T + 127) / 128;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
                          ctx->stream, g);
     }
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<scores>");
@@ -409,7 +487,7 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     o.norm = row_normalize ? norm : nullptr;
     o.mt = (T + 127) / 128;
     o.nt = (dv + 127) / 128;
-    hipLaunchKernelGGL((k_fsa_gemm_f32<1, true, 128, 128, 2, 2>), dim3(8 * groups * o.mt * o.nt), dim3(256), 0,
+    hipLaunchKernelGGL((k_fsa_gemm_f32<1, false, true, 128, 128, 2, 2>), dim3(8 * groups * o.mt * o.nt), dim3(256), 0,
                        ctx->stream, o);
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<out>");
     return BDH_OK;
@@ -423,5 +501,97 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
   hipLaunchKernelGGL(k_fsa_row, dim3((unsigned)(S * T)), dim3(256), lds, ctx->stream, q, value, slopes_dev,
                      alibi_slopes_host ? 1 : 0, h, T, Nq, dv, block_size, active, tb, row_normalize, out);
   BDH_LAUNCH_CHECK(ctx, "k_fsa_row");
+  return BDH_OK;
+}
+
+// ------------------------------------------------------------------------------------
+// BDH::recurrent_attention (src/model/bdh.rs:258-307) over many tokens at once, f32, RoPE or PoPE:
+// for a chunk of Tc tokens  out = tril(-1)(Q Q^T) V + Q rho,  rho += Q^T V  — the same sums as the
+// token-by-token loop, reassociated, as four products on the f32 matrix cores.  The cost does not
+// depend on how many neurons are active, which is what a prompt through a densely firing model needs
+// (the sparse step kernels move every touched state row once per token).
+// ------------------------------------------------------------------------------------
+int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *out_ln) {
+  const int B = p.B, h = p.h, T = p.T, N = p.N, d = p.d;
+  const int Nq = p.rotary == BDH_POPE ? 2 * N : N;
+  const long S = (long)B * h;
+  if (p.rotary == BDH_ALIBI || p.rho_dtype != BDH_F32 || p.stamps)
+    return bdh_fail(ctx, BDH_E_INVAL, "the chunked f32 form covers RoPE and PoPE with an f32 state");
+  if (S > 0x7fffffffL / 4096) return bdh_fail(ctx, BDH_E_SHAPE, "B*h too large");
+  // chunk length: a multiple of 128 between 128 and 512 whose rotated activations stay under 4 GiB
+  const size_t per_token = sizeof(float) * (size_t)S * Nq;
+  long Tc = (long)((size_t(4) << 30) / per_token) / 128 * 128;
+  Tc = std::min<long>(512, std::max<long>(128, Tc));
+  Tc = std::min<long>(Tc, T);
+  const int Tcp = ((int)Tc + 3) & ~3;
+  const size_t q_bytes = bdh_align_up(per_token * (size_t)Tc, 256);
+  const size_t sc_bytes = bdh_align_up(sizeof(float) * (size_t)S * Tc * Tcp, 256);
+  int rc = bdh_ws_reserve(ctx, q_bytes + sc_bytes);
+  if (rc != BDH_OK) return rc;
+  float *q = static_cast<float *>(ctx->ws);
+  float *scores = reinterpret_cast<float *>(static_cast<char *>(ctx->ws) + q_bytes);
+  float *rho = static_cast<float *>(p.rho);
+  const unsigned groups = (unsigned)((S + 7) / 8);
+  const int nt_d = (d + 127) / 128;
+  if ((long)groups * 8 * ((Nq + 127) / 128) * nt_d > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
+
+  for (int t0 = 0; t0 < T; t0 += (int)Tc) {
+    const int tc = (int)std::min<long>(Tc, T - t0);
+    hipLaunchKernelGGL(k_rotate_chunk_f32, dim3((unsigned)(S * tc)), dim3(256), 0, ctx->stream, p.x + (long)t0 * N,
+                       (long)T * N, p.freqs, q, tc, N, p.rotary, (long)(p.position + t0), p.positions_dev, t0, h);
+    BDH_LAUNCH_CHECK(ctx, "k_rotate_chunk_f32");
+    {  // S = tril(-1)(Q Q^T)
+      FsaArgs g{};
+      g.A = q; g.Bm = q; g.C = scores;
+      g.a_batch = g.b_batch = (long)tc * Nq; g.c_batch = (long)Tc * Tcp;
+      g.lda = g.ldb = Nq; g.ldc = Tcp; g.M = g.N = tc; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
+      g.block_size = 1; g.tb = tc; g.h = h; g.use_alibi = 0; g.dense = 1;
+      const bool big = S * ((tc + 255) / 256) * ((tc + 255) / 256) >= 256;
+      if (big) {
+        g.mt = g.nt = (tc + 255) / 256;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 256, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512),
+                           0, ctx->stream, g);
+      } else {
+        g.mt = g.nt = (tc + 127) / 128;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256),
+                           0, ctx->stream, g);
+      }
+      BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<chunk scores>");
+    }
+    {  // out = Q rho   (the state before this chunk; B = rho [Nq,d] is k-major)
+      FsaArgs g{};
+      g.A = q; g.Bm = rho; g.C = p.out + (long)t0 * d;
+      g.a_batch = (long)tc * Nq; g.b_batch = (long)Nq * d; g.c_batch = (long)T * d;
+      g.lda = Nq; g.ldb = d; g.ldc = d; g.M = tc; g.N = d; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
+      g.block_size = 1; g.h = h; g.dense = 0; g.beta = 0;
+      g.mt = (tc + 127) / 128; g.nt = nt_d;
+      hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                         ctx->stream, g);
+      BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q rho>");
+    }
+    {  // out += S V   (K limited to the causal prefix of each row tile)
+      FsaArgs g{};
+      g.A = scores; g.Bm = p.v + (long)t0 * d; g.C = p.out + (long)t0 * d;
+      g.a_batch = (long)Tc * Tcp; g.b_batch = (long)T * d; g.c_batch = (long)T * d;
+      g.lda = Tcp; g.ldb = d; g.ldc = d; g.M = tc; g.N = d; g.K = tc; g.b_div = h; g.n_slices = (int)S;
+      g.block_size = 1; g.h = h; g.dense = 1; g.beta = 1;
+      g.mt = (tc + 127) / 128; g.nt = nt_d;
+      hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                         ctx->stream, g);
+      BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<S V>");
+    }
+    {  // rho += Q^T V   (both operands k-major: the reduction runs over the tokens)
+      FsaArgs g{};
+      g.A = q; g.Bm = p.v + (long)t0 * d; g.C = rho;
+      g.a_batch = (long)tc * Nq; g.b_batch = (long)T * d; g.c_batch = (long)Nq * d;
+      g.lda = Nq; g.ldb = d; g.ldc = d; g.M = Nq; g.N = d; g.K = tc; g.b_div = h; g.n_slices = (int)S;
+      g.block_size = 1; g.h = h; g.dense = 0; g.beta = 1;
+      g.mt = (Nq + 127) / 128; g.nt = nt_d;
+      hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                         ctx->stream, g);
+      BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q^T V>");
+    }
+  }
+  if (out_ln) return bdh_launch_layer_norm(ctx, (int64_t)S * T, d, p.out, out_ln);
   return BDH_OK;
 }

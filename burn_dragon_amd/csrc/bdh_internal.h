@@ -18,6 +18,7 @@ struct bdh_ctx {
   size_t ws_bytes = 0;
   int n_cu = 0;
   int opt_step_split = -1;  // -1 choose by grid size, 0 / 1 force the 256- / 64-pair workgroup
+  int opt_step_dense = -1;  // many-token state step as dense f32 products: -1 from T = 128, 0 never, 1 always
   int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
   char err[512] = {0};
 };
@@ -77,6 +78,9 @@ int bdh_launch_state_steps(bdh_ctx *ctx, const StateStepParams &p);
 // Variant used inside the fused model step: the readout is LayerNorm-ed on the fly
 // (src/model/bdh.rs:359) when out_ln != nullptr.
 int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
+// The same T steps as four dense products per chunk on the f32 matrix cores (attention_parallel.hip):
+// RoPE / PoPE, f32 state, no bitmask or row counts.
+int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
 // rho <- the up-to-date state, stamps <- clock, for a lazily decayed ALiBi state
 int bdh_launch_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, const float *slopes_host, int64_t clock,
                                  const int32_t *clocks_dev, void *rho, int rho_dtype, int32_t *stamps);

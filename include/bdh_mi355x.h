@@ -68,6 +68,9 @@ const char *bdh_last_error(const bdh_ctx *ctx);
 /* Launch-shape knobs for tests and tuning; no counterpart in the reference.
  *   "state_step.split": -1 (default) pick by grid size, 0 = 256 lane pairs per workgroup,
  *                       1 = 64 lane pairs per workgroup of 8 waves (small batches).
+ *   "state_step.dense_chunks": -1 (default) a call of 128+ tokens on an f32 RoPE/PoPE state without
+ *                       bitmask / row-count outputs runs as dense products on the f32 matrix cores,
+ *                       0 = always token by token, 1 = dense products for any T.
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
  *                       1 = the two products on the f32 matrix cores (T >= 128 by default). */
 int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);
@@ -104,7 +107,11 @@ int bdh_default_alibi_slopes(int n_head, float *slopes_host);
  *                        that token (RoPE: both rows of every lane pair with a non-zero
  *                        element; ALiBi/PoPE: Nq)
  *
- * RoPE requires even N (src/model/attention.rs:310).  T = 1 is the decode step.
+ * RoPE requires even N (src/model/attention.rs:310).  T = 1 is the decode step.  A call of 128 or more
+ * tokens on an f32 RoPE/PoPE state that asks for neither bitmask nor row counts computes the same sums
+ * as dense products (out = tril(-1)(Q Q^T) V + Q rho, rho += Q^T V, chunks of up to 512 tokens) on the
+ * f32 matrix cores; results agree with the token loop to f32 reassociation (option
+ * "state_step.dense_chunks").
  */
 int bdh_recurrent_attention(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary,
                             const float *x, const float *v, const float *freqs,

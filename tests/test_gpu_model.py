@@ -128,6 +128,39 @@ def test_inference_paths_run_across_configs(bda, corc, rotary):
     assert rel_err(logits2.cpu().numpy(), logits2_ref) < 1e-3
 
 
+@pytest.mark.parametrize("rotary", ["rope", "pope"])
+def test_long_prompt_takes_the_dense_chunk_form(bda, corc, rotary):
+    """A prompt of 128+ tokens runs the state update as dense products on the f32 matrix cores; logits and
+    state agree with the oracle's token loop, and decoding continues from that state."""
+    cfg = bda.BDHConfig(n_layer=2, n_embd=32, n_head=2, mlp_internal_dim_multiplier=8, vocab_size=64, dropout=0.0)
+    cfg.fused_kernels.set_block_sizes(4, 4)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse(rotary))
+    shape, w, model = _model_pair(bda, cfg, seed=23)
+    rng = np.random.default_rng(3)
+    tokens = rng.integers(0, 64, (2, 150))
+    state = model.init_state()
+    logits = model.forward_with_state(torch.from_numpy(tokens), state)
+    Nq = model.latent_q
+    rho_ref = np.zeros((2, 2, 2, Nq, 32), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, tokens, rho_ref, 0, sparse_state=False)
+    assert rel_err(logits.cpu().numpy(), logits_ref) < 1e-3
+    assert rel_err(state.storage.cpu().numpy(), rho_ref) < 1e-3
+    # the same prompt through the step kernels (dense form switched off) gives the same logits
+    ctx = bda.ffi.default_context(0)
+    try:
+        ctx.set_option("state_step.dense_chunks", 0)
+        state_s = model.init_state()
+        logits_s = model.forward_with_state(torch.from_numpy(tokens), state_s)
+    finally:
+        ctx.set_option("state_step.dense_chunks", -1)
+    assert rel_err(logits.cpu().numpy(), logits_s.cpu().numpy()) < 1e-4
+    more = rng.integers(0, 64, (2, 1))
+    logits2 = model.forward_with_state(torch.from_numpy(more), state)
+    logits2_ref, pos, _, _ = corc.forward_with_state(shape, w, more, rho_ref, pos, sparse_state=False)
+    assert state.position == 151 == pos
+    assert rel_err(logits2.cpu().numpy(), logits2_ref) < 1e-3
+
+
 def test_config1_architecture_prefill_and_greedy_decode(bda, corc):
     """BASELINE config 1 architecture (V=256, d=256, h=4, N=8192, RoPE) with L=2 and a short
     run so the oracle finishes in seconds: 16-byte prompt, 8 greedy tokens, batch 1."""

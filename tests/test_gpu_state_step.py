@@ -331,3 +331,71 @@ def test_lazy_alibi_decay_matches_the_eager_reference_semantics(gpu, corc, dtype
 
     out_e = recurrent_attention(xt, vt, rho_e, torch.zeros(N, device=dev), 0, RotaryEmbedding.ALIBI)
     assert rel_err(out, out_e.cpu().numpy()) < tol and rel_err(rho.float().cpu().numpy(), rho_e.float().cpu().numpy()) < tol
+
+
+@pytest.fixture
+def dense_chunks(gpu):
+    """Forces the many-token dense form (f32 matrix cores) for the duration of a test."""
+    ffi, _ = gpu
+    ctx = ffi.default_context(0)
+    ctx.set_option("state_step.dense_chunks", 1)
+    yield ctx
+    ctx.set_option("state_step.dense_chunks", -1)
+
+
+def _run_plain(recurrent_attention, x, v, rho, freqs, position, rotary, positions=None):
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    dev = "cuda:0"
+    rt = torch.from_numpy(rho).to(dev).contiguous()
+    pt = None if positions is None else torch.from_numpy(np.asarray(positions, np.int32)).to(dev)
+    out = recurrent_attention(torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev), rt,
+                              torch.from_numpy(freqs).to(dev), position, RotaryEmbedding(rotary), None, pt)
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), rt.cpu().numpy()
+
+
+@pytest.mark.parametrize("rotary", [orc.ROPE, orc.POPE])
+@pytest.mark.parametrize("B,h,T,N,d,density", [
+    (2, 2, 130, 64, 32, 0.3),     # one chunk, partial tiles everywhere
+    (1, 3, 600, 40, 20, 0.5),     # two chunks (512 + 88), d and N not multiples of the tile or of 8
+    (2, 4, 257, 256, 256, 0.05),  # the headline row width, sparse activations
+    (1, 1, 5, 34, 6, 1.0),        # tiny, d not a multiple of 4 (scalar loads)
+])
+def test_dense_chunk_form_matches_sequential_oracle(gpu, corc, dense_chunks, rotary, B, h, T, N, d, density):
+    """out = tril(-1)(Q Q^T) V + Q rho0 and rho += Q^T V on the f32 matrix cores against the oracle's
+    token-by-token loop (src/model/bdh.rs:286-303), from a non-zero state at a non-zero position."""
+    _, recurrent_attention = gpu
+    x, v, _ = make_inputs(7 * T + N + d, B, h, T, N, d, density)
+    Nq = 2 * N if rotary == orc.POPE else N
+    rho0 = (0.05 * np.random.default_rng(5).standard_normal((B, h, Nq, d))).astype(np.float32)
+    freqs = corc.build_freqs(N, rotary=rotary)
+    position = 37
+    out, rho_new = _run_plain(recurrent_attention, x, v, rho0, freqs, position, rotary)
+    out_ref, rho_ref = corc.recurrent_attention(corc.rotate(x, freqs, rotary, position), v, rho0.copy())
+    assert out.shape == out_ref.shape
+    assert rel_err(out, out_ref) < 2e-5, rel_err(out, out_ref)
+    assert rel_err(rho_new, rho_ref) < 2e-5, rel_err(rho_new, rho_ref)
+
+
+def test_dense_chunk_form_equals_step_kernels_and_handles_device_positions(gpu, corc):
+    """The same call through the sparse step kernels and through the dense form; per-sequence device
+    positions; T = 128 takes the dense form by default."""
+    ffi, recurrent_attention = gpu
+    ctx = ffi.default_context(0)
+    B, h, T, N, d = 3, 2, 128, 128, 256
+    x, v, rho = make_inputs(99, B, h, T, N, d, 0.1, rho_scale=0.05)
+    freqs = corc.build_freqs(N)
+    positions = [0, 77, 4000]
+    try:
+        ctx.set_option("state_step.dense_chunks", 0)
+        out_s, rho_s = _run_plain(recurrent_attention, x, v, rho, freqs, 0, orc.ROPE, positions)
+    finally:
+        ctx.set_option("state_step.dense_chunks", -1)
+    out_d, rho_d = _run_plain(recurrent_attention, x, v, rho, freqs, 0, orc.ROPE, positions)
+    assert rel_err(out_d, out_s) < 2e-5 and rel_err(rho_d, rho_s) < 2e-5
+    assert not np.array_equal(out_d, out_s)  # different summation order: the dense form did run
+    for b, pos in enumerate(positions):
+        o_ref, r_ref = corc.recurrent_attention(corc.rotate(x[b : b + 1], freqs, orc.ROPE, pos), v[b : b + 1],
+                                                rho[b : b + 1].copy())
+        assert rel_err(out_d[b : b + 1], o_ref) < 2e-5 and rel_err(rho_d[b : b + 1], r_ref) < 2e-5
