@@ -175,6 +175,9 @@ struct FsaArgs {
   // output epilogue
   const float *norm;            // [slices][M] or null
   int beta;                     // EPI 2: C += acc instead of C = acc
+  // mod > 0: slice = s1 * mod + s2 and operand X starts at s1 * x_batch + s2 * x_mod_stride
+  int mod;
+  long a_mod_stride, b_mod_stride, c_mod_stride;
 };
 
 __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_ok) {
@@ -220,6 +223,12 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
   const float *A = g.A + (long)slice * g.a_batch;
   const float *Bm = g.Bm + (long)(slice / g.b_div) * g.b_batch;
   float *C = g.C + (long)slice * g.c_batch;
+  if (g.mod > 0) {
+    const long s1 = slice / g.mod, s2 = slice % g.mod;
+    A = g.A + s1 * g.a_batch + s2 * g.a_mod_stride;
+    Bm = g.Bm + s1 * g.b_batch + s2 * g.b_mod_stride;
+    C = g.C + s1 * g.c_batch + s2 * g.c_mod_stride;
+  }
   const int bs = g.block_size;
 
   int K = g.K;
@@ -593,5 +602,28 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
     }
   }
   if (out_ln) return bdh_launch_layer_norm(ctx, (int64_t)S * T, d, p.out, out_ln);
+  return BDH_OK;
+}
+
+// The encoder E over many rows (src/model/bdh.rs:383,436-438): mixed [B*T, h*N] . decoder [h*N, d], as one
+// product per (sequence, head) on the f32 matrix cores.  partial [h][B*T][d] receives the h per-head terms
+// of every output row; the caller sums them in head order.
+int bdh_launch_decoder_partials_f32(bdh_ctx *ctx, int B, int T, int h, int N, int d, const float *xy,
+                                    const float *decoder, float *partial) {
+  const long S = (long)B * h;
+  const unsigned groups = (unsigned)((S + 7) / 8);
+  FsaArgs g{};
+  g.A = xy; g.Bm = decoder; g.C = partial;
+  g.mod = h;
+  g.a_batch = (long)h * T * N; g.a_mod_stride = (long)T * N;  // xy [B,h,T,N]
+  g.b_batch = 0; g.b_mod_stride = (long)N * d;                // decoder rows hh*N .. hh*N+N-1
+  g.c_batch = (long)T * d; g.c_mod_stride = (long)B * T * d;
+  g.lda = N; g.ldb = d; g.ldc = d; g.M = T; g.N = d; g.K = N; g.b_div = 1; g.n_slices = (int)S;
+  g.block_size = 1; g.h = h; g.dense = 0; g.beta = 0;
+  g.mt = (T + 127) / 128; g.nt = (d + 127) / 128;
+  if ((long)groups * 8 * g.mt * g.nt > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
+  hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                     ctx->stream, g);
+  BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<decoder>");
   return BDH_OK;
 }

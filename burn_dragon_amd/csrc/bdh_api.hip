@@ -112,6 +112,16 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     ctx->opt_step_dense = value;
     return BDH_OK;
   }
+  if (strcmp(name, "relu_lowrank.tile") == 0) {
+    if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "relu_lowrank.tile takes 0 or 1");
+    ctx->opt_lowrank_tile = value;
+    return BDH_OK;
+  }
+  if (strcmp(name, "decoder.mfma") == 0) {
+    if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "decoder.mfma takes 0 or 1");
+    ctx->opt_decoder_mfma = value;
+    return BDH_OK;
+  }
   if (strcmp(name, "fused_state_aligned.path") == 0) {
     if (value < -1 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "fused_state_aligned.path takes -1, 0 or 1");
     ctx->opt_fsa_path = value;

@@ -19,6 +19,8 @@ struct bdh_ctx {
   int n_cu = 0;
   int opt_step_split = -1;  // -1 choose by grid size, 0 / 1 force the 256- / 64-pair workgroup
   int opt_step_dense = -1;  // many-token state step as dense f32 products: -1 from T = 128, 0 never, 1 always
+  int opt_lowrank_tile = 1;  // 0: relu_lowrank never takes the 64-row tile kernel
+  int opt_decoder_mfma = 1;  // 0: the encoder E never takes the f32 matrix-core form
   int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
   char err[512] = {0};
 };
@@ -107,6 +109,9 @@ int bdh_launch_embed_ln(bdh_ctx *ctx, const int64_t *tokens, int64_t rows, int d
 int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
                                 const float *xy, const float *decoder, float *cur);
 // logits = cur . lm_head (+ argmax of the last token per sequence) (src/model/bdh.rs:446-449)
+// attention_parallel.hip: partial[hh][b*T+t][:] = xy[b,hh,t,:] . decoder[hh*N.., :] on the f32 matrix cores
+int bdh_launch_decoder_partials_f32(bdh_ctx *ctx, int B, int T, int h, int N, int d, const float *xy,
+                                    const float *decoder, float *partial);
 int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cur,
                        const float *lm_head, float *logits, int64_t *next_tokens);
 // positions[b] = min(positions[b] + delta, INT32_MAX): the device-side form of state.position += T

@@ -91,6 +91,100 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank(const float *__restrict__
   }
 }
 
+// Many input rows (a prompt, a large batch): a 64-row x 256-column tile per workgroup, 16 rows x 4
+// adjacent columns per thread.  Wave w owns rows 16w..16w+15, so an input value is one LDS broadcast
+// for the whole wave; a weight row segment is one float4 per lane.  The inputs are staged 64 k at a
+// time.  Every output is still one k-sequential fmaf chain, so the values are those of k_relu_lowrank
+// bit for bit; the tile only cuts the weight re-reads from one per 8 rows to one per 64.
+__global__ __launch_bounds__(256) void k_relu_lowrank_tile(const float *__restrict__ in, int h_in, int T, int d,
+                                                          const float *__restrict__ w, int h, int N,
+                                                          const float *__restrict__ bias, float thr,
+                                                          const unsigned char *__restrict__ block_active,
+                                                          int block_size, int n_blocks,
+                                                          const float *__restrict__ gate, float *__restrict__ out,
+                                                          int M) {
+  constexpr int RT = 16, KC = 64;
+  __shared__ __attribute__((aligned(16))) float s_x[64 * KC];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int hh = blockIdx.y;
+  const int n = (blockIdx.x * 64 + lane) * 4;  // N % 4 == 0: a thread's four columns are all in or all out
+  const int m0 = blockIdx.z * 64;
+  const bool live = n < N;
+
+  float4 acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+  const float *wp = w + (long)hh * d * N + (live ? n : 0);
+  const float *sx = s_x + wave * RT * KC;
+  for (int kc = 0; kc < d; kc += KC) {  // d % 4 == 0
+    const int kn = min(KC, d - kc);
+    __syncthreads();
+    for (int i = tid; i < 64 * KC / 4; i += 256) {
+      const int r = i / (KC / 4), k4 = (i - r * (KC / 4)) * 4;
+      const int m = m0 + r;
+      float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (m < M && k4 < kn) {
+        const int b = m / T, t = m - b * T;
+        val = *reinterpret_cast<const float4 *>(in + (((long)b * h_in + (h_in == 1 ? 0 : hh)) * T + t) * d + kc + k4);
+      }
+      *reinterpret_cast<float4 *>(s_x + r * KC + k4) = val;
+    }
+    __syncthreads();
+    if (live) {
+      for (int k0 = 0; k0 < kn; k0 += 4) {
+        float4 wv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) wv[u] = *reinterpret_cast<const float4 *>(wp + (long)(kc + k0 + u) * N);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+          const float4 xin = *reinterpret_cast<const float4 *>(sx + r * KC + k0);
+          const float xs[4] = {xin.x, xin.y, xin.z, xin.w};
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            acc[r].x = __builtin_fmaf(xs[u], wv[u].x, acc[r].x);
+            acc[r].y = __builtin_fmaf(xs[u], wv[u].y, acc[r].y);
+            acc[r].z = __builtin_fmaf(xs[u], wv[u].z, acc[r].z);
+            acc[r].w = __builtin_fmaf(xs[u], wv[u].w, acc[r].w);
+          }
+        }
+      }
+    }
+  }
+  if (!live) return;
+  float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (bias) bv = *reinterpret_cast<const float4 *>(bias + (long)hh * N + n);
+  float mk[4] = {1.f, 1.f, 1.f, 1.f};
+  if (block_active)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int blk = (n + c) / block_size;
+      mk[c] = (blk < n_blocks && block_active[blk]) ? 1.0f : 0.0f;
+    }
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int m = m0 + wave * RT + r;
+    if (m < M) {
+      const int b = m / T, t = m - b * T;
+      const long o = (((long)b * h + hh) * T + t) * N + n;
+      float p[4] = {acc[r].x, acc[r].y, acc[r].z, acc[r].w};
+      const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+      float4 gv = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (gate) gv = *reinterpret_cast<const float4 *>(gate + o);
+      const float gg[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if (bias) p[c] = p[c] + bb[c];
+        if (thr != 0.0f) p[c] = p[c] - thr;
+        float y = p[c] > 0.0f ? p[c] : 0.0f;
+        if (block_active) y = y * mk[c];
+        if (gate) y = gg[c] * y;
+        p[c] = y;
+      }
+      *reinterpret_cast<float4 *>(out + o) = make_float4(p[0], p[1], p[2], p[3]);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // LayerNorm rows (one workgroup per row); in == out allowed.  The row is staged in LDS and
 // every thread walks it in index order, so mean and variance are the same left-to-right f32
@@ -424,6 +518,18 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
     }
     mask_dev = static_cast<const unsigned char *>(ctx->ws);
   }
+  // many rows: the 64 x 256 tile (same values, an eighth of the weight traffic)
+  const bool aligned16 = bdh_aligned(p.in, 16) && bdh_aligned(p.weight, 16) && bdh_aligned(p.out, 16) &&
+                         bdh_aligned(p.bias, 16) && bdh_aligned(p.gate, 16);
+  if (M >= 64 && ctx->opt_lowrank_tile != 0 && (p.N & 3) == 0 && (p.d & 3) == 0 && p.d > 0 && aligned16) {
+    const long row_tiles = (M + 63) / 64;
+    if (row_tiles > 65535 || p.h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (row tiles %ld)", row_tiles);
+    hipLaunchKernelGGL(k_relu_lowrank_tile, dim3((p.N / 4 + 63) / 64, p.h, (unsigned)row_tiles), dim3(256), 0, ctx->stream,
+                       p.in, p.h_in, p.T, p.d, p.weight, p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks,
+                       p.gate, p.out, (int)M);
+    BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_tile");
+    return BDH_OK;
+  }
   const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
   const size_t lds = sizeof(float) * (size_t)RT * (p.d > 0 ? p.d : 1);
   if (lds > 64 * 1024) return bdh_fail(ctx, BDH_E_SHAPE, "d=%d too large for the projection tile", p.d);
@@ -460,6 +566,17 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   const int M = B * T;
   const long K = (long)h * N;
   if (d > 1024 || (d & 3)) return bdh_fail(ctx, BDH_E_SHAPE, "decoder needs d %% 4 == 0 and d <= 1024, got %d", d);
+  if (T >= 128 && ctx->opt_decoder_mfma != 0) {
+    // many tokens per sequence: one product per (sequence, head) on the f32 matrix cores, h partials per row
+    int rc = bdh_ws_reserve(ctx, sizeof(float) * (size_t)h * M * d);
+    if (rc != BDH_OK) return rc;
+    float *partial = static_cast<float *>(ctx->ws);
+    rc = bdh_launch_decoder_partials_f32(ctx, B, T, h, N, d, xy, decoder, partial);
+    if (rc != BDH_OK) return rc;
+    hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, h, M, d, cur);
+    BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
+    return BDH_OK;
+  }
   const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
   const int row_tiles = (M + RT - 1) / RT;
   // k-block size: enough workgroups to fill the chip, few enough partials

@@ -71,6 +71,10 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *   "state_step.dense_chunks": -1 (default) a call of 128+ tokens on an f32 RoPE/PoPE state without
  *                       bitmask / row-count outputs runs as dense products on the f32 matrix cores,
  *                       0 = always token by token, 1 = dense products for any T.
+ *   "relu_lowrank.tile": 1 (default) calls with 64+ rows take the 64-row tile kernel (same values),
+ *                       0 = always the 8-row kernel.
+ *   "decoder.mfma":     1 (default) the encoder E of a call with 128+ tokens per sequence runs on
+ *                       the f32 matrix cores, 0 = always the VALU kernel.
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
  *                       1 = the two products on the f32 matrix cores (T >= 128 by default). */
 int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);

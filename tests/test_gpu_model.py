@@ -53,7 +53,7 @@ def test_relu_lowrank_fused_matches_reference(bda):
     assert_close(fused.cpu().numpy(), reference.numpy(), 1e-5, 1e-5)
 
 
-@pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (32, 1, 1), (1, 64, 4)])
+@pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (32, 1, 1), (1, 64, 4), (2, 100, 1), (3, 43, 4)])
 def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
     """One k-sequential FMA chain per output on both sides: values, and therefore the active
     sets, are identical bit for bit whatever the launch tiling."""
@@ -72,6 +72,31 @@ def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
     gated = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
                                        bda.BlockPattern1d.dense(64), gate=torch.from_numpy(gate).to(DEV))
     assert np.array_equal(gated.cpu().numpy(), gate * ref)
+
+
+def test_relu_lowrank_many_rows_with_bias_threshold_and_mask(bda, corc):
+    """The 64-row tile kernel (B*T >= 64) with every optional input, bit-exact against the oracle, and
+    identical to the 8-row kernel."""
+    from burn_dragon_amd.kernel import relu_lowrank
+
+    B, T, h, d, N = 2, 70, 3, 36, 200  # ragged in rows, columns and k
+    rng = np.random.default_rng(8)
+    inp = rng.standard_normal((B, 1, T, d)).astype(np.float32)
+    weight = (0.2 * rng.standard_normal((h, d, N))).astype(np.float32)
+    bias = (0.1 * rng.standard_normal((h, 1, N))).astype(np.float32)
+    layout = bda.BlockPattern1d.from_blocks(8, [0, 3, 4, 17, 24])
+    ref = corc.relu_lowrank(inp, weight, bias.reshape(h, N), 0.05, 8, [0, 3, 4, 17, 24])
+    args = (torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), torch.from_numpy(bias).to(DEV), 0.05, layout)
+    got = relu_lowrank.fused_forward(*args).cpu().numpy()
+    assert np.array_equal(got, ref)
+    assert 0.05 < (ref > 0).mean() < 0.2
+    ctx = bda.ffi.default_context(0)
+    try:
+        ctx.set_option("relu_lowrank.tile", 0)
+        small = relu_lowrank.fused_forward(*args).cpu().numpy()
+    finally:
+        ctx.set_option("relu_lowrank.tile", 1)
+    assert np.array_equal(got, small)
 
 
 def test_layer_norm_matches_oracle_and_library(bda, corc):
