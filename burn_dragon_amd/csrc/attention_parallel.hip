@@ -9,6 +9,7 @@
 // slice, a row pass sums |S|, and out = (S V) / (norm + eps).  The bf16 form for inference is in
 // prefill.hip.
 #include <algorithm>
+#include <cstring>
 #include <vector>
 
 #include "bdh_internal.h"
@@ -90,6 +91,15 @@ __global__ __launch_bounds__(256) void k_rotate_chunk_f32(const float *__restric
     qr[n] = m * cs;
     qr[N + n] = m * sn;
   }
+}
+
+// stamps[b,h,n] = clock (or clocks_dev[b] + add), saturated to the stamp range
+__global__ __launch_bounds__(256) void k_set_stamps(int32_t *__restrict__ stamps, long rows, long rows_per_seq,
+                                                    long clock, const int32_t *__restrict__ clocks_dev, int add) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows) return;
+  const long c = clocks_dev ? (long)clocks_dev[i / rows_per_seq] + add : clock;
+  stamps[i] = (int32_t)min(c, 0x7fffffffL);
 }
 
 // one workgroup per (slice, query row i)
@@ -178,7 +188,14 @@ struct FsaArgs {
   // mod > 0: slice = s1 * mod + s2 and operand X starts at s1 * x_batch + s2 * x_mod_stride
   int mod;
   long a_mod_stride, b_mod_stride, c_mod_stride;
+  // ALiBi state decay (src/model/bdh.rs:299-301) in the many-token form, g = exp(log_decay[slice % h]):
+  //   FSA_DECAY_SCORES  EPI 0: S[t,s] *= g^(t-s)
+  //   FSA_DECAY_ROWS    EPI 2: acc[t,:] *= g^t
+  //   FSA_DECAY_STATE   EPI 2, A k-major: A[k,:] *= g^(K-k) on load and C = g^K * C + acc
+  int decay_mode;
+  float log_decay[64];
 };
+constexpr int FSA_DECAY_SCORES = 1, FSA_DECAY_ROWS = 2, FSA_DECAY_STATE = 4;
 
 __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_ok) {
   if (n_valid >= 4 && vec_ok) return *reinterpret_cast<const float4 *>(p);
@@ -241,6 +258,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
     K = min(K, ((min(m0 + BM, g.M) - 1) / bs + 1) * bs);  // S is zero beyond the row tile's last block
   }
   if (K <= 0) tile_active = false;
+  const float ld = g.decay_mode ? g.log_decay[slice % g.h] : 0.0f;
 
   f32x16 acc[MI][NJ];
 #pragma unroll
@@ -266,6 +284,10 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
           const int kr = chunk / (BM / 4), mc = (chunk % (BM / 4)) * 4;  // BM/4 chunks of 4 rows per k row
           pa[c] = (k0 + kr < K) ? fsa_ld4(A + (long)(k0 + kr) * g.lda + m0 + mc, g.M - (m0 + mc), a_vec)
                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+          if (EPI == 2 && (g.decay_mode & FSA_DECAY_STATE)) {  // token k of K is decayed K - k times by the end
+            const float f = expf((float)(K - (k0 + kr)) * ld);
+            pa[c].x *= f; pa[c].y *= f; pa[c].z *= f; pa[c].w *= f;
+          }
         }
       }
 #pragma unroll
@@ -374,6 +396,7 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
             const bool act = g.dense ? (cbk <= rbk) : (g.active[(long)rbk * g.tb + cbk] != 0);
             if (act) {
               v = (rbk == cbk && col >= row) ? 0.0f : acc[i][j][e];  // tril(-1) on diagonal blocks (:88-90)
+              if ((g.decay_mode & FSA_DECAY_SCORES) && col < row) v = v * expf((float)(row - col) * ld);
               if (g.use_alibi) {  // added to every entry of an active block (:97-100)
                 const float al = slope * ((float)col - (float)row);
                 v = v + al;
@@ -389,7 +412,12 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
         } else {
           if (col >= g.N) continue;
           float *p = C + (long)row * g.ldc + col;
-          *p = g.beta ? *p + acc[i][j][e] : acc[i][j][e];
+          float v = acc[i][j][e];
+          if (g.decay_mode & FSA_DECAY_ROWS) v = v * expf((float)row * ld);
+          if (g.decay_mode & FSA_DECAY_STATE)
+            *p = *p * expf((float)g.K * ld) + v;
+          else
+            *p = g.beta ? *p + v : v;
         }
       }
     }
@@ -524,8 +552,17 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
   const int B = p.B, h = p.h, T = p.T, N = p.N, d = p.d;
   const int Nq = p.rotary == BDH_POPE ? 2 * N : N;
   const long S = (long)B * h;
-  if (p.rotary == BDH_ALIBI || p.rho_dtype != BDH_F32 || p.stamps)
-    return bdh_fail(ctx, BDH_E_INVAL, "the chunked f32 form covers RoPE and PoPE with an f32 state");
+  if (p.rho_dtype != BDH_F32) return bdh_fail(ctx, BDH_E_INVAL, "the chunked f32 form needs an f32 state");
+  const bool alibi = p.rotary == BDH_ALIBI;
+  if (p.stamps && !alibi) return bdh_fail(ctx, BDH_E_INVAL, "decay stamps only apply to ALiBi");
+  float log_decay[64] = {0};
+  if (alibi)  // log of the ROUNDED per-token factor, as in the lazily decayed step (src/model/attention.rs:181-186)
+    for (int i = 0; i < h; ++i) log_decay[i] = (float)log((double)expf(-p.slopes_host[i]));
+  if (p.stamps) {  // a lazily decayed state: apply what is pending, the products below decay every row themselves
+    int rc0 = bdh_launch_alibi_materialize(ctx, B, h, N, d, p.slopes_host, p.position, p.positions_dev, p.rho,
+                                           p.rho_dtype, p.stamps);
+    if (rc0 != BDH_OK) return rc0;
+  }
   if (S > 0x7fffffffL / 4096) return bdh_fail(ctx, BDH_E_SHAPE, "B*h too large");
   // chunk length: a multiple of 128 between 128 and 512 whose rotated activations stay under 4 GiB
   const size_t per_token = sizeof(float) * (size_t)S * Nq;
@@ -533,7 +570,7 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
   Tc = std::min<long>(512, std::max<long>(128, Tc));
   Tc = std::min<long>(Tc, T);
   const int Tcp = ((int)Tc + 3) & ~3;
-  const size_t q_bytes = bdh_align_up(per_token * (size_t)Tc, 256);
+  const size_t q_bytes = alibi ? 0 : bdh_align_up(per_token * (size_t)Tc, 256);  // ALiBi does not rotate: q = x
   const size_t sc_bytes = bdh_align_up(sizeof(float) * (size_t)S * Tc * Tcp, 256);
   int rc = bdh_ws_reserve(ctx, q_bytes + sc_bytes);
   if (rc != BDH_OK) return rc;
@@ -546,15 +583,28 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
 
   for (int t0 = 0; t0 < T; t0 += (int)Tc) {
     const int tc = (int)std::min<long>(Tc, T - t0);
-    hipLaunchKernelGGL(k_rotate_chunk_f32, dim3((unsigned)(S * tc)), dim3(256), 0, ctx->stream, p.x + (long)t0 * N,
-                       (long)T * N, p.freqs, q, tc, N, p.rotary, (long)(p.position + t0), p.positions_dev, t0, h);
-    BDH_LAUNCH_CHECK(ctx, "k_rotate_chunk_f32");
-    {  // S = tril(-1)(Q Q^T)
+    const float *qc = q;           // this chunk's rotated activations [S][tc][Nq]
+    long q_batch = (long)tc * Nq;
+    if (alibi) {
+      qc = p.x + (long)t0 * N;
+      q_batch = (long)T * N;
+    } else {
+      hipLaunchKernelGGL(k_rotate_chunk_f32, dim3((unsigned)(S * tc)), dim3(256), 0, ctx->stream, p.x + (long)t0 * N,
+                         (long)T * N, p.freqs, q, tc, N, p.rotary, (long)(p.position + t0), p.positions_dev, t0, h);
+      BDH_LAUNCH_CHECK(ctx, "k_rotate_chunk_f32");
+    }
+    auto with_decay = [&](FsaArgs &g, int mode) {
+      if (!alibi) return;
+      g.decay_mode = mode;
+      memcpy(g.log_decay, log_decay, sizeof(log_decay));
+    };
+    {  // S = tril(-1)(Q Q^T)   (ALiBi: S[t,s] *= decay^(t-s))
       FsaArgs g{};
-      g.A = q; g.Bm = q; g.C = scores;
-      g.a_batch = g.b_batch = (long)tc * Nq; g.c_batch = (long)Tc * Tcp;
+      g.A = qc; g.Bm = qc; g.C = scores;
+      g.a_batch = g.b_batch = q_batch; g.c_batch = (long)Tc * Tcp;
       g.lda = g.ldb = Nq; g.ldc = Tcp; g.M = g.N = tc; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
       g.block_size = 1; g.tb = tc; g.h = h; g.use_alibi = 0; g.dense = 1;
+      with_decay(g, FSA_DECAY_SCORES);
       const bool big = S * ((tc + 255) / 256) * ((tc + 255) / 256) >= 256;
       if (big) {
         g.mt = g.nt = (tc + 255) / 256;
@@ -567,12 +617,13 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
       }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<chunk scores>");
     }
-    {  // out = Q rho   (the state before this chunk; B = rho [Nq,d] is k-major)
+    {  // out = Q rho   (the state before this chunk; B = rho [Nq,d] is k-major; ALiBi: row t *= decay^t)
       FsaArgs g{};
-      g.A = q; g.Bm = rho; g.C = p.out + (long)t0 * d;
-      g.a_batch = (long)tc * Nq; g.b_batch = (long)Nq * d; g.c_batch = (long)T * d;
+      g.A = qc; g.Bm = rho; g.C = p.out + (long)t0 * d;
+      g.a_batch = q_batch; g.b_batch = (long)Nq * d; g.c_batch = (long)T * d;
       g.lda = Nq; g.ldb = d; g.ldc = d; g.M = tc; g.N = d; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
       g.block_size = 1; g.h = h; g.dense = 0; g.beta = 0;
+      with_decay(g, FSA_DECAY_ROWS);
       g.mt = (tc + 127) / 128; g.nt = nt_d;
       hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
                          ctx->stream, g);
@@ -590,16 +641,24 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<S V>");
     }
     {  // rho += Q^T V   (both operands k-major: the reduction runs over the tokens)
+       // ALiBi: rho = decay^tc * rho + sum_s decay^(tc-s) q_s (x) v_s
       FsaArgs g{};
-      g.A = q; g.Bm = p.v + (long)t0 * d; g.C = rho;
-      g.a_batch = (long)tc * Nq; g.b_batch = (long)T * d; g.c_batch = (long)Nq * d;
+      g.A = qc; g.Bm = p.v + (long)t0 * d; g.C = rho;
+      g.a_batch = q_batch; g.b_batch = (long)T * d; g.c_batch = (long)Nq * d;
       g.lda = Nq; g.ldb = d; g.ldc = d; g.M = Nq; g.N = d; g.K = tc; g.b_div = h; g.n_slices = (int)S;
       g.block_size = 1; g.h = h; g.dense = 0; g.beta = 1;
+      with_decay(g, FSA_DECAY_STATE);
       g.mt = (Nq + 127) / 128; g.nt = nt_d;
       hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
                          ctx->stream, g);
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q^T V>");
     }
+  }
+  if (p.stamps) {  // every row is now up to date as of the end of the call
+    const long rows = S * N;
+    hipLaunchKernelGGL(k_set_stamps, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, ctx->stream, p.stamps, rows,
+                       (long)h * N, (long)(p.position + T), p.positions_dev, T);
+    BDH_LAUNCH_CHECK(ctx, "k_set_stamps");
   }
   if (out_ln) return bdh_launch_layer_norm(ctx, (int64_t)S * T, d, p.out, out_ln);
   return BDH_OK;

@@ -856,8 +856,8 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
     }
     return BDH_OK;
   }
-  // many tokens, f32 state, no decay and no per-token by-products: the dense form on the f32 matrix cores
-  if (p.rho_dtype == BDH_F32 && p.rotary != BDH_ALIBI && !p.bitmask && !p.rows_touched &&
+  // many tokens, f32 state, no per-token by-products: the dense form on the f32 matrix cores
+  if (p.rho_dtype == BDH_F32 && !p.bitmask && !p.rows_touched &&
       (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : T >= 128))
     return bdh_launch_state_chunks_f32(ctx, p, out_ln);
   // tokens per launch: only the f32 RoPE kernel walks several, as many as 64 MiB of partials allow

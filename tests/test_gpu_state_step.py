@@ -399,3 +399,51 @@ def test_dense_chunk_form_equals_step_kernels_and_handles_device_positions(gpu, 
         o_ref, r_ref = corc.recurrent_attention(corc.rotate(x[b : b + 1], freqs, orc.ROPE, pos), v[b : b + 1],
                                                 rho[b : b + 1].copy())
         assert rel_err(out_d[b : b + 1], o_ref) < 2e-5 and rel_err(rho_d[b : b + 1], r_ref) < 2e-5
+
+
+@pytest.mark.parametrize("B,h,T,N,d,density", [(2, 3, 130, 64, 32, 0.3), (1, 2, 600, 40, 20, 0.5), (2, 4, 200, 256, 256, 0.05)])
+def test_dense_chunk_form_alibi_matches_sequential_oracle(gpu, corc, dense_chunks, B, h, T, N, d, density):
+    """ALiBi in the many-token form: S[t,s] *= decay^(t-s), out_t gets decay^t (q_t . rho0), the state ends as
+    decay^T rho0 + sum_s decay^(T-s) q_s (x) v_s — against the oracle's loop (src/model/bdh.rs:286-303).
+    decay^k is exp(k log decay) here and k roundings of a product there: 1e-4 relative."""
+    _, recurrent_attention = gpu
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    x, v, rho0 = make_inputs(3 * T + N, B, h, T, N, d, density, rho_scale=0.05)
+    slopes = np.array([0.05 * (i + 1) for i in range(h)], np.float32)  # slow decay: old tokens still matter
+    dev = "cuda:0"
+    rt = torch.from_numpy(rho0).to(dev).contiguous()
+    out = recurrent_attention(torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev), rt,
+                              torch.zeros(N, device=dev), 11, RotaryEmbedding.ALIBI, slopes)
+    torch.cuda.synchronize()
+    out_ref, rho_ref = corc.recurrent_attention(x, v, rho0.copy(), corc.alibi_decay(slopes))
+    assert rel_err(out.cpu().numpy(), out_ref) < 1e-4, rel_err(out.cpu().numpy(), out_ref)
+    assert rel_err(rt.cpu().numpy(), rho_ref) < 1e-4, rel_err(rt.cpu().numpy(), rho_ref)
+
+
+def test_dense_chunk_form_on_a_lazily_decayed_alibi_state(gpu, corc):
+    """T = 150 on a state with pending decay: the call applies it, runs the dense form (default from T = 128)
+    and leaves every stamp at clock + T; a following single-token lazy step continues correctly."""
+    from burn_dragon_amd.recurrent import alibi_materialize, recurrent_attention_lazy_alibi
+
+    rng = np.random.default_rng(12)
+    B, h, T, N, d = 2, 2, 150, 128, 256
+    x, v, rho0 = make_inputs(77, B, h, T + 1, N, d, 0.1, rho_scale=0.05)
+    slopes = np.array([0.02, 0.3], np.float32)
+    clock = 60
+    stamps0 = rng.integers(0, clock + 1, (B, h, N)).astype(np.int32)
+    dev = "cuda:0"
+    rt, st = torch.from_numpy(rho0).to(dev).contiguous(), torch.from_numpy(stamps0).to(dev)
+    xt, vt = torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev)
+    out = recurrent_attention_lazy_alibi(xt[:, :, :T].contiguous(), vt[:, :T].contiguous(), rt, st, clock, slopes)
+    out1 = recurrent_attention_lazy_alibi(xt[:, :, T:].contiguous(), vt[:, T:].contiguous(), rt, st, clock + T, slopes)
+    alibi_materialize(rt, st, clock + T + 1, slopes)
+    torch.cuda.synchronize()
+    # oracle: the state the stamps stand for, then the eager loop over all T + 1 tokens
+    decay = corc.alibi_decay(slopes).astype(np.float64)
+    start = rho0.astype(np.float64) * (decay[None, :, None] ** (clock - stamps0))[..., None]
+    out_ref, rho_ref = corc.recurrent_attention(x, v, start.astype(np.float32), corc.alibi_decay(slopes))
+    assert rel_err(out.cpu().numpy(), out_ref[:, :, :T]) < 1e-4
+    assert rel_err(out1.cpu().numpy(), out_ref[:, :, T:]) < 1e-4
+    assert rel_err(rt.cpu().numpy(), rho_ref) < 1e-4
+    assert (st.cpu().numpy() == clock + T + 1).all()
