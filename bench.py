@@ -158,7 +158,10 @@ def bench_prefill(args):
                                f"accumulate, {args.density:.0%} active, RoPE positions 0..T, fresh state",
                    "algorithmic_flop_per_step": flop},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     # HBM bytes of one call, all kernels: FETCH_SIZE (scaled x2 as for a copy of known size) +
+                     # WRITE_SIZE from profiles/prefill_config3_bf16_kernel_trace.md; measured at the default shape only
+                     "traffic": 7.56e9 if (B, T, h, N, d) == (8, 2048, 4, 8192, 256) else None,
                      "kernel": "whole bdh_prefill_chunked call (k_rope_bf16 + 3 k_gemm launches); algorithmic FLOP "
                                "= B*h*[T(T-1)N + T(T-1)d + 2TNd]"},
     }))
