@@ -306,6 +306,70 @@ def bench_parallel(args):
     }))
 
 
+def bench_chunks(args):
+    """BDH::recurrent_attention (src/model/bdh.rs:258-307) over --time tokens per call at the config-2 state
+    shape, f32: the many-token form (dense products on the f32 matrix cores) with the token loop of the
+    sparse step kernels timed beside it on the same inputs."""
+    import torch
+    from scipy.stats import norm
+
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.kernel.linear_attention import build_freqs
+    from burn_dragon_amd.positional import RotaryEmbedding
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    dev = torch.device("cuda:0")
+    B, h, N, d = args.batch, args.heads, args.latent, args.embd
+    T = 256 if args.time == 2048 else args.time
+    steps = 10 if args.steps == 1000 else args.steps
+    warmup = min(args.warmup, 2)
+    g = torch.Generator(device=dev).manual_seed(5)
+    mu = float(norm.ppf(args.density))
+    x = torch.empty((B, h, T, N), device=dev)
+    for b in range(B):
+        x[b] = torch.relu(torch.randn((h, T, N), device=dev, generator=g) + mu)
+    v = torch.randn((B, T, d), device=dev, generator=g)
+    rho = 0.01 * torch.randn((B, h, N, d), device=dev, generator=g)
+    f = build_freqs(N, 65536.0, RotaryEmbedding.ROPE, device=dev).reshape(-1)
+    ctx = ffi.default_context(0)
+
+    def timed(n):
+        for _ in range(warmup):
+            recurrent_attention(x, v, rho, f, 0, RotaryEmbedding.ROPE)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(n):
+            recurrent_attention(x, v, rho, f, i * T, RotaryEmbedding.ROPE)
+        e1.record()
+        torch.cuda.synchronize()
+        return max(e0.elapsed_time(e1), (time.perf_counter() - t0) * 1e3) / n
+
+    ms = timed(steps)
+    ctx.set_option("state_step.dense_chunks", 0)
+    try:
+        ms_loop = timed(max(1, steps // 5))
+    finally:
+        ctx.set_option("state_step.dense_chunks", -1)
+    S = float(B * h)
+    flop = S * (T * (T - 1.0) * N + T * (T - 1.0) * d + 4.0 * T * N * d)
+    achieved = flop / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "tokens/sec, many-token recurrent state step (f32 dense products)",
+        "value": B * T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"recurrent_attention B={B} h={h} T={T} N={N} d={d}, f32 state, RoPE, "
+                               f"{args.density:.0%} active, state carried from call to call",
+                   "algorithmic_flop_per_step": flop, "token_loop_ms_per_step": ms_loop,
+                   "token_loop_tokens_per_s": B * T / (ms_loop * 1e-3)},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": F32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / F32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "whole call (k_rotate_chunk_f32 + 4 k_fsa_gemm_f32 launches); algorithmic FLOP = "
+                               "B*h*[T(T-1)N + T(T-1)d + 4TNd]"},
+    }))
+
+
 def bench_model(args):
     """Full-model greedy decode (BDH::forward_with_state per token, argmax on the device).
     c1 = BASELINE config 1 (V=256, d=256, h=4, N=8192, L=6, B=1, 64-byte prompt, 256 tokens);
@@ -387,11 +451,12 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--prefill-chunk", type=int, default=0,
                     help="model workload: feed the prompt in calls of this many tokens (0 = one call)")
-    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy", "alibi", "parallel"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy", "alibi", "parallel", "chunks"], default="decode",
                     help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA); "
                          "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4); "
                          "alibi = ALiBi state step, lazily decayed state beside the eager dense decay; "
-                         "parallel = fused_state_aligned in f32 at the config-3 shape; copy = counter calibration")
+                         "parallel = fused_state_aligned in f32 at the config-3 shape; chunks = many-token state step "
+                         "(f32 dense products) beside the token loop at the config-2 shape; copy = counter calibration")
     ap.add_argument("--model-config", choices=["c1", "c4"], default="c1")
     ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
     ap.add_argument("--graph", action="store_true", help="model: replay one captured HIP graph per token")
@@ -428,6 +493,8 @@ def main():
         return bench_alibi(args)
     if args.workload == "parallel":
         return bench_parallel(args)
+    if args.workload == "chunks":
+        return bench_chunks(args)
     B, h, N, d = args.batch, args.heads, args.latent, args.embd
     ctx = ffi.default_context(0)
     lib = ctx.lib
