@@ -1,7 +1,7 @@
 // bdh_host_io.hpp — the callers either side of the model step, for a C++ host:
 //   tokenizer::{Tokenizer, ByteTokenizer, CharVocab}   src/tokenizer/mod.rs:17-27, byte.rs, char_vocab.rs
 //   record::{load_record, parse_record}                BinFileRecorder files, src/bin/infer.rs:177-186
-//   generation::{GenerationSettings, prefill_state, sample_next_token, generate_tokens, generate_text}
+//   generation::{GenerationSettings, prefill_state, sample_next_token, generate_tokens, generate_text, bdh_generate}
 //                                                      src/generation.rs:12-260
 // Everything here is host logic over bdh_host.hpp; the draw of the next token happens on the device
 // (bdh_sample_top_k), so only one uniform variate goes up and one token comes down per step.
@@ -479,6 +479,24 @@ inline int64_t sample_next_token(const Context &ctx, BDH &model, ModelState &sta
   const int64_t next = sample_from_logits(ctx, logits.data() + (T - 1) * V, V, temperature, top_k, u);
   logits = model.forward_with_state({next}, 1, 1, state);
   return next;
+}
+
+// BDH::generate (src/model/bdh.rs:170-252): the prompt, then max_new_tokens draws from
+// softmax(logits / temperature) over the top_k values; rng supplies the uniform variates the reference
+// takes from thread_rng.  Batch size 1, as in the reference.
+template <typename Rng>
+std::vector<int64_t> bdh_generate(const Context &ctx, BDH &model, std::vector<int64_t> indices, size_t max_new_tokens,
+                                  float temperature, std::optional<size_t> top_k, Rng &rng) {
+  if (indices.empty()) throw std::invalid_argument("generate needs at least one prompt token");
+  ModelState state = model.init_state();
+  Tensor logits = model.forward_with_state(indices, 1, indices.size(), state);
+  std::uniform_real_distribution<float> uniform(0.0f, 1.0f);
+  for (size_t i = 0; i < max_new_tokens; ++i) {
+    float u = uniform(rng);
+    if (u >= 1.0f) u = std::nextafter(1.0f, 0.0f);  // some library versions round up to the bound
+    indices.push_back(sample_next_token(ctx, model, state, logits, temperature, top_k, u));
+  }
+  return indices;
 }
 
 template <typename Rng>

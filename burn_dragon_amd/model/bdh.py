@@ -154,17 +154,27 @@ class BDH:
         """src/model/bdh.rs:91-94."""
         return self.forward_with_state(tokens, self.init_state())
 
-    def generate(self, indices: torch.Tensor, max_new_tokens: int) -> torch.Tensor:
-        """Greedy form (top_k = 1) of src/model/bdh.rs:170-252; the argmax stays on the device."""
+    def generate(self, indices: torch.Tensor, max_new_tokens: int, temperature: float = 1.0,
+                 top_k: Optional[int] = 1, generator: Optional[torch.Generator] = None) -> torch.Tensor:
+        """src/model/bdh.rs:170-252: prompt through forward_with_state, then max_new_tokens draws from
+        softmax(logits / temperature) restricted to the top_k values (None or 0 = all).  The draw runs on the
+        device (bdh_sample_top_k) with uniform variates from `generator` standing for the reference's
+        thread_rng; top_k = 1 is greedy decoding and takes the argmax the lm_head kernel already wrote."""
         assert indices.shape[0] == 1, "generation currently supports batch size 1"  # :178
         state = self.init_state()
         indices = indices.to(self.device, torch.int64)
-        _, nxt = self.forward_with_state(indices, state, want_next=True)
+        greedy = top_k == 1
+        logits, nxt = self.forward_with_state(indices, state, want_next=True)
         out = [indices]
         for _ in range(max_new_tokens):
+            if not greedy:
+                from ..generation import sample_from_logits
+
+                u = torch.rand((1,), device=self.device, generator=generator)
+                nxt = sample_from_logits(self, logits[:, -1], temperature, top_k, u)
             tok = nxt.reshape(1, 1)
             out.append(tok)
-            _, nxt = self.forward_with_state(tok, state, want_next=True)
+            logits, nxt = self.forward_with_state(tok, state, want_next=True)
         return torch.cat(out, dim=1)
 
 

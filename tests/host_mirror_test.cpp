@@ -310,6 +310,13 @@ static void trained_checkpoint(const Context &ctx, const std::string &dir) {
   }
   std::vector<uint32_t> out32(all.begin(), all.end());
   std::printf("  greedy: %s\n", tok.decode(out32).c_str());
+  // BDH::generate with the reference's signature: top_k = 1 repeats the greedy run, a sampled run is
+  // reproducible from its generator
+  std::mt19937 g1(9), g2(9), g3(9);
+  EXPECT(generation::bdh_generate(ctx, model, prompt, 32, 1.0f, std::optional<size_t>(1), g1) == all);
+  const auto s1 = generation::bdh_generate(ctx, model, prompt, 16, 0.9f, std::optional<size_t>(12), g2);
+  const auto s2 = generation::bdh_generate(ctx, model, prompt, 16, 0.9f, std::optional<size_t>(12), g3);
+  EXPECT(s1 == s2 && s1.size() == prompt.size() + 16);
 
   // sampled text is reproducible from the seed and the on-device draw agrees with the oracle's
   generation::GenerationConfig gc;

@@ -201,3 +201,23 @@ def test_trained_checkpoint_with_lazily_decayed_state(trained, corc):
     torch.cuda.synchronize()
     assert (state.stamps == state.position).all()
     assert rel_err(state.storage.cpu().numpy(), rho_ref) < 1e-3
+
+
+def test_model_generate_has_the_reference_signature(trained):
+    """BDH::generate (src/model/bdh.rs:170-252): indices [1,T] -> [1,T+n]; top_k = 1 equals the greedy
+    generate_tokens run, a sampled run is reproducible from its generator and equals generate_tokens with
+    the same variates."""
+    from burn_dragon_amd.generation import GenerationSettings, generate_tokens
+
+    model, tok, _, _, _ = trained
+    prompt = tok.encode("JULIET:\n")
+    idx = torch.tensor([prompt])
+    greedy = model.generate(idx, 24, 1.0, 1)
+    assert tuple(greedy.shape) == (1, len(prompt) + 24)
+    assert greedy[0].tolist() == generate_tokens(model, prompt, GenerationSettings(24, 1.0, 1))
+    a = model.generate(idx, 24, 0.9, 12, torch.Generator(device=DEV).manual_seed(3))[0].tolist()
+    b = model.generate(idx, 24, 0.9, 12, torch.Generator(device=DEV).manual_seed(3))[0].tolist()
+    c = generate_tokens(model, prompt, GenerationSettings(24, 0.9, 12), None, torch.Generator(device=DEV).manual_seed(3))
+    assert a == b == c and a != greedy[0].tolist()
+    with pytest.raises(AssertionError):
+        model.generate(torch.tensor([prompt, prompt]), 1)  # batch size 1 only, as in the reference
