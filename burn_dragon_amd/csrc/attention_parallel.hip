@@ -686,3 +686,28 @@ int bdh_launch_decoder_partials_f32(bdh_ctx *ctx, int B, int T, int h, int N, in
   BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<decoder>");
   return BDH_OK;
 }
+
+extern "C" int bdh_rotate(bdh_ctx *ctx, int B, int h, int T, int N, int rotary, const float *x, const float *freqs,
+                          int64_t position, const int32_t *positions_dev, float *q) {
+  if (!ctx) return BDH_E_INVAL;
+  if (B < 0 || h < 0 || T < 0 || N < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
+  if (rotary != BDH_ROPE && rotary != BDH_ALIBI && rotary != BDH_POPE)
+    return bdh_fail(ctx, BDH_E_INVAL, "rotary %d is not a bdh_rotary value", rotary);
+  if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
+  if (rotary == BDH_ROPE && (N & 1)) return bdh_fail(ctx, BDH_E_SHAPE, "RoPE needs an even latent size, got N=%d", N);
+  const long rows = (long)B * h * T;
+  if (rows == 0 || N == 0) return BDH_OK;
+  if (!x || !q || (rotary != BDH_ALIBI && !freqs)) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  if (!bdh_aligned(x, 8) || !bdh_aligned(q, 8) || !bdh_aligned(freqs, 8))
+    return bdh_fail(ctx, BDH_E_ALIGN, "x, q and freqs need 8-byte alignment");
+  if (rows > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "B*h*T too large");
+  if (rotary == BDH_ALIBI) {  // Attention::rotate returns its input (src/model/attention.rs:333-335)
+    if (q != x)
+      BDH_HIP_CHECK(ctx, hipMemcpyAsync(q, x, sizeof(float) * (size_t)rows * N, hipMemcpyDeviceToDevice, ctx->stream));
+    return BDH_OK;
+  }
+  hipLaunchKernelGGL(k_rotate_chunk_f32, dim3((unsigned)rows), dim3(256), 0, ctx->stream, x, (long)T * N, freqs, q, T, N,
+                     rotary, (long)position, positions_dev, 0, h);
+  BDH_LAUNCH_CHECK(ctx, "k_rotate_chunk_f32");
+  return BDH_OK;
+}

@@ -26,7 +26,7 @@ EXPORTS = [
     "bdh_fused_state_aligned", "bdh_prefill_chunked", "bdh_model_create", "bdh_model_destroy",
     "bdh_model_state_bytes", "bdh_model_forward", "bdh_model_forward_ex", "bdh_advance_positions",
     "bdh_sample_top_k", "bdh_recurrent_attention_lazy_alibi", "bdh_alibi_materialize", "bdh_model_forward_lazy",
-    "bdh_rho_energy", "bdh_model_forward_viz",
+    "bdh_rho_energy", "bdh_model_forward_viz", "bdh_rotate",
 ]
 
 
@@ -101,6 +101,7 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
                                                        c_int, P, P, P, P]
     lib.bdh_alibi_materialize.argtypes = [P, c_int, c_int, c_int, c_int, c_int64, P, P, P, c_int, P]
     lib.bdh_model_forward_lazy.argtypes = [P, P, c_int, c_int, P, c_int, P, c_int64, P, P, P, P]
+    lib.bdh_rotate.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, c_int64, P, P]
     lib.bdh_rho_energy.argtypes = [P, c_int, c_int, c_int, c_int, P, c_int, P, c_int64, P, P, P]
     lib.bdh_model_forward_viz.argtypes = [P, P, c_int, c_int, P, c_int, P, c_int64, P, P, P, P, P]
     for name in EXPORTS:

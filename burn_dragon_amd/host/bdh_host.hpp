@@ -10,6 +10,7 @@
 //                                          src/kernel/linear_attention.rs:11-163
 //   FusedKernelConfig, BDHConfig           src/model/config.rs:10-164
 //   LayerState, ModelState                 src/model/state.rs:5-57
+//   Attention::{new, forward, rotate_positions, alibi_decay}
 //   BDH::{new, init_state, forward_with_state, forward, generate}
 //                                          src/model/bdh.rs:37-84, 91-94, 170-256, 309-450
 //   ModelOverrides, build_model_config     src/config/core.rs:43-53, src/inference.rs:4-40
@@ -297,6 +298,57 @@ inline BDHConfig build_model_config(const ModelOverrides &o, size_t training_blo
   if (o.rotary_embedding) c.fused_kernels.set_rotary_embedding(*o.rotary_embedding);
   return c;
 }
+
+// ---- model::Attention (src/model/attention.rs:102-349) ---------------------------------
+class Attention {
+ public:
+  Attention(size_t latent, size_t n_head, const FusedKernelConfig &kernel)
+      : n_head_(n_head), fused_(kernel.enabled), block_pattern_(kernel.block_sparse.time),
+        use_alibi_(kernel.rotary_embedding == RotaryEmbedding::Alibi), rotary_embedding_(kernel.rotary_embedding) {
+    freqs_ = Tensor::from_host(kernel::linear_attention::build_freqs(latent, kernel.rope_theta, kernel.rotary_embedding),
+                               {1, 1, 1, latent});
+    if (use_alibi_)
+      alibi_slopes_ = kernel.alibi_slopes ? *kernel.alibi_slopes : kernel::linear_attention::default_alibi_slopes(n_head);
+    else
+      alibi_slopes_.assign(n_head, 0.0f);  // zeros when ALiBi is off, as the reference stores them
+  }
+
+  // :142-175  query [B,h,T,N], value [B,1,T,dv] -> [B,h,T,dv].  The plain branch masks with tril(-1)
+  // element-wise: the fused computation with time blocks of one token.
+  Tensor forward(const Context &ctx, const Tensor &query, const Tensor &value) const {
+    const kernel::BlockPattern2d plain = kernel::BlockPattern2d::dense(1);
+    return kernel::linear_attention::fused_state_aligned(ctx, query, value, freqs_, use_alibi_ ? &alibi_slopes_ : nullptr,
+                                                         fused_ ? block_pattern_ : plain, rotary_embedding_);
+  }
+
+  // :177-179, :332-349  values [B,h,T,N] at positions start..start+T -> [B,h,T,N] (PoPE: 2N columns)
+  Tensor rotate_positions(const Context &ctx, const Tensor &values, size_t start) const {
+    const size_t B = values.dim(0), h = values.dim(1), T = values.dim(2), N = values.dim(3);
+    Tensor out({B, h, T, rotary_embedding_ == RotaryEmbedding::Pope ? 2 * N : N});
+    ctx.check(bdh_rotate(ctx.raw(), (int)B, (int)h, (int)T, (int)N, (int)rotary_embedding_, values.data(), freqs_.data(),
+                         (int64_t)start, nullptr, out.data()));
+    return out;
+  }
+
+  // :181-186  exp(-slopes), or nothing without ALiBi
+  std::optional<std::vector<float>> alibi_decay() const {
+    if (!use_alibi_) return std::nullopt;
+    std::vector<float> d(alibi_slopes_.size());
+    for (size_t i = 0; i < d.size(); ++i) d[i] = std::exp(-alibi_slopes_[i]);
+    return d;
+  }
+
+  const std::vector<float> &alibi_slopes() const { return alibi_slopes_; }
+
+ private:
+  Tensor freqs_;
+  size_t n_head_;
+  bool fused_;
+  kernel::BlockPattern2d block_pattern_;
+  bool use_alibi_;
+  std::vector<float> alibi_slopes_;
+  RotaryEmbedding rotary_embedding_;
+};
 
 // ---- model::state ---------------------------------------------------------------------
 // src/model/state.rs:17-24 (the reference's "viz" feature): [h,N] maps on the host

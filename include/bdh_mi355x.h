@@ -85,6 +85,14 @@ int bdh_build_freqs(int latent, float theta, int rotary, float *freqs_host);
 /* src/kernel/linear_attention.rs:152-163  default_alibi_slopes -> slopes_host[n_head] */
 int bdh_default_alibi_slopes(int n_head, float *slopes_host);
 
+/* Attention::rotate / rotate_positions (src/model/attention.rs:177-179,332-349; rope :305-321, pope
+ * :323-330) on its own: x [B,h,T,N] -> q [B,h,T,Nq] (Nq = 2N for BDH_POPE, else N; BDH_ALIBI copies),
+ * token t at position + t, or positions_dev[b] + t (device int32 [B]) when given.  x and q must not
+ * overlap unless equal for BDH_ALIBI.  The state step and the attention entry points below rotate
+ * internally with the same arithmetic; this entry point serves callers that want the rotated values. */
+int bdh_rotate(bdh_ctx *ctx, int B, int h, int T, int N, int rotary, const float *x, const float *freqs,
+               int64_t position, const int32_t *positions_dev, float *q);
+
 /* ---- a5 + a4: the recurrent state step ------------------------------------------- */
 /*
  * Replaces BDH::recurrent_attention (src/model/bdh.rs:258-307) including the

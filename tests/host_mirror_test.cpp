@@ -133,6 +133,33 @@ static void inference_paths_run_across_configs(const Context &ctx) {
   }
 }
 
+// src/model/attention.rs:383-432, the reference's own two known-answer tests, through the mirror
+static void attention_alibi_kats(const Context &ctx) {
+  FusedKernelConfig kernel;
+  kernel.set_rotary_embedding(RotaryEmbedding::Alibi);
+  kernel.set_alibi_slopes({0.5f, 1.0f});
+  Attention two(1, 2, kernel);
+  const auto decay = two.alibi_decay();
+  EXPECT(decay && std::fabs((*decay)[0] - std::exp(-0.5f)) < 1e-6f && std::fabs((*decay)[1] - std::exp(-1.0f)) < 1e-6f);
+  kernel.set_alibi_slopes({0.5f});
+  Attention one(1, 1, kernel);
+  Tensor query = Tensor::from_host({1.0f, 1.0f}, {1, 1, 2, 1}), value = Tensor::from_host({1.0f, 3.0f}, {1, 1, 2, 1});
+  const std::vector<float> out = one.forward(ctx, query, value).to_host();
+  EXPECT(out.size() == 2 && std::fabs(out[0]) < 1e-6f && std::fabs(out[1] - 1.0f) < 1e-4f);
+  // rotation at position 0 is the identity for RoPE
+  FusedKernelConfig rope;
+  rope.set_rotary_embedding(RotaryEmbedding::Rope);
+  Attention att(8, 1, rope);
+  const std::vector<float> x{0.f, 1.f, 2.f, 0.f, 0.f, 0.f, 3.f, 4.f};
+  Tensor xt = Tensor::from_host(x, {1, 1, 1, 8});
+  EXPECT(att.rotate_positions(ctx, xt, 0).to_host() == x);
+  const std::vector<float> r = att.rotate_positions(ctx, xt, 5).to_host();
+  double n0 = 0, n1 = 0;  // a rotation keeps the norm of every pair
+  for (int i = 0; i < 8; ++i) { n0 += (double)x[i] * x[i]; n1 += (double)r[i] * r[i]; }
+  EXPECT(std::fabs(n0 - n1) < 1e-4 && r[4] == 0.0f && r[5] == 0.0f);
+  EXPECT(!att.alibi_decay());
+}
+
 static void relu_lowrank_fused_matches_reference(const Context &ctx) {
   std::mt19937 g(42);
   auto input = randn(g, 2 * 1 * 5 * 6, 1.0f), weight = randn(g, 1 * 3 * 6 * 8, 1.0f), bias = randn(g, 3 * 1 * 8, 0.5f);
@@ -339,6 +366,7 @@ static void trained_checkpoint(const Context &ctx, const std::string &dir) {
 }
 
 int main(int argc, char **argv) {
+  std::setvbuf(stdout, nullptr, _IOLBF, 0);  // every section name reaches the log before its GPU work starts
   try {
     Context ctx(0);
     config_and_state_semantics();
@@ -349,6 +377,8 @@ int main(int argc, char **argv) {
     }
     std::printf("inference_paths_run_across_configs\n");
     inference_paths_run_across_configs(ctx);
+    std::printf("attention_alibi_kats\n");
+    attention_alibi_kats(ctx);
     std::printf("relu_lowrank_fused_matches_reference\n");
     relu_lowrank_fused_matches_reference(ctx);
     std::printf("fused_attention_matches_reference\n");
