@@ -18,5 +18,5 @@ def test_cpp_host_mirror():
                                               "/opt/rocm/lib", env.get("LD_LIBRARY_PATH", "")])
     proc = subprocess.run([BIN, os.path.join(ROOT, "tests", "golden", "tiny_shakespeare")], capture_output=True, text=True, timeout=120, env=env)
     print(proc.stdout, proc.stderr)
-    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert proc.returncode == 0, f"exit status {proc.returncode}\n{proc.stdout}{proc.stderr}"
     assert proc.stdout.strip().endswith("OK")
