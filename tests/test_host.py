@@ -141,3 +141,20 @@ def test_product_does_not_import_the_oracle():
             if name.endswith((".py", ".hip", ".h", ".cpp", ".hpp")):
                 text = open(os.path.join(dirpath, name)).read()
                 assert "oracle" not in text.lower(), f"{name} mentions the oracle"
+
+
+def test_bench_refuses_more_than_one_gpu_and_fails_loudly_without_a_device():
+    """bench.py --gpus N with N > 1 exits with a message (the path has no multi-GPU part); without a HIP
+    device it fails instead of falling back to a CPU path."""
+    import subprocess
+    import sys
+
+    bench = os.path.join(ROOT, "bench.py")
+    two = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert two.returncode != 0 and "one GPU" in two.stderr and not two.stdout.strip()
+    import torch
+
+    if not torch.cuda.is_available():
+        one = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0"], capture_output=True, text=True,
+                             timeout=300)
+        assert one.returncode != 0 and "no HIP device" in one.stderr and not one.stdout.strip()
