@@ -194,4 +194,44 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
   return bdh_launch_lm_head(ctx, B, T, d, V, cur, m->w.lm_head, logits, next_tokens);
 }
 
+int bdh_model_forward_fast(bdh_model *m, const int64_t *tokens, int B, int T, int time_block_size, float *logits) {
+  if (!m) return BDH_E_INVAL;
+  bdh_ctx *ctx = m->ctx;
+  if (B < 0 || T < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative batch or time");
+  if (B == 0 || T == 0) return BDH_OK;
+  if (!tokens || !logits) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  const bdh_model_config &c = m->cfg;
+  const int d = c.n_embd, h = c.n_head, N = c.latent, V = c.vocab, L = c.n_layer;
+  const size_t M = (size_t)B * T;
+  // activation scratch: cur [M,d] | x [B,h,T,N] | xy [B,h,T,N] | attn [B,h,T,d] | attn_ln [B,h,T,d]
+  const size_t n_cur = bdh_align_up(M * d, 64), n_x = bdh_align_up(M * h * N, 64), n_a = bdh_align_up(M * h * d, 64);
+  int rc = ensure_act(m, sizeof(float) * (n_cur + 2 * n_x + 2 * n_a));
+  if (rc != BDH_OK) return rc;
+  float *cur = static_cast<float *>(m->act);
+  float *x = cur + n_cur;
+  float *xy = x + n_x;
+  float *attn = xy + n_x;
+  float *attn_ln = attn + n_a;
+  rc = bdh_launch_embed_ln(ctx, tokens, (int64_t)M, d, V, m->w.embed, cur);  // :97-100
+  if (rc != BDH_OK) return rc;
+  const int block = time_block_size > 0 ? time_block_size : 1;  // plain branch: element-wise tril(-1)
+  for (int l = 0; l < L; ++l) {  // :113
+    ReluLowrankParams px{B, 1, T, d, h, N, cur, m->w.encoder, nullptr, c.relu_threshold, 1, nullptr, 0, nullptr, x};
+    rc = bdh_launch_relu_lowrank(ctx, px);  // :114-129
+    if (rc != BDH_OK) return rc;
+    // :131  Attention::forward: all tokens at once from position 0, row-normalised
+    rc = bdh_fused_state_aligned(ctx, B, h, T, N, d, x, cur, m->freqs, c.rotary == BDH_ALIBI ? m->slopes : nullptr, block,
+                                 nullptr, 0, c.rotary, 1, attn);
+    if (rc != BDH_OK) return rc;
+    rc = bdh_launch_layer_norm(ctx, (int64_t)M * h, d, attn, attn_ln);  // :132
+    if (rc != BDH_OK) return rc;
+    ReluLowrankParams py{B, h, T, d, h, N, attn_ln, m->w.encoder_v, nullptr, c.relu_threshold, 1, nullptr, 0, x, xy};
+    rc = bdh_launch_relu_lowrank(ctx, py);  // :134-151
+    if (rc != BDH_OK) return rc;
+    rc = bdh_launch_decoder_residual(ctx, B, T, h, N, d, xy, m->w.decoder, cur);  // :153-162
+    if (rc != BDH_OK) return rc;
+  }
+  return bdh_launch_lm_head(ctx, B, T, d, V, cur, m->w.lm_head, logits, nullptr);  // :164-168
+}
+
 }  // extern "C"

@@ -27,6 +27,7 @@ EXPORTS = [
     "bdh_model_state_bytes", "bdh_model_forward", "bdh_model_forward_ex", "bdh_advance_positions",
     "bdh_sample_top_k", "bdh_recurrent_attention_lazy_alibi", "bdh_alibi_materialize", "bdh_model_forward_lazy",
     "bdh_rho_energy", "bdh_model_forward_viz", "bdh_rotate",
+    "bdh_model_forward_fast",
 ]
 
 
@@ -101,6 +102,7 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
                                                        c_int, P, P, P, P]
     lib.bdh_alibi_materialize.argtypes = [P, c_int, c_int, c_int, c_int, c_int64, P, P, P, c_int, P]
     lib.bdh_model_forward_lazy.argtypes = [P, P, c_int, c_int, P, c_int, P, c_int64, P, P, P, P]
+    lib.bdh_model_forward_fast.argtypes = [P, P, c_int, c_int, c_int, P]
     lib.bdh_rotate.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, c_int64, P, P]
     lib.bdh_rho_energy.argtypes = [P, c_int, c_int, c_int, c_int, P, c_int, P, c_int64, P, P, P]
     lib.bdh_model_forward_viz.argtypes = [P, P, c_int, c_int, P, c_int, P, c_int64, P, P, P, P, P]

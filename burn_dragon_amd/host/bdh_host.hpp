@@ -11,7 +11,7 @@
 //   FusedKernelConfig, BDHConfig           src/model/config.rs:10-164
 //   LayerState, ModelState                 src/model/state.rs:5-57
 //   Attention::{new, forward, rotate_positions, alibi_decay}
-//   BDH::{new, init_state, forward_with_state, forward, generate}
+//   BDH::{new, init_state, forward_with_state, forward, forward_fast, generate}
 //                                          src/model/bdh.rs:37-84, 91-94, 170-256, 309-450
 //   ModelOverrides, build_model_config     src/config/core.rs:43-53, src/inference.rs:4-40
 // Contract violations that panic in the reference throw std::logic_error here; failures of the
@@ -466,6 +466,25 @@ class BDH {
   Tensor forward(const std::vector<int64_t> &tokens, size_t batch, size_t time) {
     ModelState st = init_state();
     return forward_with_state(tokens, batch, time, st);
+  }
+
+  // BDH::forward_fast (src/model/bdh.rs:96-168): the stateless forward over all tokens at once
+  Tensor forward_fast(const std::vector<int64_t> &tokens, size_t batch, size_t time) {
+    if (tokens.size() != batch * time) throw std::logic_error("tokens do not match [batch, time]");
+    const auto &k = config_.fused_kernels;
+    if (k.enabled && (k.block_sparse.latent.is_sparse() || k.block_sparse.time.is_sparse()))
+      throw std::logic_error("forward_fast takes dense block patterns");
+    Tensor logits({batch, time, config_.vocab_size});
+    if (tokens.empty()) return logits;
+    int64_t *tok_dev = nullptr;
+    hip_check(hipMalloc(reinterpret_cast<void **>(&tok_dev), sizeof(int64_t) * tokens.size()), "hipMalloc");
+    hip_check(hipMemcpy(tok_dev, tokens.data(), sizeof(int64_t) * tokens.size(), hipMemcpyHostToDevice), "hipMemcpy");
+    const int block = k.enabled ? (int)std::max<size_t>(k.block_sparse.time.block_size(), 1) : 0;
+    const int rc = bdh_model_forward_fast(model_, tok_dev, (int)batch, (int)time, block, logits.data());
+    ctx_.synchronize();
+    (void)hipFree(tok_dev);
+    ctx_.check(rc);
+    return logits;
   }
 
   // greedy form (top_k = 1) of BDH::generate; batch must be 1 as in the reference

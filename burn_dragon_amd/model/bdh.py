@@ -154,6 +154,21 @@ class BDH:
         """src/model/bdh.rs:91-94."""
         return self.forward_with_state(tokens, self.init_state())
 
+    def forward_fast(self, tokens: torch.Tensor) -> torch.Tensor:
+        """src/model/bdh.rs:96-168: the stateless forward over all tokens at once (the form the reference
+        trains with): Attention::forward in place of the recurrent state.  tokens [B,T] -> logits [B,T,V]."""
+        if self.kernel.enabled and (self.kernel.block_sparse.latent.is_sparse() or
+                                    self.kernel.block_sparse.time.is_sparse()):
+            raise NotImplementedError("forward_fast takes dense block patterns (build_model_config makes no others); "
+                                      "sparse patterns are available through kernel.relu_lowrank / linear_attention")
+        tokens = tokens.to(self.device, torch.int64).contiguous()
+        B, T = tokens.shape
+        logits = torch.empty((B, T, self.vocab_size), device=self.device, dtype=torch.float32)
+        block = max(self.kernel.block_sparse.time.block_size, 1) if self.kernel.enabled else 0
+        self.ctx.check(self.ctx.lib.bdh_model_forward_fast(self.handle, tokens.data_ptr(), B, T, block,
+                                                           logits.data_ptr()))
+        return logits
+
     def generate(self, indices: torch.Tensor, max_new_tokens: int, temperature: float = 1.0,
                  top_k: Optional[int] = 1, generator: Optional[torch.Generator] = None) -> torch.Tensor:
         """src/model/bdh.rs:170-252: prompt through forward_with_state, then max_new_tokens draws from

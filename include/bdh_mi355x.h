@@ -262,6 +262,15 @@ int bdh_model_forward_ex(bdh_model *model, const int64_t *tokens, int B, int T, 
                          int rho_dtype, int64_t position, const int32_t *positions_dev,
                          float *logits, int64_t *next_tokens, float *x_tap);
 
+/* Replaces BDH::forward_fast (src/model/bdh.rs:96-168), the stateless forward over all tokens at once
+ * that the reference trains with: the same layer as bdh_model_forward, but the attention is
+ * Attention::forward (row-normalised causal scores from position 0, bdh_fused_state_aligned) instead of
+ * the recurrent state.  time_block_size > 0 selects the fused branch with dense time blocks of that
+ * size (FusedKernelConfig.enabled; the latent block pattern is dense, as build_model_config makes it);
+ * <= 0 the plain branch.  tokens [B,T] int64 -> logits [B,T,V].  Inference only: no gradients. */
+int bdh_model_forward_fast(bdh_model *model, const int64_t *tokens, int B, int T, int time_block_size,
+                           float *logits);
+
 /* positions_dev[b] = saturating(positions_dev[b] + delta): the device-side form of
  * `state.position += T` (src/model/bdh.rs:445). */
 int bdh_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta);

@@ -55,6 +55,9 @@
  *                              for top_k = 1, draw frequencies (tests/test_oracle.py);
  *                              the reference's own draw uses thread_rng and cannot be
  *                              replayed
+ *   forward_fast (numpy only,  composition of the pinned relu_lowrank, attention_forward /
+ *   oracle/bdh_oracle.py)      fused_state_aligned and layer_norm; the reference checks its shape
+ *                              only (tests/model_paths.rs:48,81): "parity unpinned" as a whole
  *   orc_rho_energy,            pinned: numpy float64 mean(|rho|) over d and the batch;
  *   orc_forward_with_state_viz the other three taps are slices of x, y and x*y of the
  *                              pinned forward pass, checked against the numpy

@@ -314,6 +314,36 @@ def forward_with_state(shape: BDHShape, w: BDHWeights, tokens, state: ModelState
     return np.matmul(cur.reshape(B * T, d), w.lm_head).reshape(B, T, shape.vocab_size)  # :446-449
 
 
+def forward_fast(shape: BDHShape, w: BDHWeights, tokens, fused: bool = False, time_block: int = 64):
+    """src/model/bdh.rs:96-168, numpy statement: the stateless forward over all tokens at once, a
+    composition of relu_lowrank, Attention::forward (plain branch) or fused_state_aligned (fused branch),
+    layer_norm and two matmuls.  tokens [B,T] ints -> logits [B,T,V].  The parts are pinned (see the C
+    file's header); the reference itself checks only the shape of the result (tests/model_paths.rs:48,81),
+    so the composition as a whole is "parity unpinned"."""
+    dtype = w.encoder.dtype
+    tokens = np.asarray(tokens)
+    B, T = tokens.shape
+    h, d, N = shape.n_head, shape.n_embd, shape.latent_per_head
+    cur = layer_norm(w.embed[tokens].reshape(B, 1, T, d))  # :97-100
+    freqs = build_freqs(N, shape.rope_theta, shape.rotary, dtype)
+    slopes = None
+    if shape.rotary == ALIBI:
+        slopes = default_alibi_slopes(h, dtype) if shape.alibi_slopes is None else np.asarray(shape.alibi_slopes, dtype)
+    for _ in range(shape.n_layer):
+        x = relu_lowrank(cur, w.encoder, None, shape.relu_threshold)  # :114-129
+        if fused:  # :131, src/model/attention.rs:142-152
+            attn = fused_state_aligned(x, cur[:, 0], freqs, slopes, time_block, shape.rotary)
+        else:  # src/model/attention.rs:154-174
+            attn = attention_forward(x, cur[:, 0], freqs, slopes, shape.rotary, True)
+        attn = layer_norm(attn.astype(dtype))  # :132
+        y = relu_lowrank(attn, w.encoder_v, None, shape.relu_threshold)  # :134-151
+        xy = x * y
+        mixed = np.swapaxes(xy, 1, 2).reshape(B * T, h * N)  # :156-160
+        mlp = layer_norm(np.matmul(mixed, w.decoder).reshape(B, 1, T, d))  # :162-164
+        cur = layer_norm(cur + mlp)  # :165
+    return np.matmul(cur.reshape(B * T, d), w.lm_head).reshape(B, T, shape.vocab_size)  # :168-172
+
+
 def rho_energy(rho):
     """src/model/bdh.rs:411-419: [B,h,N,d] -> [h,N], mean over the batch of the per-row mean |rho|."""
     B, _, _, d = rho.shape

@@ -97,6 +97,12 @@ static void inference_paths_run_across_configs(const Context &ctx) {
                      randn(g, d * V, 0.02f)};
     BDH model(ctx, config, w);
     const std::vector<int64_t> tokens{0, 1, 2, 3, 4, 5, 6, 7};
+    {  // tests/model_paths.rs:77-79: the stateless forward of the same configuration
+      Tensor fast = model.forward_fast(tokens, 2, 4);
+      EXPECT((fast.shape() == std::vector<size_t>{2, 4, 32}));
+      const std::vector<float> fv = fast.to_host();
+      EXPECT(std::all_of(fv.begin(), fv.end(), [](float v) { return std::isfinite(v); }));
+    }
     ModelState state = model.init_state();
     Tensor logits = model.forward_with_state(tokens, 2, 4, state);
     EXPECT((logits.shape() == std::vector<size_t>{2, 4, 32}));

@@ -125,15 +125,21 @@ def _model_pair(bda, cfg, seed):
     return shape, w, model
 
 
-@pytest.mark.parametrize("rotary", ["rope", "pope", "alibi"])
-def test_inference_paths_run_across_configs(bda, corc, rotary):
-    """tests/model_paths.rs:66-91: L=2, d=16, h=2, mult=4, V=32, tokens [[0,1,2,3],[4,5,6,7]] ->
-    logits [2,4,32], state.position == 4 — plus the values, against the oracle."""
+@pytest.mark.parametrize("rotary,fused", [("rope", False), ("pope", False), ("alibi", False), ("alibi", True)])
+def test_inference_paths_run_across_configs(bda, corc, rotary, fused):
+    """tests/model_paths.rs:66-91: L=2, d=16, h=2, mult=4, V=32, tokens [[0,1,2,3],[4,5,6,7]], the four
+    (rotary, fused) configurations -> forward_fast logits [2,4,32]; forward_with_state logits [2,4,32],
+    state.position == 4 — plus the values, against the oracle."""
     cfg = bda.BDHConfig(n_layer=2, n_embd=16, n_head=2, mlp_internal_dim_multiplier=4, vocab_size=32, dropout=0.0)
+    cfg.fused_kernels.enabled = fused
     cfg.fused_kernels.set_block_sizes(4, 4)
     cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse(rotary))
     shape, w, model = _model_pair(bda, cfg, seed=11)
     tokens = np.arange(8).reshape(2, 4)
+    logits_fast = model.forward_fast(torch.from_numpy(tokens))
+    assert tuple(logits_fast.shape) == (2, 4, 32)
+    fast_ref = orc.forward_fast(shape, w, tokens, fused=fused, time_block=4)
+    assert rel_err(logits_fast.cpu().numpy(), fast_ref) < 1e-3
     state = model.init_state()
     logits = model.forward_with_state(torch.from_numpy(tokens), state)
     torch.cuda.synchronize()
@@ -184,6 +190,21 @@ def test_long_prompt_takes_the_dense_chunk_form(bda, corc, rotary):
     logits2_ref, pos, _, _ = corc.forward_with_state(shape, w, more, rho_ref, pos, sparse_state=False)
     assert state.position == 151 == pos
     assert rel_err(logits2.cpu().numpy(), logits2_ref) < 1e-3
+
+
+def test_forward_fast_long_sequence_on_the_matrix_cores(bda):
+    """T = 160 takes the f32 matrix-core form of fused_state_aligned inside forward_fast; both branches against
+    the numpy composition."""
+    cfg = bda.BDHConfig(n_layer=2, n_embd=32, n_head=2, mlp_internal_dim_multiplier=8, vocab_size=64, dropout=0.0)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse("rope"))
+    tokens = np.random.default_rng(2).integers(0, 64, (2, 160))
+    for fused in (False, True):
+        cfg.fused_kernels.enabled = fused
+        cfg.fused_kernels.set_block_sizes(32, 32)
+        shape, w, model = _model_pair(bda, cfg, seed=31)
+        got = model.forward_fast(torch.from_numpy(tokens)).cpu().numpy()
+        want = orc.forward_fast(shape, w, tokens, fused=fused, time_block=32)
+        assert rel_err(got, want) < 1e-3
 
 
 def test_config1_architecture_prefill_and_greedy_decode(bda, corc):

@@ -405,6 +405,30 @@ def test_forward_viz_taps(corc, rotary):
             np.testing.assert_allclose(viz[l, 3], np.abs(rho[l].astype(np.float64)).mean(3).mean(0), rtol=1e-5)
 
 
+@pytest.mark.parametrize("rotary,fused", [(ROPE, False), (POPE, False), (ALIBI, False), (ALIBI, True)])
+def test_forward_fast_shapes_and_relation_to_the_parts(rotary, fused):
+    """tests/model_paths.rs:44-50,77-83: tokens [[0,1,2,3],[4,5,6,7]] -> logits [2,4,32] for the four
+    configurations; the first token's attention row is empty, so its logits are those of a model whose
+    attention output is zero (LN(0) = 0 -> y = relu(0) = 0 -> the layer is the identity on LN(embed))."""
+    shape = _small_shape(rotary)
+    w = orc.init_weights(shape, seed=3)
+    tokens = np.arange(8).reshape(2, 4)
+    logits = orc.forward_fast(shape, w, tokens, fused=fused, time_block=4)
+    assert logits.shape == (2, 4, 32) and np.isfinite(logits).all()
+    if not (fused and rotary == ALIBI):  # the fused ALiBi branch lets row 0 see its block through the bias
+        cur0 = orc.layer_norm(w.embed[tokens[:, 0]])
+        for _ in range(shape.n_layer):
+            cur0 = orc.layer_norm(cur0 + orc.layer_norm(np.zeros_like(cur0)))
+        np.testing.assert_allclose(logits[:, 0], cur0 @ w.lm_head, atol=1e-5)
+    # causal: changing the last token leaves the earlier positions alone
+    tokens2 = tokens.copy()
+    tokens2[:, -1] = [9, 10]
+    logits2 = orc.forward_fast(shape, w, tokens2, fused=fused, time_block=4)
+    if not (fused and rotary == ALIBI):
+        np.testing.assert_array_equal(logits2[:, :-1], logits[:, :-1])
+    assert not np.array_equal(logits2[:, -1], logits[:, -1])
+
+
 def test_forward_rejects_bad_token(corc):
     shape = _small_shape(ROPE)
     w = orc.init_weights(shape, seed=4)
