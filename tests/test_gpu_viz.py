@@ -137,3 +137,24 @@ def test_viz_taps_on_the_trained_checkpoint(bda, corc):
         frac_x = float((m.x_last > 0).float().mean())
         frac_xy = float((m.xy_last > 0).float().mean())
         assert frac_xy <= frac_x < 0.6
+
+
+def test_viz_state_collects_last_token(bda):
+    """src/viz/encoder.rs:314-348, the reference's own test of LayerVizState: L=2, d=8, h=2, mult=2, V=16,
+    default (ALiBi) kernel config with fused kernels off, tokens [[1,2,3]] -> one LayerVizState per layer
+    whose four maps are [n_head, latent_per_head]."""
+    config = bda.BDHConfig()
+    config.n_layer, config.n_embd, config.n_head = 2, 8, 2
+    config.mlp_internal_dim_multiplier, config.vocab_size, config.dropout = 2, 16, 0.0
+    config.fused_kernels.enabled = False
+    model = bda.BDH(config, DEV)
+    state = bda.ModelState.new(config.n_layer)
+    model.forward_with_state(torch.tensor([[1, 2, 3]]), state, viz=True)
+    layers = state.take_viz()
+    assert len(layers) == config.n_layer
+    for layer in layers:
+        assert layer is not None, "expected viz state per layer"
+        dims = tuple(layer.x_last.shape)
+        assert dims == (config.n_head, config.latent_per_head())
+        assert tuple(layer.y_last.shape) == dims and tuple(layer.xy_last.shape) == dims
+        assert tuple(layer.rho_last.shape) == dims
