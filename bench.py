@@ -380,22 +380,35 @@ def bench_model(args):
     import burn_dragon_amd as bda
 
     dev = torch.device("cuda:0")
-    if args.model_config == "c1":
-        cfg = bda.BDHConfig(n_layer=6, n_embd=256, n_head=4, mlp_internal_dim_multiplier=128, vocab_size=256)
+    rho_dtype = bda.ffi.F32 if args.rho_dtype == "f32" else bda.ffi.BF16
+    weights_note = "random-init weights (about half the neurons active)"
+    if args.model_config == "ckpt":
+        # the trained checkpoint the reference ships (tiny_shakespeare: L=4, d=128, h=4, N=128, V=69, ALiBi),
+        # a copy of which the tests hold as a data fixture; state kept lazily decayed
+        directory = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden", "tiny_shakespeare")
+        model, tok, _ = bda.BDH.from_checkpoint_dir(directory, dev, rho_dtype=rho_dtype, alibi_lazy=True)
+        cfg = model.config
         B = 1 if args.batch == 32 else args.batch
         steps = 256 if args.steps == 1000 else args.steps
+        text = ("First Citizen:\nBefore we proceed any further, hear me speak.\n\nAll:\nSpeak, speak.\n" * 8)[:args.prompt]
+        prompt = torch.tensor([tok.encode(text)] * B)
+        weights_note = "trained tiny_shakespeare checkpoint (ALiBi, lazily decayed state)"
     else:
-        cfg = bda.BDHConfig(n_layer=12, n_embd=512, n_head=8, mlp_internal_dim_multiplier=256, vocab_size=256)
-        B = args.batch
-        steps = 64 if args.steps == 1000 else args.steps
-    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
-    rho_dtype = bda.ffi.F32 if args.rho_dtype == "f32" else bda.ffi.BF16
-    model = bda.BDH(cfg, dev, seed=7, rho_dtype=rho_dtype)
-    prompt = torch.randint(0, 256, (B, args.prompt), generator=torch.Generator().manual_seed(1))
+        if args.model_config == "c1":
+            cfg = bda.BDHConfig(n_layer=6, n_embd=256, n_head=4, mlp_internal_dim_multiplier=128, vocab_size=256)
+            B = 1 if args.batch == 32 else args.batch
+            steps = 256 if args.steps == 1000 else args.steps
+        else:
+            cfg = bda.BDHConfig(n_layer=12, n_embd=512, n_head=8, mlp_internal_dim_multiplier=256, vocab_size=256)
+            B = args.batch
+            steps = 64 if args.steps == 1000 else args.steps
+        cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+        model = bda.BDH(cfg, dev, seed=7, rho_dtype=rho_dtype)
+        prompt = torch.randint(0, 256, (B, args.prompt), generator=torch.Generator().manual_seed(1))
     state = model.init_state()
     chunk = args.prefill_chunk or args.prompt
     t0 = time.perf_counter()
-    for lo in range(0, args.prompt, chunk):  # bounded activation memory; same result as one call
+    for lo in range(0, prompt.shape[1], chunk):  # bounded activation memory; same result as one call
         _, nxt = model.forward_with_state(prompt[:, lo:lo + chunk], state, want_next=True)
         if (lo // chunk) % 16 == 15:
             torch.cuda.synchronize()
@@ -427,10 +440,10 @@ def bench_model(args):
         "metric": "decode tokens/sec, full model, greedy", "value": B / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.rho_dtype, "data": "synthetic",
-        "config": {"workload": f"full-model greedy decode {args.model_config}: L={L} d={d} h={h} N={N} V=256 B={B}, "
-                               f"random-init weights (about half the neurons active), prompt {args.prompt} tokens"
+        "config": {"workload": f"full-model greedy decode {args.model_config}: L={L} d={d} h={h} N={N} "
+                               f"V={cfg.vocab_size} B={B}, {weights_note}, prompt {prompt.shape[1]} tokens"
                                + (", one HIP graph replay per token" if args.graph else ", eager launches"),
-                   "prefill_seconds": prefill_s, "prefill_tokens_per_s": B * args.prompt / prefill_s,
+                   "prefill_seconds": prefill_s, "prefill_tokens_per_s": B * prompt.shape[1] / prefill_s,
                    "state_bytes": L * B * h * N * d * (4 if args.rho_dtype == "f32" else 2)},
         **extra,
     }))
@@ -457,7 +470,8 @@ def main():
                          "alibi = ALiBi state step, lazily decayed state beside the eager dense decay; "
                          "parallel = fused_state_aligned in f32 at the config-3 shape; chunks = many-token state step "
                          "(f32 dense products) beside the token loop at the config-2 shape; copy = counter calibration")
-    ap.add_argument("--model-config", choices=["c1", "c4"], default="c1")
+    ap.add_argument("--model-config", choices=["c1", "c4", "ckpt"], default="c1",
+                    help="model: config 1, config 4, or the trained tiny_shakespeare checkpoint of the test fixtures")
     ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
     ap.add_argument("--graph", action="store_true", help="model: replay one captured HIP graph per token")
     ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")
