@@ -447,3 +447,51 @@ def test_dense_chunk_form_on_a_lazily_decayed_alibi_state(gpu, corc):
     assert rel_err(out1.cpu().numpy(), out_ref[:, :, T:]) < 1e-4
     assert rel_err(rt.cpu().numpy(), rho_ref) < 1e-4
     assert (st.cpu().numpy() == clock + T + 1).all()
+
+
+def test_dense_chunk_form_equals_token_loop_on_ragged_shapes(gpu, corc):
+    """Sixteen seeded shapes with every dimension ragged (tile edges, odd d, a single token, more than one
+    chunk), all three rotaries: the dense form and the token loop of the step kernels agree to f32
+    reassociation on the device, and the first shapes also against the oracle."""
+    ffi, recurrent_attention = gpu
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    ctx = ffi.default_context(0)
+    rng = np.random.default_rng(2024)
+    dev = "cuda:0"
+    for case in range(16):
+        B, h = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        T = int(rng.choice([1, 2, 17, 127, 128, 129, 255, 300, 513, 640]))
+        N = 2 * int(rng.integers(1, 100))
+        d = int(rng.choice([1, 3, 4, 8, 20, 33, 64, 70, 128, 132]))
+        rotary = int(rng.integers(0, 3))
+        density = float(rng.choice([0.0, 0.1, 0.5, 1.0]))
+        x, v, _ = make_inputs(1000 + case, B, h, T, N, d, density)
+        Nq = 2 * N if rotary == orc.POPE else N
+        rho0 = (0.05 * rng.standard_normal((B, h, Nq, d))).astype(np.float32)
+        freqs = corc.build_freqs(N, rotary=rotary)
+        slopes = np.array([0.03 * (i + 1) for i in range(h)], np.float32) if rotary == orc.ALIBI else None
+        position = int(rng.integers(0, 5000))
+        label = f"case {case}: B={B} h={h} T={T} N={N} d={d} rotary={rotary} density={density}"
+        print(label, flush=True)
+        res = []
+        for mode in (0, 1):
+            ctx.set_option("state_step.dense_chunks", mode)
+            try:
+                rt = torch.from_numpy(rho0).to(dev).contiguous()
+                out = recurrent_attention(torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev), rt,
+                                          torch.from_numpy(freqs).to(dev), position, RotaryEmbedding(rotary), slopes)
+                torch.cuda.synchronize()
+            finally:
+                ctx.set_option("state_step.dense_chunks", -1)
+            res.append((out.cpu().numpy(), rt.cpu().numpy()))
+        tol = 1e-4 if rotary == orc.ALIBI else 2e-5
+        scale_o = max(np.abs(res[0][0]).max(), 1e-6)
+        scale_r = max(np.abs(res[0][1]).max(), 1e-6)
+        assert np.abs(res[1][0] - res[0][0]).max() <= tol * scale_o, label
+        assert np.abs(res[1][1] - res[0][1]).max() <= tol * scale_r, label
+        if case < 6:
+            q = corc.rotate(x, freqs, rotary, position)
+            out_ref, rho_ref = corc.recurrent_attention(q, v, rho0.copy(), None if slopes is None else corc.alibi_decay(slopes))
+            assert np.abs(res[1][0] - out_ref).max() <= tol * max(np.abs(out_ref).max(), 1e-6), label
+            assert np.abs(res[1][1] - rho_ref).max() <= tol * max(np.abs(rho_ref).max(), 1e-6), label
