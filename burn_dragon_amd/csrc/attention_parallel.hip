@@ -102,6 +102,25 @@ __global__ __launch_bounds__(256) void k_set_stamps(int32_t *__restrict__ stamps
   stamps[i] = (int32_t)min(c, 0x7fffffffL);
 }
 
+// bf16 <-> f32 copies of a whole state (grid-stride); f32 -> bf16 rounds to nearest even
+__global__ __launch_bounds__(256) void k_widen_bf16(const unsigned short *__restrict__ in, float *__restrict__ out,
+                                                    size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    out[i] = __uint_as_float(static_cast<unsigned int>(in[i]) << 16);
+}
+__global__ __launch_bounds__(256) void k_narrow_bf16(const float *__restrict__ in, unsigned short *__restrict__ out,
+                                                     size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    unsigned int u = __float_as_uint(in[i]);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+      out[i] = static_cast<unsigned short>((u >> 16) | 0x40);
+    } else {
+      u += 0x7fffu + ((u >> 16) & 1u);
+      out[i] = static_cast<unsigned short>(u >> 16);
+    }
+  }
+}
+
 // one workgroup per (slice, query row i)
 __global__ __launch_bounds__(256) void k_fsa_row(const float *__restrict__ q, const float *__restrict__ v,
                                                  const float *__restrict__ slopes_dev, int use_alibi, int h,
@@ -552,7 +571,7 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
   const int B = p.B, h = p.h, T = p.T, N = p.N, d = p.d;
   const int Nq = p.rotary == BDH_POPE ? 2 * N : N;
   const long S = (long)B * h;
-  if (p.rho_dtype != BDH_F32) return bdh_fail(ctx, BDH_E_INVAL, "the chunked f32 form needs an f32 state");
+  const bool bf16_state = p.rho_dtype == BDH_BF16;
   const bool alibi = p.rotary == BDH_ALIBI;
   if (p.stamps && !alibi) return bdh_fail(ctx, BDH_E_INVAL, "decay stamps only apply to ALiBi");
   float log_decay[64] = {0};
@@ -572,11 +591,21 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
   const int Tcp = ((int)Tc + 3) & ~3;
   const size_t q_bytes = alibi ? 0 : bdh_align_up(per_token * (size_t)Tc, 256);  // ALiBi does not rotate: q = x
   const size_t sc_bytes = bdh_align_up(sizeof(float) * (size_t)S * Tc * Tcp, 256);
-  int rc = bdh_ws_reserve(ctx, q_bytes + sc_bytes);
+  // a bf16 state is widened to f32 for the call and rounded back once at its end (the token loop rounds
+  // after every token)
+  const size_t n_state = (size_t)S * Nq * d;
+  const size_t wide_bytes = bf16_state ? bdh_align_up(sizeof(float) * n_state, 256) : 0;
+  int rc = bdh_ws_reserve(ctx, q_bytes + sc_bytes + wide_bytes);
   if (rc != BDH_OK) return rc;
   float *q = static_cast<float *>(ctx->ws);
   float *scores = reinterpret_cast<float *>(static_cast<char *>(ctx->ws) + q_bytes);
   float *rho = static_cast<float *>(p.rho);
+  if (bf16_state) {
+    rho = reinterpret_cast<float *>(static_cast<char *>(ctx->ws) + q_bytes + sc_bytes);
+    hipLaunchKernelGGL(k_widen_bf16, dim3((unsigned)std::min<size_t>((n_state + 255) / 256, 1u << 20)), dim3(256), 0,
+                       ctx->stream, static_cast<const unsigned short *>(p.rho), rho, n_state);
+    BDH_LAUNCH_CHECK(ctx, "k_widen_bf16");
+  }
   const unsigned groups = (unsigned)((S + 7) / 8);
   const int nt_d = (d + 127) / 128;
   if ((long)groups * 8 * ((Nq + 127) / 128) * nt_d > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
@@ -653,6 +682,11 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
                          ctx->stream, g);
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q^T V>");
     }
+  }
+  if (bf16_state) {
+    hipLaunchKernelGGL(k_narrow_bf16, dim3((unsigned)std::min<size_t>((n_state + 255) / 256, 1u << 20)), dim3(256), 0,
+                       ctx->stream, rho, static_cast<unsigned short *>(p.rho), n_state);
+    BDH_LAUNCH_CHECK(ctx, "k_narrow_bf16");
   }
   if (p.stamps) {  // every row is now up to date as of the end of the call
     const long rows = S * N;

@@ -856,10 +856,11 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
     }
     return BDH_OK;
   }
-  // many tokens, f32 state, no per-token by-products: the dense form on the f32 matrix cores
+  // many tokens, no per-token by-products: the dense form on the f32 matrix cores (a bf16 state is widened for the call)
   // (not when even a 128-token chunk of rotated activations would pass 16 GiB of workspace)
-  const bool chunk_fits = sizeof(float) * (size_t)slices * Nq * 128 <= (size_t(16) << 30);
-  if (p.rho_dtype == BDH_F32 && !p.bitmask && !p.rows_touched && chunk_fits &&
+  const bool chunk_fits = sizeof(float) * (size_t)slices * Nq * 128 <= (size_t(16) << 30) &&
+                          (p.rho_dtype == BDH_F32 || sizeof(float) * (size_t)slices * Nq * d <= (size_t(64) << 30));
+  if (!p.bitmask && !p.rows_touched && chunk_fits &&
       (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : T >= 128))
     return bdh_launch_state_chunks_f32(ctx, p, out_ln);
   // tokens per launch: only the f32 RoPE kernel walks several, as many as 64 MiB of partials allow

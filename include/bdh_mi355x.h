@@ -68,7 +68,7 @@ const char *bdh_last_error(const bdh_ctx *ctx);
 /* Launch-shape knobs for tests and tuning; no counterpart in the reference.
  *   "state_step.split": -1 (default) pick by grid size, 0 = 256 lane pairs per workgroup,
  *                       1 = 64 lane pairs per workgroup of 8 waves (small batches).
- *   "state_step.dense_chunks": -1 (default) a call of 128+ tokens on an f32 state without
+ *   "state_step.dense_chunks": -1 (default) a call of 128+ tokens without
  *                       bitmask / row-count outputs runs as dense products on the f32 matrix cores,
  *                       0 = always token by token, 1 = dense products for any T.
  *   "relu_lowrank.tile": 1 (default) calls with 64+ rows take the 64-row tile kernel (same values),
@@ -120,10 +120,11 @@ int bdh_rotate(bdh_ctx *ctx, int B, int h, int T, int N, int rotary, const float
  *                        element; ALiBi/PoPE: Nq)
  *
  * RoPE requires even N (src/model/attention.rs:310).  T = 1 is the decode step.  A call of 128 or more
- * tokens on an f32 state that asks for neither bitmask nor row counts computes the same sums as dense
+ * tokens that asks for neither bitmask nor row counts computes the same sums as dense
  * products (out = tril(-1)(Q Q^T) V + Q rho, rho += Q^T V, chunks of up to 512 tokens; for ALiBi with
  * the decay powers decay^(t-s), decay^t and decay^(T-s) applied to the three terms) on the f32 matrix
- * cores; results agree with the token loop to f32 reassociation (option "state_step.dense_chunks").
+ * cores (a bf16 state is widened to f32 for the call and rounded once at its end); results agree with
+ * the token loop to f32 reassociation (option "state_step.dense_chunks").
  */
 int bdh_recurrent_attention(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary,
                             const float *x, const float *v, const float *freqs,

@@ -495,3 +495,33 @@ def test_dense_chunk_form_equals_token_loop_on_ragged_shapes(gpu, corc):
             out_ref, rho_ref = corc.recurrent_attention(q, v, rho0.copy(), None if slopes is None else corc.alibi_decay(slopes))
             assert np.abs(res[1][0] - out_ref).max() <= tol * max(np.abs(out_ref).max(), 1e-6), label
             assert np.abs(res[1][1] - rho_ref).max() <= tol * max(np.abs(rho_ref).max(), 1e-6), label
+
+
+@pytest.mark.parametrize("rotary", [orc.ROPE, orc.ALIBI])
+def test_dense_chunk_form_with_a_bf16_state(gpu, corc, rotary):
+    """bf16 storage in the many-token form: the state is widened to f32 for the call and rounded once at its
+    end, so it lands within one bf16 rounding of the f32 result (the token loop rounds after every token);
+    2e-2 relative (north_star) against the oracle."""
+    _, recurrent_attention = gpu
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    B, h, T, N, d = 2, 2, 200, 128, 64
+    x, v, rho0 = make_inputs(321, B, h, T, N, d, 0.2, rho_scale=0.05)
+    rho_b = torch.from_numpy(rho0).to(torch.bfloat16)
+    freqs = corc.build_freqs(N, rotary=rotary)
+    slopes = np.array([0.02, 0.05], np.float32) if rotary == orc.ALIBI else None
+    dev = "cuda:0"
+    rt = rho_b.to(dev).contiguous()
+    out = recurrent_attention(torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev), rt,
+                              torch.from_numpy(freqs).to(dev), 5, RotaryEmbedding(rotary), slopes)
+    torch.cuda.synchronize()
+    assert rt.dtype == torch.bfloat16
+    q = corc.rotate(x, freqs, rotary, 5)
+    out_ref, rho_ref = corc.recurrent_attention(q, v, rho_b.float().numpy().copy(),
+                                                None if slopes is None else corc.alibi_decay(slopes))
+    assert rel_err(out.cpu().numpy(), out_ref) < 1e-4  # the readouts never see a rounded state inside the call
+    got = rt.float().cpu().numpy()
+    assert rel_err(got, rho_ref) < 2e-2
+    # exactly the f32 result rounded to bf16, up to f32 reassociation before the rounding
+    want = torch.from_numpy(rho_ref).to(torch.bfloat16).float().numpy()
+    assert (got != want).mean() < 0.02
