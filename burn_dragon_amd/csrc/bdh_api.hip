@@ -122,6 +122,11 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     ctx->opt_decoder_mfma = value;
     return BDH_OK;
   }
+  if (strcmp(name, "relu_lowrank.scalar") == 0) {
+    if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "relu_lowrank.scalar takes 0 or 1");
+    ctx->opt_lowrank_scalar = value;
+    return BDH_OK;
+  }
   if (strcmp(name, "fused_state_aligned.path") == 0) {
     if (value < -1 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "fused_state_aligned.path takes -1, 0 or 1");
     ctx->opt_fsa_path = value;

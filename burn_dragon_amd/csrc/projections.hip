@@ -91,6 +91,73 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank(const float *__restrict__
   }
 }
 
+// A few input rows (a batch of 8 to 63 sequences decoding together) without LDS: the inputs of a row tile
+// are the same for every lane, so they are read through the scalar cache (wave-uniform addresses, read
+// only) and feed the FMAs as scalar operands; the vector memory pipe carries only the weights.  With the
+// inputs staged in LDS instead, three quarters of the wave wait cycles were waits for the broadcast reads.
+// Same k-sequential fmaf chain per output as k_relu_lowrank.
+template <int RT, int UK>
+__global__ __launch_bounds__(256) void k_relu_lowrank_sc(const float *__restrict__ in, int h_in, int T, int d,
+                                                        const float *__restrict__ w, int h, int N,
+                                                        const float *__restrict__ bias, float thr,
+                                                        const unsigned char *__restrict__ block_active,
+                                                        int block_size, int n_blocks,
+                                                        const float *__restrict__ gate, float *__restrict__ out,
+                                                        int M) {
+  const int hh = blockIdx.y;
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  const int m0 = blockIdx.z * RT;
+  if (n >= N) return;
+  const float *rows[RT];  // wave-uniform row pointers (rows past M alias the last valid row; never stored)
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int m = min(m0 + r, M - 1);
+    const int b = m / T, t = m - b * T;
+    rows[r] = in + (((long)b * h_in + (h_in == 1 ? 0 : hh)) * T + t) * d;
+  }
+  float acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = 0.0f;
+  const float *wp = w + (long)hh * d * N + n;
+  int k0 = 0;
+  for (; k0 + UK <= d; k0 += UK) {
+    float wv[UK];
+#pragma unroll
+    for (int u = 0; u < UK; ++u) wv[u] = wp[(long)(k0 + u) * N];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+#pragma unroll
+      for (int u = 0; u < UK; ++u) acc[r] = __builtin_fmaf(rows[r][k0 + u], wv[u], acc[r]);
+    }
+  }
+  for (; k0 < d; ++k0) {
+    const float wv = wp[(long)k0 * N];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) acc[r] = __builtin_fmaf(rows[r][k0], wv, acc[r]);
+  }
+  const float bv = bias ? bias[(long)hh * N + n] : 0.0f;
+  float maskv = 1.0f;
+  if (block_active) {
+    const int blk = n / block_size;
+    maskv = (blk < n_blocks && block_active[blk]) ? 1.0f : 0.0f;
+  }
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int m = m0 + r;
+    if (m < M) {
+      const int b = m / T, t = m - b * T;
+      float p = acc[r];
+      if (bias) p = p + bv;
+      if (thr != 0.0f) p = p - thr;
+      float y = p > 0.0f ? p : 0.0f;
+      if (block_active) y = y * maskv;
+      const long o = (((long)b * h + hh) * T + t) * N + n;
+      if (gate) y = gate[o] * y;
+      out[o] = y;
+    }
+  }
+}
+
 // Many input rows (a prompt, a large batch): a 64-row x 256-column tile per workgroup, 16 rows x 4
 // adjacent columns per thread.  Wave w owns rows 16w..16w+15, so an input value is one LDS broadcast
 // for the whole wave; a weight row segment is one float4 per lane.  The inputs are staged 64 k at a
@@ -528,6 +595,21 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
                        p.in, p.h_in, p.T, p.d, p.weight, p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks,
                        p.gate, p.out, (int)M);
     BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_tile");
+    return BDH_OK;
+  }
+  if (M >= 8 && ctx->opt_lowrank_scalar != 0) {
+    // 8 to 63 rows: inputs through the scalar cache, 16 rows (two SGPR batches of 8 k) or 8 rows per pass
+    const int rt = M >= 16 ? 16 : 8;
+    const long row_tiles = (M + rt - 1) / rt;
+    if (row_tiles > 65535 || p.h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (row tiles %ld)", row_tiles);
+    const dim3 grid((p.N + 255) / 256, p.h, (unsigned)row_tiles);
+    if (rt == 16)
+      hipLaunchKernelGGL((k_relu_lowrank_sc<16, 8>), grid, dim3(256), 0, ctx->stream, p.in, p.h_in, p.T, p.d, p.weight,
+                         p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M);
+    else
+      hipLaunchKernelGGL((k_relu_lowrank_sc<8, 8>), grid, dim3(256), 0, ctx->stream, p.in, p.h_in, p.T, p.d, p.weight,
+                         p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M);
+    BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_sc");
     return BDH_OK;
   }
   const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));

@@ -53,7 +53,8 @@ def test_relu_lowrank_fused_matches_reference(bda):
     assert_close(fused.cpu().numpy(), reference.numpy(), 1e-5, 1e-5)
 
 
-@pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (32, 1, 1), (1, 64, 4), (2, 100, 1), (3, 43, 4)])
+@pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (8, 1, 1), (17, 1, 4), (32, 1, 1), (1, 64, 4), (2, 100, 1),
+                                      (3, 43, 4)])
 def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
     """One k-sequential FMA chain per output on both sides: values, and therefore the active
     sets, are identical bit for bit whatever the launch tiling."""
@@ -69,6 +70,14 @@ def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
                                      bda.BlockPattern1d.dense(64))
     assert np.array_equal(got.cpu().numpy(), ref)
     assert 0.4 < (ref > 0).mean() < 0.6
+    ctx = bda.ffi.default_context(0)
+    try:  # the LDS-staged kernels give the same bits as the scalar-input ones that 8 to 63 rows take by default
+        ctx.set_option("relu_lowrank.scalar", 0)
+        lds = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
+                                         bda.BlockPattern1d.dense(64))
+    finally:
+        ctx.set_option("relu_lowrank.scalar", 1)
+    assert np.array_equal(lds.cpu().numpy(), ref)
     gated = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
                                        bda.BlockPattern1d.dense(64), gate=torch.from_numpy(gate).to(DEV))
     assert np.array_equal(gated.cpu().numpy(), gate * ref)
