@@ -22,6 +22,7 @@ struct bdh_ctx {
   int opt_lowrank_tile = 1;  // 0: relu_lowrank never takes the 64-row tile kernel
   int opt_decoder_mfma = 1;  // 0: the encoder E never takes the f32 matrix-core form
   int opt_lowrank_scalar = 1;  // 0: relu_lowrank with 8 to 63 rows stages its inputs in LDS instead of scalar loads
+  int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
   char err[512] = {0};
 };

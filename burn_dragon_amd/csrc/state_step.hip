@@ -668,6 +668,121 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
   }
 }
 
+// ------------------------------------------------------------------------------------
+// dense path, D in {256, 512}: PoPE (2N rows) and ALiBi with the eager decay touch every state row on
+// every token, so the step is a streaming read-modify-write of the whole slice.  Same work split and
+// the same order of operations per element as k_step_generic (a workgroup owns 64 rows, wave w takes
+// rows w, w+4, ...), but a lane owns four adjacent columns (one 16-byte access per row) and U rows are
+// in flight per wave.
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ float4 dense_load4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 dense_load4(const unsigned short *p) {
+  const uint2 v = *reinterpret_cast<const uint2 *>(p);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                     __uint_as_float(v.y & 0xffff0000u));
+}
+__device__ __forceinline__ void dense_store4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ void dense_store4(unsigned short *p, float4 v) {
+  uint2 o;
+  o.x = (unsigned int)f32_to_bf16(v.x) | ((unsigned int)f32_to_bf16(v.y) << 16);
+  o.y = (unsigned int)f32_to_bf16(v.z) | ((unsigned int)f32_to_bf16(v.w) << 16);
+  *reinterpret_cast<uint2 *>(p) = o;
+}
+
+template <typename RhoT, int D, int U>
+__global__ __launch_bounds__(256) void k_step_dense(StepPtrs a, RhoT *__restrict__ rho, int Nq, int rotary,
+                                                    HeadScalars decay) {
+  constexpr int VPL = D / 256;  // groups of four columns per lane
+  __shared__ float4 s_red[4][D / 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slice = blockIdx.x / a.S;
+  const int seg = blockIdx.x - slice * a.S;
+  const int b = slice / a.h, hh = slice - b * a.h;
+  const float pos = a.pos_dev ? (float)((long)a.pos_dev[b] + a.pos_add) : a.pos_scalar;
+  const float *xs = a.x + (long)slice * a.x_slice_stride;
+  const bool has_decay = rotary == BDH_ALIBI;
+  const float dec = has_decay ? decay.v[hh] : 1.0f;
+
+  float4 acc[VPL], vv[VPL];
+  {
+    const float4 *vrow = reinterpret_cast<const float4 *>(a.v + (long)b * a.v_batch_stride);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      vv[j] = vrow[j * 64 + lane];
+    }
+  }
+  RhoT *base = rho + ((long)slice * Nq + (long)seg * kGenRows) * D;
+  for (int r0 = wave; r0 < kGenRows; r0 += 4 * U) {
+    float4 rv[U][VPL];
+    float qn[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int r = r0 + 4 * u;
+      ok[u] = r < kGenRows && seg * kGenRows + r < Nq;
+      if (ok[u]) {
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) rv[u][j] = dense_load4(base + (long)r * D + (j * 64 + lane) * 4);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      qn[u] = 0.0f;
+      if (ok[u]) {
+        const int n = seg * kGenRows + r0 + 4 * u;
+        if (rotary == BDH_ALIBI) {
+          qn[u] = xs[n];  // ALiBi does not rotate (src/model/attention.rs:333-335)
+        } else {          // PoPE (src/model/attention.rs:323-330): rows N..2N-1 are the imaginary parts
+          const int m = n < a.N ? n : n - a.N;
+          const float mag = softplus1(xs[m]);
+          const float ph = rope_phase(pos, a.freqs[m]);
+          qn[u] = n < a.N ? mag * cosf(ph) : mag * sinf(ph);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) {
+        const float q = qn[u];
+        RhoT *row = base + (long)(r0 + 4 * u) * D;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+          float4 e = rv[u][j];
+          // readout with the old state (src/model/bdh.rs:293-295), update with the product rounded
+          // before the add (:298), ALiBi decay after the update (:299-301)
+          acc[j].x = __builtin_fmaf(e.x, q, acc[j].x);
+          acc[j].y = __builtin_fmaf(e.y, q, acc[j].y);
+          acc[j].z = __builtin_fmaf(e.z, q, acc[j].z);
+          acc[j].w = __builtin_fmaf(e.w, q, acc[j].w);
+          float t;
+          t = q * vv[j].x; e.x = e.x + t;
+          t = q * vv[j].y; e.y = e.y + t;
+          t = q * vv[j].z; e.z = e.z + t;
+          t = q * vv[j].w; e.w = e.w + t;
+          if (has_decay) {
+            e.x = e.x * dec; e.y = e.y * dec; e.z = e.z * dec; e.w = e.w * dec;
+          }
+          dense_store4(row + (j * 64 + lane) * 4, e);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) s_red[wave][j * 64 + lane] = acc[j];
+  __syncthreads();
+  float *pout = a.partial + (long)blockIdx.x * D;
+  for (int c4 = tid; c4 < D / 4; c4 += 256) {
+    float4 s = s_red[0][c4];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const float4 t = s_red[w][c4];
+      s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    reinterpret_cast<float4 *>(pout)[c4] = s;
+  }
+}
+
 // Brings every row of a lazily decayed ALiBi state up to date: row *= decay^(clock - stamp),
 // stamp = clock.  Afterwards rho is the state the reference would hold.
 template <typename RhoT>
@@ -838,6 +953,9 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   // lazily decayed ALiBi state, f32, d in {256,512}: row-compaction kernel, 512 neurons per workgroup
   const bool fast_lazy = p.rotary == BDH_ALIBI && p.stamps && p.rho_dtype == BDH_F32 && (d == 256 || d == 512) &&
                          (N % 2 == 0);  // the kernel reads x two neurons at a time
+  // PoPE, and ALiBi with the eager decay, at d in {256,512}: the dense streaming kernel (the generic kernel's split)
+  const bool fast_dense = !fast && !fast_lazy && (d == 256 || d == 512) && ctx->opt_step_dense_kernel != 0 &&
+                          (p.rotary == BDH_POPE || (p.rotary == BDH_ALIBI && !p.stamps));
   const int S = fast ? ((N / 2) + ppb - 1) / ppb : fast_lazy ? (N + 511) / 512 : (Nq + kGenRows - 1) / kGenRows;
   if (N == 0 || d == 0) {
     // nothing to read or update: the readout is an empty sum
@@ -950,6 +1068,25 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
       BDH_LAUNCH_CHECK(ctx, "k_step_alibi_lazy_f32");
       launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T, 1);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
+    } else if (fast_dense) {
+      const dim3 grid(slices * S);
+      if (p.rho_dtype == BDH_F32) {
+        float *rho = static_cast<float *>(p.rho);
+        if (d == 256) hipLaunchKernelGGL((k_step_dense<float, 256, 4>), grid, dim3(256), 0, ctx->stream, a, rho, Nq, p.rotary, decay);
+        else hipLaunchKernelGGL((k_step_dense<float, 512, 4>), grid, dim3(256), 0, ctx->stream, a, rho, Nq, p.rotary, decay);
+      } else {
+        unsigned short *rho = static_cast<unsigned short *>(p.rho);
+        if (d == 256) hipLaunchKernelGGL((k_step_dense<unsigned short, 256, 4>), grid, dim3(256), 0, ctx->stream, a, rho, Nq, p.rotary, decay);
+        else hipLaunchKernelGGL((k_step_dense<unsigned short, 512, 4>), grid, dim3(256), 0, ctx->stream, a, rho, Nq, p.rotary, decay);
+      }
+      BDH_LAUNCH_CHECK(ctx, "k_step_dense");
+      launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T);
+      BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
+      if (a.bitmask || rows_t) {
+        hipLaunchKernelGGL(k_bitmask_rows, dim3(slices), dim3(256), 0, ctx->stream, a, p.rotary, Nq, rows_t,
+                           (long)T, 0);
+        BDH_LAUNCH_CHECK(ctx, "k_bitmask_rows");
+      }
     } else {
       if (p.rho_dtype == BDH_F32)
         hipLaunchKernelGGL(k_step_generic<float>, dim3(slices * S), dim3(256), 0, ctx->stream, a,

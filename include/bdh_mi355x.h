@@ -71,6 +71,8 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *   "state_step.dense_chunks": -1 (default) a call of 128+ tokens without
  *                       bitmask / row-count outputs runs as dense products on the f32 matrix cores,
  *                       0 = always token by token, 1 = dense products for any T.
+ *   "state_step.dense_kernel": 1 (default) PoPE and eagerly decayed ALiBi steps at d in {256,512} take
+ *                       the dense streaming kernel, 0 = the generic kernel (same values).
  *   "relu_lowrank.scalar": 1 (default) calls with 8 to 63 rows read their inputs through the scalar
  *                       cache, 0 = stage them in LDS (same values).
  *   "relu_lowrank.tile": 1 (default) calls with 64+ rows take the 64-row tile kernel (same values),

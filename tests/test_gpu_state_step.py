@@ -525,3 +525,41 @@ def test_dense_chunk_form_with_a_bf16_state(gpu, corc, rotary):
     # exactly the f32 result rounded to bf16, up to f32 reassociation before the rounding
     want = torch.from_numpy(rho_ref).to(torch.bfloat16).float().numpy()
     assert (got != want).mean() < 0.02
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rotary", [orc.POPE, orc.ALIBI])
+@pytest.mark.parametrize("N,d", [(130, 256), (96, 512)])
+def test_dense_streaming_kernel_equals_generic_kernel_and_oracle(gpu, corc, rotary, N, d, dtype):
+    """PoPE and eager ALiBi at d in {256,512} take k_step_dense: the same operations per element in the same
+    order as the generic kernel (bit-identical state and readout), and the oracle's values."""
+    ffi, recurrent_attention = gpu
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    ctx = ffi.default_context(0)
+    B, h, T = 2, 3, 3
+    x, v, _ = make_inputs(55 + N + d, B, h, T, N, d, 0.3)
+    Nq = 2 * N if rotary == orc.POPE else N
+    rho0 = (0.05 * np.random.default_rng(6).standard_normal((B, h, Nq, d))).astype(np.float32)
+    rho0 = torch.from_numpy(rho0).to(dtype).float().numpy()  # representable in the storage type
+    freqs = corc.build_freqs(N, rotary=rotary)
+    slopes = np.array([0.1, 0.4, 0.9], np.float32) if rotary == orc.ALIBI else None
+    dev = "cuda:0"
+    res = []
+    for mode in (1, 0):
+        ctx.set_option("state_step.dense_kernel", mode)
+        try:
+            rt = torch.from_numpy(rho0).to(dev).to(dtype).contiguous()
+            out, rows = recurrent_attention(torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev), rt,
+                                            torch.from_numpy(freqs).to(dev), 77, RotaryEmbedding(rotary), slopes,
+                                            want_rows=True)
+            torch.cuda.synchronize()
+        finally:
+            ctx.set_option("state_step.dense_kernel", 1)
+        res.append((out.cpu().numpy(), rt.float().cpu().numpy(), rows.cpu().numpy()))
+    assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1])
+    assert (res[0][2] == Nq).all() and (res[1][2] == Nq).all()  # every row is touched on every token
+    q = corc.rotate(x, freqs, rotary, 77)
+    out_ref, rho_ref = corc.recurrent_attention(q, v, rho0.copy(), None if slopes is None else corc.alibi_decay(slopes))
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert rel_err(res[0][0], out_ref) < tol and rel_err(res[0][1], rho_ref) < tol
