@@ -238,6 +238,7 @@ int bdh_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, int64_t cloc
   if (clock < 0 || clock > 0x7fffffffLL) return bdh_fail(ctx, BDH_E_INVAL, "clock outside the 31-bit stamp range");
   if (B == 0 || h == 0 || N == 0) return BDH_OK;
   if (!rho || !stamps) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  if (!bdh_aligned(rho, 16)) return bdh_fail(ctx, BDH_E_ALIGN, "rho needs 16-byte alignment");
   float slopes[64];
   if (alibi_slopes_host)
     memcpy(slopes, alibi_slopes_host, sizeof(float) * h);

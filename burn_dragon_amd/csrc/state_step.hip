@@ -800,7 +800,15 @@ __global__ __launch_bounds__(256) void k_alibi_materialize(RhoT *__restrict__ rh
   if (k > 0) {
     const float scale = expf((float)k * log_decay.v[hh]);
     RhoT *p = rho + row * d;
-    for (int c = lane; c < d; c += 64) rho_store(p + c, rho_load<RhoT>(p + c) * scale);
+    if ((d & 3) == 0) {  // rows start on 16-byte (f32) / 8-byte (bf16) boundaries: four elements per access
+      for (int c = lane * 4; c < d; c += 256) {
+        float4 e = dense_load4(p + c);
+        e.x = e.x * scale; e.y = e.y * scale; e.z = e.z * scale; e.w = e.w * scale;
+        dense_store4(p + c, e);
+      }
+    } else {
+      for (int c = lane; c < d; c += 64) rho_store(p + c, rho_load<RhoT>(p + c) * scale);
+    }
   }
   if (lane == 0) stamps[row] = (int32_t)min(clock, 0x7fffffffL);
 }
