@@ -648,7 +648,9 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   const int M = B * T;
   const long K = (long)h * N;
   if (d > 1024 || (d & 3)) return bdh_fail(ctx, BDH_E_SHAPE, "decoder needs d %% 4 == 0 and d <= 1024, got %d", d);
-  if (T >= 128 && ctx->opt_decoder_mfma != 0) {
+  // (the matrix-core form needs enough (sequence, head, tile) products to cover the chip)
+  const long mfma_tiles = (long)B * h * ((T + 127) / 128) * ((d + 127) / 128);
+  if (T >= 128 && ctx->opt_decoder_mfma != 0 && mfma_tiles >= (ctx->n_cu > 0 ? ctx->n_cu : 256) / 2) {
     // many tokens per sequence: one product per (sequence, head) on the f32 matrix cores, h partials per row
     int rc = bdh_ws_reserve(ctx, sizeof(float) * (size_t)h * M * d);
     if (rc != BDH_OK) return rc;

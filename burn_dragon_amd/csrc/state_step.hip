@@ -986,8 +986,13 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   // (not when even a 128-token chunk of rotated activations would pass 16 GiB of workspace)
   const bool chunk_fits = sizeof(float) * (size_t)slices * Nq * 128 <= (size_t(16) << 30) &&
                           (p.rho_dtype == BDH_F32 || sizeof(float) * (size_t)slices * Nq * d <= (size_t(64) << 30));
-  if (!p.bitmask && !p.rows_touched && chunk_fits &&
-      (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : T >= 128))
+  // By default from 128 tokens on; where the token loop is cheap (the f32 RoPE kernel walks many tokens per
+  // launch) only once the products have enough tiles to cover the chip (measured at N=8192, d=256, T=512:
+  // B*h = 4 or 8 slices lose to the loop at 5 % density, 16 slices win at any density).
+  const bool loop_is_cheap = fast && p.rho_dtype == BDH_F32;
+  const long state_tiles = (long)slices * ((std::min(T, 512) + 127) / 128) * ((d + 127) / 128);
+  const bool dense_auto = T >= 128 && (!loop_is_cheap || state_tiles >= n_cu / 2);
+  if (!p.bitmask && !p.rows_touched && chunk_fits && (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : dense_auto))
     return bdh_launch_state_chunks_f32(ctx, p, out_ln);
   // tokens per launch: only the f32 RoPE kernel walks several, as many as 64 MiB of partials allow
   const size_t partial_one = bdh_align_up(sizeof(float) * (size_t)slices * S * d, 256);

@@ -380,13 +380,14 @@ def test_dense_chunk_form_matches_sequential_oracle(gpu, corc, dense_chunks, rot
 
 def test_dense_chunk_form_equals_step_kernels_and_handles_device_positions(gpu, corc):
     """The same call through the sparse step kernels and through the dense form; per-sequence device
-    positions; T = 128 takes the dense form by default."""
+    positions; T = 128 takes the dense form by default once the products have enough tiles to cover the
+    chip (B*h = 96 slices here; with a handful of slices the multi-token f32 RoPE kernel is kept)."""
     ffi, recurrent_attention = gpu
     ctx = ffi.default_context(0)
-    B, h, T, N, d = 3, 2, 128, 128, 256
+    B, h, T, N, d = 24, 4, 128, 128, 256
     x, v, rho = make_inputs(99, B, h, T, N, d, 0.1, rho_scale=0.05)
     freqs = corc.build_freqs(N)
-    positions = [0, 77, 4000]
+    positions = [int(p) for p in np.random.default_rng(1).integers(0, 4000, B)]
     try:
         ctx.set_option("state_step.dense_chunks", 0)
         out_s, rho_s = _run_plain(recurrent_attention, x, v, rho, freqs, 0, orc.ROPE, positions)
@@ -395,7 +396,15 @@ def test_dense_chunk_form_equals_step_kernels_and_handles_device_positions(gpu, 
     out_d, rho_d = _run_plain(recurrent_attention, x, v, rho, freqs, 0, orc.ROPE, positions)
     assert rel_err(out_d, out_s) < 2e-5 and rel_err(rho_d, rho_s) < 2e-5
     assert not np.array_equal(out_d, out_s)  # different summation order: the dense form did run
-    for b, pos in enumerate(positions):
+    # a handful of slices at the same shape: the default keeps the token loop (identical bits)
+    try:
+        ctx.set_option("state_step.dense_chunks", 0)
+        out_few_loop, _ = _run_plain(recurrent_attention, x[:1], v[:1], rho[:1], freqs, 5, orc.ROPE)
+    finally:
+        ctx.set_option("state_step.dense_chunks", -1)
+    out_few, _ = _run_plain(recurrent_attention, x[:1], v[:1], rho[:1], freqs, 5, orc.ROPE)
+    assert np.array_equal(out_few, out_few_loop)
+    for b, pos in list(enumerate(positions))[:3]:
         o_ref, r_ref = corc.recurrent_attention(corc.rotate(x[b : b + 1], freqs, orc.ROPE, pos), v[b : b + 1],
                                                 rho[b : b + 1].copy())
         assert rel_err(out_d[b : b + 1], o_ref) < 2e-5 and rel_err(rho_d[b : b + 1], r_ref) < 2e-5
