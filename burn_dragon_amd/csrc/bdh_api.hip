@@ -113,7 +113,7 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     return BDH_OK;
   }
   if (strcmp(name, "relu_lowrank.tile") == 0) {
-    if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "relu_lowrank.tile takes 0 or 1");
+    if (value < 0 || value > 2) return bdh_fail(ctx, BDH_E_INVAL, "relu_lowrank.tile takes 0, 1 or 2");
     ctx->opt_lowrank_tile = value;
     return BDH_OK;
   }

@@ -588,7 +588,9 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
   // many rows: the 64 x 256 tile (same values, an eighth of the weight traffic)
   const bool aligned16 = bdh_aligned(p.in, 16) && bdh_aligned(p.weight, 16) && bdh_aligned(p.out, 16) &&
                          bdh_aligned(p.bias, 16) && bdh_aligned(p.gate, 16);
-  if (M >= 64 && ctx->opt_lowrank_tile != 0 && (p.N & 3) == 0 && (p.d & 3) == 0 && p.d > 0 && aligned16) {
+  const long tile_wgs = (long)((p.N / 4 + 63) / 64) * p.h * ((M + 63) / 64);  // enough of them to cover the chip
+  if (M >= 64 && ctx->opt_lowrank_tile != 0 && (p.N & 3) == 0 && (p.d & 3) == 0 && p.d > 0 && aligned16 &&
+      (ctx->opt_lowrank_tile == 2 || tile_wgs >= (ctx->n_cu > 0 ? ctx->n_cu : 256))) {
     const long row_tiles = (M + 63) / 64;
     if (row_tiles > 65535 || p.h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (row tiles %ld)", row_tiles);
     hipLaunchKernelGGL(k_relu_lowrank_tile, dim3((p.N / 4 + 63) / 64, p.h, (unsigned)row_tiles), dim3(256), 0, ctx->stream,

@@ -76,8 +76,8 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       the dense streaming kernel, 0 = the generic kernel (same values).
  *   "relu_lowrank.scalar": 1 (default) calls with 8 to 63 rows read their inputs through the scalar
  *                       cache, 0 = stage them in LDS (same values).
- *   "relu_lowrank.tile": 1 (default) calls with 64+ rows take the 64-row tile kernel (same values),
- *                       0 = always the 8-row kernel.
+ *   "relu_lowrank.tile": 1 (default) calls with 64+ rows take the 64-row tile kernel (same values) when
+ *                       its grid covers the chip, 2 = whenever the shape allows, 0 = never.
  *   "decoder.mfma":     1 (default) the encoder E of a call with 128+ tokens per sequence runs on
  *                       the f32 matrix cores, 0 = always the VALU kernel.
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,

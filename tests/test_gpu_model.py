@@ -96,16 +96,23 @@ def test_relu_lowrank_many_rows_with_bias_threshold_and_mask(bda, corc):
     layout = bda.BlockPattern1d.from_blocks(8, [0, 3, 4, 17, 24])
     ref = corc.relu_lowrank(inp, weight, bias.reshape(h, N), 0.05, 8, [0, 3, 4, 17, 24])
     args = (torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), torch.from_numpy(bias).to(DEV), 0.05, layout)
-    got = relu_lowrank.fused_forward(*args).cpu().numpy()
-    assert np.array_equal(got, ref)
-    assert 0.05 < (ref > 0).mean() < 0.2
     ctx = bda.ffi.default_context(0)
     try:
+        ctx.set_option("relu_lowrank.tile", 2)  # the default keeps the tile kernel for grids that cover the chip
+        got = relu_lowrank.fused_forward(*args).cpu().numpy()
         ctx.set_option("relu_lowrank.tile", 0)
         small = relu_lowrank.fused_forward(*args).cpu().numpy()
     finally:
         ctx.set_option("relu_lowrank.tile", 1)
+    assert np.array_equal(got, ref)
+    assert 0.05 < (ref > 0).mean() < 0.2
     assert np.array_equal(got, small)
+    # a shape whose tile grid covers the chip takes the tile kernel by default
+    big_w = (0.05 * rng.standard_normal((4, 64, 8192))).astype(np.float32)
+    big_in = rng.standard_normal((2, 1, 128, 64)).astype(np.float32)
+    big = relu_lowrank.fused_forward(torch.from_numpy(big_in).to(DEV), torch.from_numpy(big_w).to(DEV), None, 0.0,
+                                     bda.BlockPattern1d.dense(64)).cpu().numpy()
+    assert np.array_equal(big, corc.relu_lowrank(big_in, big_w))
 
 
 def test_layer_norm_matches_oracle_and_library(bda, corc):
