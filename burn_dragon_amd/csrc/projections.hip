@@ -399,35 +399,40 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
 }
 
 // cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))   (src/model/bdh.rs:438-441)
-// 1024 threads: four groups each add a quarter of the k-block partials (index order within a
-// group, groups combined in order); after the one barrier the first wavefront applies the two
-// LayerNorms with wave shuffles only.
+// 1024 threads = 16 groups of 64 lanes; a lane owns four adjacent columns (one 16-byte load per partial
+// row), a group adds a sixteenth of the k-block partials in index order with up to 16 loads in flight,
+// the groups are combined in order; after the one barrier the first wavefront applies the two LayerNorms
+// with wave shuffles only.
 __global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restrict__ partial, int KBN, int M,
                                                            int d, float *__restrict__ cur) {
-  __shared__ float s_grp[4][1024];
-  const int m = blockIdx.x, tid = threadIdx.x & 255, grp = threadIdx.x >> 8;
-  const int per = (KBN + 3) >> 2;
-  const int kb0 = grp * per, kb1 = min(KBN, kb0 + per);
+  __shared__ float s_grp[16][1024];
+  const int m = blockIdx.x, lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int per = (KBN + 15) >> 4;
+  const int kb0 = min(KBN, grp * per), kb1 = min(KBN, kb0 + per);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int c = j * 256 + tid;
-    float v = 0.0f;
+    const int c = (j * 64 + lane) * 4;  // d % 4 == 0
     if (c < d) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       int kb = kb0;
       for (; kb + 16 <= kb1; kb += 16) {
-        float t[16];
+        float4 t[16];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) t[u] = partial[((long)(kb + u) * M + m) * d + c];
+        for (int u = 0; u < 16; ++u) t[u] = *reinterpret_cast<const float4 *>(partial + ((long)(kb + u) * M + m) * d + c);
 #pragma unroll
-        for (int u = 0; u < 16; ++u) v += t[u];
+        for (int u = 0; u < 16; ++u) {
+          v.x += t[u].x; v.y += t[u].y; v.z += t[u].z; v.w += t[u].w;
+        }
       }
-      for (; kb < kb1; ++kb) v += partial[((long)kb * M + m) * d + c];
+      for (; kb < kb1; ++kb) {
+        const float4 t = *reinterpret_cast<const float4 *>(partial + ((long)kb * M + m) * d + c);
+        v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+      }
+      *reinterpret_cast<float4 *>(&s_grp[grp][c]) = v;
     }
-    s_grp[grp][c] = v;
   }
   __syncthreads();
   if (threadIdx.x >= 64) return;  // no barrier follows: the first wave finishes the row alone
-  const int lane = threadIdx.x;
   float vals[16];  // column c = j*64 + lane, d <= 1024
   float s = 0.0f;
 #pragma unroll
@@ -435,7 +440,9 @@ __global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restri
     const int c = j * 64 + lane;
     float v = 0.0f;
     if (c < d) {
-      v = ((s_grp[0][c] + s_grp[1][c]) + s_grp[2][c]) + s_grp[3][c];
+      v = s_grp[0][c];
+#pragma unroll
+      for (int g = 1; g < 16; ++g) v += s_grp[g][c];
       s += v;
     }
     vals[j] = v;
