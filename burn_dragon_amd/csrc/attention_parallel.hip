@@ -745,3 +745,25 @@ extern "C" int bdh_rotate(bdh_ctx *ctx, int B, int h, int T, int N, int rotary, 
   BDH_LAUNCH_CHECK(ctx, "k_rotate_chunk_f32");
   return BDH_OK;
 }
+
+// The encoder E of a decode step for a batch of sequences (T = 1, src/model/bdh.rs:383,436-438): mixed [B, h*N] is
+// contiguous per sequence, so the product is one [B x K] . [K x d] GEMM split over K: slice s takes k in
+// [s*KB, (s+1)*KB) and writes partial[s][B][d].  With 8 or more sequences nearly every row of E is needed by some
+// sequence, so the weights are streamed once through the matrix cores instead of skipping inactive rows.
+int bdh_launch_decoder_splitk_f32(bdh_ctx *ctx, int M, long K, int d, int KB, const float *xy, const float *decoder,
+                                  float *partial) {
+  const long KBN = (K + KB - 1) / KB;
+  const unsigned groups = (unsigned)((KBN + 7) / 8);
+  FsaArgs g{};
+  g.A = xy; g.Bm = decoder; g.C = partial;
+  g.a_batch = KB; g.b_batch = (long)KB * d; g.c_batch = (long)M * d;
+  g.lda = (int)K; g.ldb = d; g.ldc = d; g.M = M; g.N = d; g.K = KB; g.b_div = 1; g.n_slices = (int)KBN;
+  g.block_size = 1; g.h = 1; g.dense = 0; g.beta = 0;
+  g.mt = (M + 31) / 32; g.nt = (d + 63) / 64;
+  if (K % KB != 0) return bdh_fail(ctx, BDH_E_SHAPE, "split-K block %d does not divide K=%ld", KB, K);
+  if ((long)groups * 8 * g.mt * g.nt > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
+  hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128), 0,
+                     ctx->stream, g);
+  BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<decoder split-K>");
+  return BDH_OK;
+}

@@ -132,6 +132,11 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     ctx->opt_step_dense_kernel = value;
     return BDH_OK;
   }
+  if (strcmp(name, "decoder.splitk_rows") == 0) {
+    if (value < 1) return bdh_fail(ctx, BDH_E_INVAL, "decoder.splitk_rows takes a positive row count");
+    ctx->opt_decoder_splitk_rows = value;
+    return BDH_OK;
+  }
   if (strcmp(name, "fused_state_aligned.path") == 0) {
     if (value < -1 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "fused_state_aligned.path takes -1, 0 or 1");
     ctx->opt_fsa_path = value;

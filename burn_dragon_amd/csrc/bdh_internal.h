@@ -23,6 +23,7 @@ struct bdh_ctx {
   int opt_decoder_mfma = 1;  // 0: the encoder E never takes the f32 matrix-core form
   int opt_lowrank_scalar = 1;  // 0: relu_lowrank with 8 to 63 rows stages its inputs in LDS instead of scalar loads
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
+  int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on
   int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
   char err[512] = {0};
 };
@@ -114,6 +115,9 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
 // attention_parallel.hip: partial[hh][b*T+t][:] = xy[b,hh,t,:] . decoder[hh*N.., :] on the f32 matrix cores
 int bdh_launch_decoder_partials_f32(bdh_ctx *ctx, int B, int T, int h, int N, int d, const float *xy,
                                     const float *decoder, float *partial);
+// attention_parallel.hip: decode-step encoder for a batch (T = 1): partial[s][m][:] = xy[m, s*KB..] . decoder[s*KB.., :]
+int bdh_launch_decoder_splitk_f32(bdh_ctx *ctx, int M, long K, int d, int KB, const float *xy, const float *decoder,
+                                  float *partial);
 int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cur,
                        const float *lm_head, float *logits, int64_t *next_tokens);
 // positions[b] = min(positions[b] + delta, INT32_MAX): the device-side form of state.position += T

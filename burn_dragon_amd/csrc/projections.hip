@@ -670,6 +670,19 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
     BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
     return BDH_OK;
   }
+  if (T == 1 && M >= ctx->opt_decoder_splitk_rows && (K % 1024) == 0) {
+    // a batch of decoding sequences: split-K product on the f32 matrix cores, KB = 1024
+    const int KB = 1024;
+    const int KBN = (int)(K / KB);
+    int rc = bdh_ws_reserve(ctx, sizeof(float) * (size_t)KBN * M * d);
+    if (rc != BDH_OK) return rc;
+    float *partial = static_cast<float *>(ctx->ws);
+    rc = bdh_launch_decoder_splitk_f32(ctx, M, K, d, KB, xy, decoder, partial);
+    if (rc != BDH_OK) return rc;
+    hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur);
+    BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
+    return BDH_OK;
+  }
   const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
   const int row_tiles = (M + RT - 1) / RT;
   // k-block size: enough workgroups to fill the chip, few enough partials

@@ -80,6 +80,9 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       its grid covers the chip, 2 = whenever the shape allows, 0 = never.
  *   "decoder.mfma":     1 (default) the encoder E of a call with 128+ tokens per sequence runs on
  *                       the f32 matrix cores, 0 = always the VALU kernel.
+ *   "decoder.splitk_rows": 24 (default) a decode step (T = 1) of this many or more sequences runs the
+ *                       encoder E as a split-K product on the f32 matrix cores (all of E is streamed
+ *                       once); fewer sequences take the VALU kernel that skips inactive rows of E.
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
  *                       1 = the two products on the f32 matrix cores (T >= 128 by default). */
 int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);

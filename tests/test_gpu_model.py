@@ -223,6 +223,34 @@ def test_forward_fast_long_sequence_on_the_matrix_cores(bda):
         assert rel_err(got, want) < 1e-3
 
 
+def test_batched_decode_step_takes_the_split_k_encoder(bda, corc):
+    """24+ sequences decoding together: the encoder E runs as a split-K product on the f32 matrix cores (the
+    weights are streamed once); logits against the oracle and against the VALU kernel."""
+    cfg = bda.BDHConfig(n_layer=2, n_embd=64, n_head=4, mlp_internal_dim_multiplier=64, vocab_size=64)  # N = 1024
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse("rope"))
+    shape, w, model = _model_pair(bda, cfg, seed=5)
+    rng = np.random.default_rng(1)
+    B = 26
+    steps = [rng.integers(0, 64, (B, 1)) for _ in range(3)]
+    ctx = bda.ffi.default_context(0)
+    outs = {}
+    for rows in (24, 1 << 30):
+        ctx.set_option("decoder.splitk_rows", rows)
+        try:
+            state = model.init_state()
+            outs[rows] = np.concatenate([model.forward_with_state(torch.from_numpy(t), state).cpu().numpy() for t in steps], 1)
+        finally:
+            ctx.set_option("decoder.splitk_rows", 24)
+    rho_ref = np.zeros((2, B, 4, 1024, 64), np.float32)
+    pos, refs = 0, []
+    for t in steps:
+        lg, pos, _, _ = corc.forward_with_state(shape, w, t, rho_ref, pos, sparse_state=True)
+        refs.append(lg)
+    ref = np.concatenate(refs, 1)
+    assert rel_err(outs[24], ref) < 1e-3 and rel_err(outs[1 << 30], ref) < 1e-3
+    assert rel_err(outs[24], outs[1 << 30]) < 1e-5 and not np.array_equal(outs[24], outs[1 << 30])
+
+
 def test_config1_architecture_prefill_and_greedy_decode(bda, corc):
     """BASELINE config 1 architecture (V=256, d=256, h=4, N=8192, RoPE) with L=2 and a short
     run so the oracle finishes in seconds: 16-byte prompt, 8 greedy tokens, batch 1."""
