@@ -62,6 +62,17 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank(const float *__restrict__
 #pragma unroll
       for (int r = 0; r < RT; ++r) acc[r] = __builtin_fmaf(s_in[r * d + k0 + u], wv[u], acc[r]);
   }
+  if (UK > 16) {  // what a large batch leaves over, 16 rows at a time
+    for (; k0 + 16 <= d; k0 += 16) {
+      float wv[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) wv[u] = wp[(long)(k0 + u) * N];
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+#pragma unroll
+        for (int r = 0; r < RT; ++r) acc[r] = __builtin_fmaf(s_in[r * d + k0 + u], wv[u], acc[r]);
+    }
+  }
   for (; k0 < d; ++k0) {
     const float wv = wp[(long)k0 * N];
 #pragma unroll
@@ -303,7 +314,7 @@ __global__ __launch_bounds__(256) void k_embed_ln(const int64_t *__restrict__ to
 // mixed[m = b*T+t, k = hh*N+n] = xy[b,hh,t,n].  Rows of E whose xy is zero for every row
 // of the tile are never loaded.
 // ------------------------------------------------------------------------------------
-template <int RT, int MAXV>
+template <int RT, int MAXV, int UF = 4>
 __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict__ xy,
                                                          const float *__restrict__ E,
                                                          float *__restrict__ partial, int T, int h, int N,
@@ -335,13 +346,13 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) acc[r][j] = make_float4(0.f, 0.f, 0.f, 0.f);
 
-  // each wave takes k = wave, wave+4, ...; four of its E rows are in flight at a time
-  for (int kk0 = wave; kk0 < KB; kk0 += 16) {
-    float xs[4][RT];
-    bool any[4];
-    float4 e[4][MAXV];
+  // each wave takes k = wave, wave+4, ...; UF of its E rows are in flight at a time
+  for (int kk0 = wave; kk0 < KB; kk0 += 4 * UF) {
+    float xs[UF][RT];
+    bool any[UF];
+    float4 e[UF][MAXV];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < UF; ++u) {
       const int kk = kk0 + 4 * u;
       const int k = kb * KB + kk;
       any[u] = false;
@@ -362,7 +373,7 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
       }
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < UF; ++u) {
       if (any[u]) {
 #pragma unroll
         for (int j = 0; j < MAXV; ++j) {
@@ -409,6 +420,13 @@ __global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restri
   const int m = blockIdx.x, lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
   const int per = (KBN + 15) >> 4;
   const int kb0 = min(KBN, grp * per), kb1 = min(KBN, kb0 + per);
+  // the residual row is fetched while the partials are summed: it was written by another
+  // workgroup of an earlier launch, so the load is a trip to memory
+  float res[16];
+  if (grp == 0) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) res[j] = (j * 64 + lane < d) ? cur[(long)m * d + j * 64 + lane] : 0.0f;
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int c = (j * 64 + lane) * 4;  // d % 4 == 0
@@ -466,7 +484,7 @@ __global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restri
     const int c = j * 64 + lane;
     if (c < d) {
       const float mlp = (vals[j] - mean) / den;
-      vals[j] = cur[(long)m * d + c] + mlp;
+      vals[j] = res[j] + mlp;
       s += vals[j];
     }
   }
@@ -568,7 +586,7 @@ __global__ void k_advance_positions(int32_t *pos, int B, int delta) {
 template <int RT>
 void launch_relu(hipStream_t st, dim3 grid, size_t lds, const ReluLowrankParams &p, const unsigned char *mask,
                  int M) {
-  constexpr int UK = RT == 1 ? 32 : 16;      // weight rows in flight per thread
+  constexpr int UK = RT == 1 ? 64 : 16;      // weight rows in flight per thread (the counter of outstanding loads ends at 63)
   constexpr int NTHR = RT == 1 ? 128 : 256;  // a single input row: smaller workgroups, one per CU at N*h = 32768
   grid.x = (p.N + NTHR - 1) / NTHR;
   hipLaunchKernelGGL((k_relu_lowrank<RT, UK, NTHR>), grid, dim3(NTHR), lds, st, p.in, p.h_in, p.T, p.d, p.weight,
@@ -702,9 +720,15 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
                      N, d, KB, M)
   const int mv = d <= 256 ? 1 : (d <= 512 ? 2 : 4);
   if (mv == 1) {
-    if (RT == 8) BDH_DEC(8, 1); else if (RT == 4) BDH_DEC(4, 1); else if (RT == 2) BDH_DEC(2, 1); else BDH_DEC(1, 1);
+    if (RT == 8) BDH_DEC(8, 1); else if (RT == 4) BDH_DEC(4, 1); else if (RT == 2) BDH_DEC(2, 1);
+    else  // one row: the kernel is a chain of round trips, so more E rows per trip
+      hipLaunchKernelGGL((k_decoder_partial<1, 1, 16>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d,
+                         KB, M);
   } else if (mv == 2) {
-    if (RT == 8) BDH_DEC(8, 2); else if (RT == 4) BDH_DEC(4, 2); else if (RT == 2) BDH_DEC(2, 2); else BDH_DEC(1, 2);
+    if (RT == 8) BDH_DEC(8, 2); else if (RT == 4) BDH_DEC(4, 2); else if (RT == 2) BDH_DEC(2, 2);
+    else
+      hipLaunchKernelGGL((k_decoder_partial<1, 2, 8>), grid, dim3(256), lds, ctx->stream, xy, decoder, partial, T, h, N, d,
+                         KB, M);
   } else {
     if (RT >= 4) BDH_DEC(4, 4); else if (RT == 2) BDH_DEC(2, 4); else BDH_DEC(1, 4);
   }

@@ -1052,7 +1052,7 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
       if (p.rho_dtype == BDH_F32) {
         float *rho = static_cast<float *>(p.rho);
         if (d == 256 && !split) launch_fast<256, 4, 2, 1>(ctx->stream, blocks, a, rho);
-        if (d == 256 && split) launch_fast<256, 8, 4, 8>(ctx->stream, blocks, a, rho);
+        if (d == 256 && split) launch_fast<256, 8, 8, 8>(ctx->stream, blocks, a, rho);
         if (d == 512 && !split) launch_fast<512, 4, 2, 1>(ctx->stream, blocks, a, rho);
         if (d == 512 && split) launch_fast<512, 8, 2, 8>(ctx->stream, blocks, a, rho);
       } else {
