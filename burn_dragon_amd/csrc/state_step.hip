@@ -553,6 +553,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsig
 // ------------------------------------------------------------------------------------
 constexpr int kGenRows = 64;
 constexpr int kGenMaxCols = 16;  // d <= 64 * 16
+constexpr int kGenFlight = 4;    // state rows in flight per wave
 
 template <typename RhoT>
 __device__ __forceinline__ float rho_load(const RhoT *p);
@@ -563,26 +564,8 @@ __device__ __forceinline__ float rho_load<unsigned short>(const unsigned short *
 __device__ __forceinline__ void rho_store(float *p, float v) { *p = v; }
 __device__ __forceinline__ void rho_store(unsigned short *p, float v) { *p = f32_to_bf16(v); }
 
-// One state row (all d columns) of the generic path: readout with the old row, rank-1 update,
-// optional decay.  `scale` brings a lazily decayed row up to date first (1 otherwise).
-template <typename RhoT>
-__device__ __forceinline__ void generic_row(RhoT *row, int d, int ncol, int lane, float qn, const float *vrow,
-                                            float scale, bool lazy, bool has_decay, float dec, float *acc) {
-#pragma unroll
-  for (int j = 0; j < kGenMaxCols; ++j) {
-    const int c = j * 64 + lane;
-    if (j < ncol && c < d) {
-      float rv = rho_load<RhoT>(row + c);
-      if (lazy) rv = rv * scale;
-      acc[j] = __builtin_fmaf(rv, qn, acc[j]);
-      const float outer = qn * vrow[c];
-      rv = rv + outer;
-      if (has_decay) rv = rv * dec;  // src/model/bdh.rs:299-301
-      rho_store(row + c, rv);
-    }
-  }
-}
-
+// Per state row (all d columns) of the generic path: readout with the old row, rank-1 update, optional
+// decay; a lazily decayed row is brought up to date first.
 // stamps != nullptr (ALiBi only): the state is kept lazily decayed.  Row n of a slice holds the
 // value it had when the sequence had absorbed stamps[n] tokens; its current value is that times
 // decay^(clock - stamps[n]).  Only rows with a non-zero activation are read, brought up to date,
@@ -607,54 +590,93 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
 #pragma unroll
   for (int j = 0; j < kGenMaxCols; ++j) acc[j] = 0.0f;
 
-  if (rotary == BDH_ALIBI) {
-    // q = x (src/model/attention.rs:332-349: ALiBi does not rotate).  Lane l < 16 fetches the
-    // activation of row wave + 4l of this segment; the ballot lists the rows to visit.
-    const bool lazy = stamps != nullptr;
-    const long clock = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
-    const int n_l = seg * kGenRows + wave + 4 * lane;
-    const bool in_range = lane < kGenRows / 4 && n_l < Nq;
-    const float xl = in_range ? xs[n_l] : 0.0f;
-    unsigned long long m = __ballot(lazy ? (xl != 0.0f) : in_range);
-    int32_t *st = lazy ? stamps + (long)slice * Nq : nullptr;
-    while (m) {
-      const int l = __builtin_ctzll(m);
-      m &= m - 1;
-      const float qn = __shfl(xl, l, 64);
-      const int n = seg * kGenRows + wave + 4 * l;
-      float scale = 1.0f;
-      if (lazy) {
-        const long k = clock - (long)st[n];
-        if (k > 0) scale = expf((float)k * log_decay.v[hh]);
+  // Lane l < 16 prepares row wave + 4l of this segment: its query value, whether the row is visited and,
+  // for a lazily decayed state, the factor that brings it up to date.  The ballot lists the rows to visit;
+  // they are then walked in index order, kGenFlight rows in flight at a time.
+  const bool lazy = rotary == BDH_ALIBI && stamps != nullptr;
+  const long clock = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
+  int32_t *st = lazy ? stamps + (long)slice * Nq : nullptr;
+  const int n_l = seg * kGenRows + wave + 4 * lane;
+  const bool in_range = lane < kGenRows / 4 && n_l < Nq;
+  float q_l = 0.0f, scale_l = 1.0f;
+  bool touch_l = false;
+  if (in_range) {
+    if (rotary == BDH_ALIBI) {
+      // q = x (src/model/attention.rs:332-349: ALiBi does not rotate)
+      q_l = xs[n_l];
+      touch_l = lazy ? (q_l != 0.0f) : true;
+      if (lazy && touch_l) {
+        const long k = clock - (long)st[n_l];
+        if (k > 0) scale_l = expf((float)k * log_decay.v[hh]);
       }
-      generic_row<RhoT>(rho + ((long)slice * Nq + n) * d, d, ncol, lane, qn, vrow, scale, lazy, true, dec, acc);
-      if (lazy && lane == 0) st[n] = (int32_t)min(clock + 1, 0x7fffffffL);
-    }
-  } else {
-    for (int r = wave; r < kGenRows; r += 4) {
-      const int n = seg * kGenRows + r;
-      if (n >= Nq) break;
-      float qn;
-      bool touch;
-      if (rotary == BDH_ROPE) {
-        const float xn = xs[n], xo = xs[n ^ 1];
-        touch = (xn != 0.0f) || (xo != 0.0f);
-        float s, c;
-        sincosf(rope_phase(pos, a.freqs[n]), &s, &c);
-        const float rot = (n & 1) ? xo : -xo;
-        const float t0 = xn * c, t1 = rot * s;
-        qn = t0 + t1;
-      } else {
-        const int m = n < a.N ? n : n - a.N;
-        const float mag = softplus1(xs[m]);
-        const float ph = rope_phase(pos, a.freqs[m]);
-        qn = n < a.N ? mag * cosf(ph) : mag * sinf(ph);
-        touch = true;
-      }
-      if (!touch) continue;
-      generic_row<RhoT>(rho + ((long)slice * Nq + n) * d, d, ncol, lane, qn, vrow, 1.0f, false, false, 1.0f, acc);
+    } else if (rotary == BDH_ROPE) {
+      const float xn = xs[n_l], xo = xs[n_l ^ 1];
+      touch_l = (xn != 0.0f) || (xo != 0.0f);
+      float sn, cs;
+      sincosf(rope_phase(pos, a.freqs[n_l]), &sn, &cs);
+      const float rot = (n_l & 1) ? xo : -xo;
+      const float t0 = xn * cs, t1 = rot * sn;
+      q_l = t0 + t1;
+    } else {
+      const int m = n_l < a.N ? n_l : n_l - a.N;
+      const float mag = softplus1(xs[m]);
+      const float ph = rope_phase(pos, a.freqs[m]);
+      q_l = n_l < a.N ? mag * cosf(ph) : mag * sinf(ph);
+      touch_l = true;
     }
   }
+  const bool has_dec = rotary == BDH_ALIBI;  // src/model/bdh.rs:299-301
+  float vv[kGenMaxCols];
+#pragma unroll
+  for (int j = 0; j < kGenMaxCols; ++j) {
+    const int c = j * 64 + lane;
+    vv[j] = (j < ncol && c < d) ? vrow[c] : 0.0f;
+  }
+  unsigned long long m = __ballot(touch_l);
+  while (m) {
+    int ls[kGenFlight];
+    bool ok[kGenFlight];
+    float rv[kGenFlight][kGenMaxCols];
+#pragma unroll
+    for (int u = 0; u < kGenFlight; ++u) {
+      ok[u] = m != 0ull;
+      ls[u] = ok[u] ? __builtin_ctzll(m) : 0;
+      if (ok[u]) m &= m - 1;
+    }
+#pragma unroll
+    for (int u = 0; u < kGenFlight; ++u) {
+      if (ok[u]) {
+        const RhoT *row = rho + ((long)slice * Nq + seg * kGenRows + wave + 4 * ls[u]) * d;
+#pragma unroll
+        for (int j = 0; j < kGenMaxCols; ++j) {
+          const int c = j * 64 + lane;
+          if (j < ncol && c < d) rv[u][j] = rho_load<RhoT>(row + c);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kGenFlight; ++u) {
+      const float qn = __shfl(q_l, ls[u], 64);
+      const float scale = __shfl(scale_l, ls[u], 64);
+      if (ok[u]) {
+        RhoT *row = rho + ((long)slice * Nq + seg * kGenRows + wave + 4 * ls[u]) * d;
+#pragma unroll
+        for (int j = 0; j < kGenMaxCols; ++j) {
+          const int c = j * 64 + lane;
+          if (j < ncol && c < d) {
+            float r = rv[u][j];
+            if (lazy) r = r * scale;
+            acc[j] = __builtin_fmaf(r, qn, acc[j]);
+            const float outer = qn * vv[j];
+            r = r + outer;
+            if (has_dec) r = r * dec;
+            rho_store(row + c, r);
+          }
+        }
+      }
+    }
+  }
+  if (lazy && touch_l) st[n_l] = (int32_t)min(clock + 1, 0x7fffffffL);
 #pragma unroll
   for (int j = 0; j < kGenMaxCols; ++j) s_red[wave][j * 64 + lane] = acc[j];
   __syncthreads();
