@@ -553,7 +553,6 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsig
 // ------------------------------------------------------------------------------------
 constexpr int kGenRows = 64;
 constexpr int kGenMaxCols = 16;  // d <= 64 * 16
-constexpr int kGenFlight = 4;    // state rows in flight per wave
 
 template <typename RhoT>
 __device__ __forceinline__ float rho_load(const RhoT *p);
@@ -571,11 +570,11 @@ __device__ __forceinline__ void rho_store(unsigned short *p, float v) { *p = f32
 // decay^(clock - stamps[n]).  Only rows with a non-zero activation are read, brought up to date,
 // updated, decayed once (src/model/bdh.rs:299-301) and stamped clock+1; all other rows are left
 // alone, so the step stays as sparse as the activations.
-template <typename RhoT>
+template <typename RhoT, int MAXC, int FL>  // d <= 64 * MAXC; FL state rows in flight per wave
 __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restrict__ rho, int d, int Nq,
                                                       int rotary, int has_decay, HeadScalars decay,
                                                       HeadScalars log_decay, int32_t *__restrict__ stamps) {
-  __shared__ float s_red[4][64 * kGenMaxCols];
+  __shared__ float s_red[4][64 * MAXC];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int slice = blockIdx.x / a.S;
   const int seg = blockIdx.x - slice * a.S;
@@ -586,13 +585,13 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
   const float dec = has_decay ? decay.v[hh] : 1.0f;
   const int ncol = (d + 63) >> 6;
 
-  float acc[kGenMaxCols];
+  float acc[MAXC];
 #pragma unroll
-  for (int j = 0; j < kGenMaxCols; ++j) acc[j] = 0.0f;
+  for (int j = 0; j < MAXC; ++j) acc[j] = 0.0f;
 
   // Lane l < 16 prepares row wave + 4l of this segment: its query value, whether the row is visited and,
   // for a lazily decayed state, the factor that brings it up to date.  The ballot lists the rows to visit;
-  // they are then walked in index order, kGenFlight rows in flight at a time.
+  // they are then walked in index order, FL rows in flight at a time.
   const bool lazy = rotary == BDH_ALIBI && stamps != nullptr;
   const long clock = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
   int32_t *st = lazy ? stamps + (long)slice * Nq : nullptr;
@@ -626,42 +625,42 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
     }
   }
   const bool has_dec = rotary == BDH_ALIBI;  // src/model/bdh.rs:299-301
-  float vv[kGenMaxCols];
+  float vv[MAXC];
 #pragma unroll
-  for (int j = 0; j < kGenMaxCols; ++j) {
+  for (int j = 0; j < MAXC; ++j) {
     const int c = j * 64 + lane;
     vv[j] = (j < ncol && c < d) ? vrow[c] : 0.0f;
   }
   unsigned long long m = __ballot(touch_l);
   while (m) {
-    int ls[kGenFlight];
-    bool ok[kGenFlight];
-    float rv[kGenFlight][kGenMaxCols];
+    int ls[FL];
+    bool ok[FL];
+    float rv[FL][MAXC];
 #pragma unroll
-    for (int u = 0; u < kGenFlight; ++u) {
+    for (int u = 0; u < FL; ++u) {
       ok[u] = m != 0ull;
       ls[u] = ok[u] ? __builtin_ctzll(m) : 0;
       if (ok[u]) m &= m - 1;
     }
 #pragma unroll
-    for (int u = 0; u < kGenFlight; ++u) {
+    for (int u = 0; u < FL; ++u) {
       if (ok[u]) {
         const RhoT *row = rho + ((long)slice * Nq + seg * kGenRows + wave + 4 * ls[u]) * d;
 #pragma unroll
-        for (int j = 0; j < kGenMaxCols; ++j) {
+        for (int j = 0; j < MAXC; ++j) {
           const int c = j * 64 + lane;
           if (j < ncol && c < d) rv[u][j] = rho_load<RhoT>(row + c);
         }
       }
     }
 #pragma unroll
-    for (int u = 0; u < kGenFlight; ++u) {
+    for (int u = 0; u < FL; ++u) {
       const float qn = __shfl(q_l, ls[u], 64);
       const float scale = __shfl(scale_l, ls[u], 64);
       if (ok[u]) {
         RhoT *row = rho + ((long)slice * Nq + seg * kGenRows + wave + 4 * ls[u]) * d;
 #pragma unroll
-        for (int j = 0; j < kGenMaxCols; ++j) {
+        for (int j = 0; j < MAXC; ++j) {
           const int c = j * 64 + lane;
           if (j < ncol && c < d) {
             float r = rv[u][j];
@@ -678,7 +677,7 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
   }
   if (lazy && touch_l) st[n_l] = (int32_t)min(clock + 1, 0x7fffffffL);
 #pragma unroll
-  for (int j = 0; j < kGenMaxCols; ++j) s_red[wave][j * 64 + lane] = acc[j];
+  for (int j = 0; j < MAXC; ++j) s_red[wave][j * 64 + lane] = acc[j];
   __syncthreads();
   float *pout = a.partial + (long)blockIdx.x * d;
   for (int c = tid; c < d; c += 256) {
@@ -1123,13 +1122,18 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
         BDH_LAUNCH_CHECK(ctx, "k_bitmask_rows");
       }
     } else {
-      if (p.rho_dtype == BDH_F32)
-        hipLaunchKernelGGL(k_step_generic<float>, dim3(slices * S), dim3(256), 0, ctx->stream, a,
-                           static_cast<float *>(p.rho), d, Nq, p.rotary, has_decay, decay, log_decay, p.stamps);
-      else
-        hipLaunchKernelGGL(k_step_generic<unsigned short>, dim3(slices * S), dim3(256), 0, ctx->stream, a,
-                           static_cast<unsigned short *>(p.rho), d, Nq, p.rotary, has_decay, decay, log_decay,
-                           p.stamps);
+      // registers for the columns a row really has: the narrower the rows, the more of them in flight
+#define BDH_GEN(T_, MAXC_, FL_)                                                                                   \
+  hipLaunchKernelGGL((k_step_generic<T_, MAXC_, FL_>), dim3(slices * S), dim3(256), 0, ctx->stream, a,           \
+                     static_cast<T_ *>(p.rho), d, Nq, p.rotary, has_decay, decay, log_decay, p.stamps)
+      if (p.rho_dtype == BDH_F32) {
+        if (d <= 128) BDH_GEN(float, 2, 16); else if (d <= 256) BDH_GEN(float, 4, 8);
+        else if (d <= 512) BDH_GEN(float, 8, 4); else BDH_GEN(float, 16, 4);
+      } else {
+        if (d <= 128) BDH_GEN(unsigned short, 2, 16); else if (d <= 256) BDH_GEN(unsigned short, 4, 8);
+        else if (d <= 512) BDH_GEN(unsigned short, 8, 4); else BDH_GEN(unsigned short, 16, 4);
+      }
+#undef BDH_GEN
       BDH_LAUNCH_CHECK(ctx, "k_step_generic");
       launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
