@@ -127,6 +127,11 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     ctx->opt_lowrank_scalar = value;
     return BDH_OK;
   }
+  if (strcmp(name, "model.one_launch") == 0) {
+    if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "model.one_launch takes 0 or 1");
+    ctx->opt_model_one_launch = value;
+    return BDH_OK;
+  }
   if (strcmp(name, "state_step.dense_kernel") == 0) {
     if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "state_step.dense_kernel takes 0 or 1");
     ctx->opt_step_dense_kernel = value;

@@ -21,6 +21,7 @@ struct bdh_ctx {
   int opt_step_dense = -1;  // many-token state step as dense f32 products: -1 from T = 128, 0 never, 1 always
   int opt_lowrank_tile = 1;  // 0: relu_lowrank never takes the 64-row tile kernel
   int opt_decoder_mfma = 1;  // 0: the encoder E never takes the f32 matrix-core form
+  int opt_model_one_launch = 1;  // 0: a small model's decode step runs kernel by kernel like any other
   int opt_lowrank_scalar = 1;  // 0: relu_lowrank with 8 to 63 rows stages its inputs in LDS instead of scalar loads
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on
@@ -40,6 +41,11 @@ struct bdh_model {
 };
 
 int bdh_fail(bdh_ctx *ctx, int status, const char *fmt, ...);
+
+// model_small.hip: the one-launch decode step of a small model (T = 1, f32 state, RoPE or ALiBi)
+bool bdh_model_small_fits(const bdh_model_config &c);
+int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, float *rho, int32_t *stamps, int64_t position,
+                           const int32_t *positions_dev, float *logits, int64_t *next_tokens);
 
 // Grows ctx->ws to at least `bytes` (synchronises the stream before freeing the old one).
 int bdh_ws_reserve(bdh_ctx *ctx, size_t bytes);

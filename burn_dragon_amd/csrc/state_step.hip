@@ -655,8 +655,9 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
     }
 #pragma unroll
     for (int u = 0; u < FL; ++u) {
-      const float qn = __shfl(q_l, ls[u], 64);
-      const float scale = __shfl(scale_l, ls[u], 64);
+      const int lu = __builtin_amdgcn_readfirstlane(ls[u]);  // the row list is the same in every lane
+            const float qn = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(q_l), lu));
+      const float scale = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(scale_l), lu));
       if (ok[u]) {
         RhoT *row = rho + ((long)slice * Nq + seg * kGenRows + wave + 4 * ls[u]) * d;
 #pragma unroll

@@ -334,17 +334,78 @@ def test_config1_full_run_against_oracle(bda, corc):
 
 
 def test_decode_equals_prefill_on_device(bda):
-    """T tokens in one call == T single-token calls carrying the state."""
+    """T tokens in one call == T single-token calls carrying the state: bit for bit when the single-token calls
+    run kernel by kernel, to a few ulp when they take the one-launch decode step this model is small enough for
+    (its sums over state rows and over the decoder's k are taken in a tree of its own)."""
     cfg = bda.BDHConfig(n_layer=3, n_embd=256, n_head=4, mlp_internal_dim_multiplier=8, vocab_size=64)
     cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
     model = bda.BDH(cfg, DEV, seed=9)
     tokens = torch.randint(0, 64, (4, 6), generator=torch.Generator().manual_seed(1))
-    sa, sb = model.init_state(), model.init_state()
+    sa, sb, sc = model.init_state(), model.init_state(), model.init_state()
     la = model.forward_with_state(tokens, sa)
-    rows = [model.forward_with_state(tokens[:, t : t + 1], sb) for t in range(6)]
+    ctx = bda.ffi.default_context(0)
+    try:
+        ctx.set_option("model.one_launch", 0)
+        rows = [model.forward_with_state(tokens[:, t : t + 1], sb) for t in range(6)]
+    finally:
+        ctx.set_option("model.one_launch", 1)
     torch.cuda.synchronize()
     assert torch.equal(torch.cat(rows, 1), la)
     assert torch.equal(sa.storage, sb.storage) and sa.position == sb.position == 6
+    one = torch.cat([model.forward_with_state(tokens[:, t : t + 1], sc) for t in range(6)], 1)
+    torch.cuda.synchronize()
+    assert not torch.equal(one, torch.zeros_like(one))
+    assert rel_err(one.cpu().numpy(), la.cpu().numpy()) < 1e-5
+    assert rel_err(sc.storage.cpu().numpy(), sa.storage.cpu().numpy()) < 1e-5 and sc.position == 6
+
+
+@pytest.mark.parametrize("rotary,lazy", [("rope", False), ("alibi", False), ("alibi", True)])
+@pytest.mark.parametrize("d,h,mult,L,V", [(64, 1, 4, 2, 40), (128, 4, 4, 3, 69), (256, 8, 8, 2, 256), (32, 16, 16, 2, 17)])
+def test_one_launch_decode_step(bda, corc, rotary, lazy, d, h, mult, L, V):
+    """A small model's decode step (one token per sequence, no by-products) runs as ONE launch, a workgroup per
+    sequence.  Logits, state and greedy tokens against the C oracle (1e-3) and against the same steps run kernel by
+    kernel (1e-5: only the summation trees differ), after a prompt that went through the many-token path."""
+    cfg = bda.BDHConfig(n_layer=L, n_embd=d, n_head=h, mlp_internal_dim_multiplier=mult, vocab_size=V, dropout=0.0)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse(rotary))
+    shape = _shape_from_cfg(cfg)
+    w = orc.init_weights(shape, seed=d + h)
+    weights = {"embed": w.embed, "encoder": w.encoder, "encoder_v": w.encoder_v, "decoder": w.decoder, "lm_head": w.lm_head}
+    one = bda.BDH(cfg, DEV, weights=weights, alibi_lazy=lazy)
+    ref = bda.BDH(cfg, DEV, weights=weights, alibi_lazy=lazy)
+    B, T0, steps = 3, 5, 4
+    rng = np.random.default_rng(7 * d + h)
+    prompt = rng.integers(0, V, (B, T0))
+    N = one.latent
+    rho_ref = np.zeros((L, B, h, N, d), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, prompt, rho_ref, 0, sparse_state=False)
+    s_one, s_ref = one.init_state(), ref.init_state()
+    ctx = bda.ffi.default_context(0)
+    _, nxt = one.forward_with_state(torch.from_numpy(prompt), s_one, want_next=True)
+    ref.forward_with_state(torch.from_numpy(prompt), s_ref)
+    feed = logits_ref[:, -1].argmax(-1)
+    for step in range(steps):
+        tok = feed.reshape(B, 1)
+        logits_ref, pos, _, _ = corc.forward_with_state(shape, w, tok, rho_ref, pos, sparse_state=False)
+        got, nxt = one.forward_with_state(torch.from_numpy(tok), s_one, want_next=True)
+        try:
+            ctx.set_option("model.one_launch", 0)
+            kbk = ref.forward_with_state(torch.from_numpy(tok), s_ref)
+        finally:
+            ctx.set_option("model.one_launch", 1)
+        torch.cuda.synchronize()
+        got_np = got.cpu().numpy()
+        assert rel_err(got_np, logits_ref) < 1e-3, f"step {step} against the oracle"
+        assert rel_err(got_np, kbk.cpu().numpy()) < 1e-5, f"step {step} against the kernel-by-kernel step"
+        assert np.array_equal(nxt.cpu().numpy(), got_np[:, 0].argmax(-1))
+        feed = logits_ref[:, -1].argmax(-1)
+    assert s_one.position == T0 + steps == pos
+    one.materialize_state(s_one)
+    ref.materialize_state(s_ref)
+    torch.cuda.synchronize()
+    assert rel_err(s_one.storage.cpu().numpy(), rho_ref) < 1e-3
+    assert rel_err(s_one.storage.cpu().numpy(), s_ref.storage.cpu().numpy()) < 1e-5
+    if lazy:
+        assert torch.equal(s_one.stamps, s_ref.stamps)
 
 
 def test_bad_token_poisons_only_its_row(bda):
