@@ -579,24 +579,31 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
   const int slice = blockIdx.x / a.S;
   const int seg = blockIdx.x - slice * a.S;
   const int b = slice / a.h, hh = slice - b * a.h;
-  const float pos = a.pos_dev ? (float)((long)a.pos_dev[b] + a.pos_add) : a.pos_scalar;
-  const float *xs = a.x + (long)slice * a.x_slice_stride;
-  const float *vrow = a.v + (long)b * a.v_batch_stride;
   const float dec = has_decay ? decay.v[hh] : 1.0f;
   const int ncol = (d + 63) >> 6;
-
-  float acc[MAXC];
-#pragma unroll
-  for (int j = 0; j < MAXC; ++j) acc[j] = 0.0f;
 
   // Lane l < 16 prepares row wave + 4l of this segment: its query value, whether the row is visited and,
   // for a lazily decayed state, the factor that brings it up to date.  The ballot lists the rows to visit;
   // they are then walked in index order, FL rows in flight at a time.
   const bool lazy = rotary == BDH_ALIBI && stamps != nullptr;
-  const long clock = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
+  const long clock0 = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
   int32_t *st = lazy ? stamps + (long)slice * Nq : nullptr;
   const int n_l = seg * kGenRows + wave + 4 * lane;
   const bool in_range = lane < kGenRows / 4 && n_l < Nq;
+  // the stamp of this lane's row lives in a register over the tokens of the launch
+  long stamp_l = (lazy && in_range) ? (long)st[n_l] : 0;
+  bool stamp_dirty = false;
+
+  // Tokens of this launch, in order.  A workgroup touches only its own state rows, and the barriers of a
+  // token order its row stores before the row loads of the next.
+  for (int t = 0; t < a.nt; ++t) {
+  const long clock = clock0 + t;
+  const float pos = (float)clock;
+  const float *xs = a.x + (long)t * a.x_t_stride + (long)slice * a.x_slice_stride;
+  const float *vrow = a.v + (long)t * a.v_t_stride + (long)b * a.v_batch_stride;
+  float acc[MAXC];
+#pragma unroll
+  for (int j = 0; j < MAXC; ++j) acc[j] = 0.0f;
   float q_l = 0.0f, scale_l = 1.0f;
   bool touch_l = false;
   if (in_range) {
@@ -605,7 +612,7 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
       q_l = xs[n_l];
       touch_l = lazy ? (q_l != 0.0f) : true;
       if (lazy && touch_l) {
-        const long k = clock - (long)st[n_l];
+        const long k = clock - stamp_l;
         if (k > 0) scale_l = expf((float)k * log_decay.v[hh]);
       }
     } else if (rotary == BDH_ROPE) {
@@ -676,11 +683,14 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
       }
     }
   }
-  if (lazy && touch_l) st[n_l] = (int32_t)min(clock + 1, 0x7fffffffL);
+  if (lazy && touch_l) {
+    stamp_l = min(clock + 1, 0x7fffffffL);
+    stamp_dirty = true;
+  }
 #pragma unroll
   for (int j = 0; j < MAXC; ++j) s_red[wave][j * 64 + lane] = acc[j];
   __syncthreads();
-  float *pout = a.partial + (long)blockIdx.x * d;
+  float *pout = a.partial + (long)t * a.partial_t_stride + (long)blockIdx.x * d;
   for (int c = tid; c < d; c += 256) {
     float s = s_red[0][c];
     s += s_red[1][c];
@@ -688,6 +698,9 @@ __global__ __launch_bounds__(256) void k_step_generic(StepPtrs a, RhoT *__restri
     s += s_red[3][c];
     pout[c] = s;
   }
+  __syncthreads();  // s_red is written again by the next token
+  }
+  if (stamp_dirty) st[n_l] = (int32_t)stamp_l;
 }
 
 // ------------------------------------------------------------------------------------
@@ -1016,11 +1029,13 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   const bool dense_auto = T >= 128 && (!loop_is_cheap || state_tiles >= n_cu / 2);
   if (!p.bitmask && !p.rows_touched && chunk_fits && (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : dense_auto))
     return bdh_launch_state_chunks_f32(ctx, p, out_ln);
-  // tokens per launch: only the f32 RoPE kernel walks several, as many as 64 MiB of partials allow
+  // tokens per launch: the f32 RoPE kernel and the generic kernel walk several, as many as 64 MiB of partials allow
   const size_t partial_one = bdh_align_up(sizeof(float) * (size_t)slices * S * d, 256);
   const size_t cnt_one = bdh_align_up(sizeof(int) * (size_t)slices * S, 256);
+  // (the generic kernel only when no per-token by-products are asked for)
+  const bool generic = !fast && !fast_lazy && !fast_dense;
   int group = 1;
-  if (fast && p.rho_dtype == BDH_F32 && T > 1)
+  if (T > 1 && ((fast && p.rho_dtype == BDH_F32) || (generic && !p.bitmask && !p.rows_touched)))
     group = (int)std::max<size_t>(1, std::min<size_t>((size_t)T, (size_t(64) << 20) / partial_one));
   const size_t partial_bytes = partial_one * group;
   const size_t cnt_bytes = cnt_one * group;
@@ -1136,7 +1151,8 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
       }
 #undef BDH_GEN
       BDH_LAUNCH_CHECK(ctx, "k_step_generic");
-      launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T);
+      launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T, 2, nt,
+                      a.partial_t_stride, a.cnt_t_stride);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
       if (a.bitmask || rows_t) {
         hipLaunchKernelGGL(k_bitmask_rows, dim3(slices), dim3(256), 0, ctx->stream, a, p.rotary, Nq, rows_t,
