@@ -128,7 +128,7 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     return BDH_OK;
   }
   if (strcmp(name, "model.one_launch") == 0) {
-    if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "model.one_launch takes 0 or 1");
+    if (value < 0 || value > 2) return bdh_fail(ctx, BDH_E_INVAL, "model.one_launch takes 0, 1 or 2");
     ctx->opt_model_one_launch = value;
     return BDH_OK;
   }

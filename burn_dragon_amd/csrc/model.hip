@@ -133,9 +133,15 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
   const size_t M = (size_t)B * T;
 
   // a decode step of a small model with no by-products: the whole step in one launch, a workgroup per sequence
-  if (T == 1 && !x_tap && !viz && rho_dtype == BDH_F32 && ctx->opt_model_one_launch != 0 && bdh_model_small_fits(c))
-    return bdh_launch_model_small(m, tokens, B, static_cast<float *>(rho), stamps, position, positions_dev, logits,
-                                  next_tokens);
+  // (one CU streams all the weights of a step, W bytes: measured on the reference's tiny / small / base sizes, W = 3,
+  // 6.75 and 12 MiB, the launch wins from 1, 2 and 8 sequences on)
+  if (T == 1 && !x_tap && !viz && rho_dtype == BDH_F32 && ctx->opt_model_one_launch != 0 && bdh_model_small_fits(c)) {
+    const size_t w_bytes = sizeof(float) * (size_t)3 * h * N * d * L;
+    const int b_min = w_bytes <= (size_t(4) << 20) ? 1 : (w_bytes <= (size_t(8) << 20) ? 2 : 8);
+    if (ctx->opt_model_one_launch == 2 || B >= b_min)
+      return bdh_launch_model_small(m, tokens, B, static_cast<float *>(rho), stamps, position, positions_dev, logits,
+                                    next_tokens);
+  }
 
   // activation scratch: cur [M,d] | x [B,h,T,N] | xy [B,h,T,N] | attn [B,h,T,d] | attn_ln [B,h,T,d] | last [h,d]
   const size_t n_cur = bdh_align_up(M * d, 64), n_x = bdh_align_up(M * h * N, 64), n_a = bdh_align_up(M * h * d, 64);

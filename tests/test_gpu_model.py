@@ -352,7 +352,11 @@ def test_decode_equals_prefill_on_device(bda):
     torch.cuda.synchronize()
     assert torch.equal(torch.cat(rows, 1), la)
     assert torch.equal(sa.storage, sb.storage) and sa.position == sb.position == 6
-    one = torch.cat([model.forward_with_state(tokens[:, t : t + 1], sc) for t in range(6)], 1)
+    try:
+        ctx.set_option("model.one_launch", 2)  # by default only from 8 sequences on for a model of this size
+        one = torch.cat([model.forward_with_state(tokens[:, t : t + 1], sc) for t in range(6)], 1)
+    finally:
+        ctx.set_option("model.one_launch", 1)
     torch.cuda.synchronize()
     assert not torch.equal(one, torch.zeros_like(one))
     assert rel_err(one.cpu().numpy(), la.cpu().numpy()) < 1e-5
@@ -386,8 +390,9 @@ def test_one_launch_decode_step(bda, corc, rotary, lazy, d, h, mult, L, V):
     for step in range(steps):
         tok = feed.reshape(B, 1)
         logits_ref, pos, _, _ = corc.forward_with_state(shape, w, tok, rho_ref, pos, sparse_state=False)
-        got, nxt = one.forward_with_state(torch.from_numpy(tok), s_one, want_next=True)
         try:
+            ctx.set_option("model.one_launch", 2)  # whatever the size and the batch
+            got, nxt = one.forward_with_state(torch.from_numpy(tok), s_one, want_next=True)
             ctx.set_option("model.one_launch", 0)
             kbk = ref.forward_with_state(torch.from_numpy(tok), s_ref)
         finally:
