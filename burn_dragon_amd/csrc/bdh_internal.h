@@ -22,6 +22,7 @@ struct bdh_ctx {
   int opt_lowrank_tile = 1;  // 0: relu_lowrank never takes the 64-row tile kernel
   int opt_decoder_mfma = 1;  // 0: the encoder E never takes the f32 matrix-core form
   int opt_model_one_launch = 1;  // small model's decode step in one launch: 1 when it pays, 2 whenever it fits, 0 never
+  int opt_lowrank_row = 1;     // 0: relu_lowrank with one input row and a small matrix uses the column-per-thread kernel
   int opt_lowrank_scalar = 1;  // 0: relu_lowrank with 8 to 63 rows stages its inputs in LDS instead of scalar loads
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on

@@ -76,6 +76,9 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       the dense streaming kernel, 0 = the generic kernel (same values).
  *   "relu_lowrank.scalar": 1 (default) calls with 8 to 63 rows read their inputs through the scalar
  *                       cache, 0 = stage them in LDS (same values).
+ *   "relu_lowrank.row": 1 (default) a call with one input row, 128 <= d <= 512 and at most 16 MiB of
+ *                       weights takes the kernel that keeps every weight in flight at once, 0 = the
+ *                       column-per-thread kernel (same values).
  *   "relu_lowrank.tile": 1 (default) calls with 64+ rows take the 64-row tile kernel (same values) when
  *                       its grid covers the chip, 2 = whenever the shape allows, 0 = never.
  *   "decoder.mfma":     1 (default) the encoder E of a call with 128+ tokens per sequence runs on

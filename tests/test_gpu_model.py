@@ -53,6 +53,35 @@ def test_relu_lowrank_fused_matches_reference(bda):
     assert_close(fused.cpu().numpy(), reference.numpy(), 1e-5, 1e-5)
 
 
+@pytest.mark.parametrize("d,N,h,h_in", [(128, 200, 4, 1), (192, 192, 4, 4), (256, 640, 4, 1), (320, 100, 2, 2), (512, 256, 8, 8)])
+def test_relu_lowrank_single_row_small_matrix_bit_exact(bda, corc, d, N, h, h_in):
+    """One input row against a matrix of a few MiB takes the kernel whose waves each fetch a 64-row span of k at once and
+    hand the fmaf chain on in k order: same bits as the oracle's k-sequential chain and as the column-per-thread kernel,
+    with bias, threshold and gate, for d that is and is not a multiple of the spans."""
+    from burn_dragon_amd.kernel import relu_lowrank
+
+    rng = np.random.default_rng(d + N)
+    inp = rng.standard_normal((1, h_in, 1, d)).astype(np.float32)
+    weight = (0.05 * rng.standard_normal((h, d, N))).astype(np.float32)
+    bias = (0.1 * rng.standard_normal((h, 1, N))).astype(np.float32)
+    gate = np.maximum(rng.standard_normal((1, h, 1, N)), 0).astype(np.float32)
+    ref = corc.relu_lowrank(inp, weight, bias.reshape(h, N), 0.125)
+    dense = bda.BlockPattern1d.dense(64)
+    args = (torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), torch.from_numpy(bias).to(DEV), 0.125, dense)
+    got = relu_lowrank.fused_forward(*args)
+    gated = relu_lowrank.fused_forward(*args, gate=torch.from_numpy(gate).to(DEV))
+    ctx = bda.ffi.default_context(0)
+    try:
+        ctx.set_option("relu_lowrank.row", 0)
+        plain = relu_lowrank.fused_forward(*args)
+    finally:
+        ctx.set_option("relu_lowrank.row", 1)
+    assert np.array_equal(got.cpu().numpy(), ref)
+    assert np.array_equal(plain.cpu().numpy(), ref)
+    assert np.array_equal(gated.cpu().numpy(), gate * ref)
+    assert 0.2 < (ref > 0).mean() < 0.8
+
+
 @pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (8, 1, 1), (17, 1, 4), (32, 1, 1), (1, 64, 4), (2, 100, 1),
                                       (3, 43, 4)])
 def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
