@@ -244,10 +244,10 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
           }
 #pragma unroll
           for (int u = 0; u < kFlight; ++u) {
-            if (ok[u]) {
-              const float *row = rho + (size_t)(row0 + base + ls[u]) * d;
-              if (has_c) load_vec<MAXC>(row + lane * MAXC, rv[u]);
-            }
+            // unconditional (an unused slot reads the wave's first row again): loads under a branch are not
+            // issued back to back
+            const float *row = rho + (size_t)(row0 + base + ls[u]) * d;
+            load_vec<MAXC>(row + (has_c ? lane * MAXC : 0), rv[u]);
           }
 #pragma unroll
           for (int u = 0; u < kFlight; ++u) {
