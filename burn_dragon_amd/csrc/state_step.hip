@@ -733,14 +733,18 @@ __global__ __launch_bounds__(256) void k_step_dense(StepPtrs a, RhoT *__restrict
   const int slice = blockIdx.x / a.S;
   const int seg = blockIdx.x - slice * a.S;
   const int b = slice / a.h, hh = slice - b * a.h;
-  const float pos = a.pos_dev ? (float)((long)a.pos_dev[b] + a.pos_add) : a.pos_scalar;
-  const float *xs = a.x + (long)slice * a.x_slice_stride;
+  const long clock0 = a.pos_dev ? (long)a.pos_dev[b] + a.pos_add : a.pos_int;
   const bool has_decay = rotary == BDH_ALIBI;
   const float dec = has_decay ? decay.v[hh] : 1.0f;
 
+  // Tokens of this launch, in order.  A workgroup touches only its own state rows, and the barriers of a
+  // token order its row stores before the row loads of the next.
+  for (int t = 0; t < a.nt; ++t) {
+  const float pos = (float)(clock0 + t);
+  const float *xs = a.x + (long)t * a.x_t_stride + (long)slice * a.x_slice_stride;
   float4 acc[VPL], vv[VPL];
   {
-    const float4 *vrow = reinterpret_cast<const float4 *>(a.v + (long)b * a.v_batch_stride);
+    const float4 *vrow = reinterpret_cast<const float4 *>(a.v + (long)t * a.v_t_stride + (long)b * a.v_batch_stride);
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -806,15 +810,17 @@ __global__ __launch_bounds__(256) void k_step_dense(StepPtrs a, RhoT *__restrict
 #pragma unroll
   for (int j = 0; j < VPL; ++j) s_red[wave][j * 64 + lane] = acc[j];
   __syncthreads();
-  float *pout = a.partial + (long)blockIdx.x * D;
+  float *pout = a.partial + (long)t * a.partial_t_stride + (long)blockIdx.x * D;
   for (int c4 = tid; c4 < D / 4; c4 += 256) {
     float4 s = s_red[0][c4];
 #pragma unroll
     for (int w = 1; w < 4; ++w) {
-      const float4 t = s_red[w][c4];
-      s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+      const float4 p4 = s_red[w][c4];
+      s.x += p4.x; s.y += p4.y; s.z += p4.z; s.w += p4.w;
     }
     reinterpret_cast<float4 *>(pout)[c4] = s;
+  }
+  __syncthreads();  // s_red is written again by the next token
   }
 }
 
@@ -1029,11 +1035,12 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   const bool dense_auto = T >= 128 && (!loop_is_cheap || state_tiles >= n_cu / 2);
   if (!p.bitmask && !p.rows_touched && chunk_fits && (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : dense_auto))
     return bdh_launch_state_chunks_f32(ctx, p, out_ln);
-  // tokens per launch: the f32 RoPE kernel and the generic kernel walk several, as many as 64 MiB of partials allow
+  // tokens per launch: the f32 RoPE kernel, the generic and the dense streaming kernel walk several, as many as
+  // 64 MiB of partials allow
   const size_t partial_one = bdh_align_up(sizeof(float) * (size_t)slices * S * d, 256);
   const size_t cnt_one = bdh_align_up(sizeof(int) * (size_t)slices * S, 256);
-  // (the generic kernel only when no per-token by-products are asked for)
-  const bool generic = !fast && !fast_lazy && !fast_dense;
+  // (the latter two only when no per-token by-products are asked for)
+  const bool generic = !fast && !fast_lazy;  // k_step_generic or k_step_dense
   int group = 1;
   if (T > 1 && ((fast && p.rho_dtype == BDH_F32) || (generic && !p.bitmask && !p.rows_touched)))
     group = (int)std::max<size_t>(1, std::min<size_t>((size_t)T, (size_t(64) << 20) / partial_one));
@@ -1130,7 +1137,8 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
         else hipLaunchKernelGGL((k_step_dense<unsigned short, 512, 4>), grid, dim3(256), 0, ctx->stream, a, rho, Nq, p.rotary, decay);
       }
       BDH_LAUNCH_CHECK(ctx, "k_step_dense");
-      launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T);
+      launch_finalize(ctx->stream, slices, partial, nullptr, S, d, out_t, (long)T * d, out_ln_t, nullptr, (long)T, 2, nt,
+                      a.partial_t_stride, a.cnt_t_stride);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");
       if (a.bitmask || rows_t) {
         hipLaunchKernelGGL(k_bitmask_rows, dim3(slices), dim3(256), 0, ctx->stream, a, p.rotary, Nq, rows_t,
