@@ -126,36 +126,19 @@ __device__ __forceinline__ float matvec_cols(const float *s_in, int K, const flo
   return v;
 }
 
-// MAXC adjacent floats as one access (the address is MAXC*4-byte aligned)
-template <int MAXC>
-__device__ __forceinline__ void load_vec(const float *p, float *out) {
-  if constexpr (MAXC == 4) {
-    const float4 v = *reinterpret_cast<const float4 *>(p);
-    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
-  } else if constexpr (MAXC == 2) {
-    const float2 v = *reinterpret_cast<const float2 *>(p);
-    out[0] = v.x; out[1] = v.y;
-  } else {
-    out[0] = *p;
-  }
-}
-template <int MAXC>
-__device__ __forceinline__ void store_vec(float *p, const float *in) {
-  if constexpr (MAXC == 4) *reinterpret_cast<float4 *>(p) = make_float4(in[0], in[1], in[2], in[3]);
-  else if constexpr (MAXC == 2) *reinterpret_cast<float2 *>(p) = make_float2(in[0], in[1]);
-  else *p = in[0];
-}
-
-// MAXC: columns of a state row per lane (d <= 64 * MAXC); 32 / MAXC state rows are in flight per wave
-template <int MAXC>
+// LPR: lanes per state row, four adjacent columns each (d <= 4 * LPR); a wave instruction covers 64 / LPR rows and
+// 8 such groups of rows are in flight per wave
+template <int LPR>
 __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
-  constexpr int kFlight = 32 / MAXC;
+  constexpr int RPI = 64 / LPR;  // rows per instruction
+  constexpr int kFlight = 8;
   __shared__ float s_cur[kMaxD];
   __shared__ float s_x[kMaxCols];
   __shared__ float s_xy[kMaxCols];
   __shared__ float s_attn[16 * kMaxD];  // [h][d]: readout, then its LayerNorm
   __shared__ float s_red[kWaves][kMaxD];
   __shared__ float s_st[8];
+  __shared__ unsigned char s_list[kWaves][64];  // per wave: the lanes whose rows are visited, compacted
   __shared__ float s_best[kWaves];
   __shared__ int s_arg[kWaves];
 
@@ -196,12 +179,14 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
       int32_t *st = a.stamps ? a.stamps + (size_t)l * a.stamps_layer_stride + (size_t)b * cols : nullptr;
       const bool lazy = alibi && st != nullptr;
       const float dec = alibi ? a.decay[hh_w] : 1.0f;
-      const bool has_c = lane * MAXC < d;  // a lane owns MAXC adjacent columns (d % MAXC == 0): one access per row
-      float acc[MAXC], vv[MAXC];
+      const int sub = lane / LPR, cl = lane - sub * LPR;  // this lane's row within an instruction, its column group
+      const bool has_c = cl * 4 < d;                      // d % 4 == 0
+      const int coff = has_c ? cl * 4 : 0;
+      float acc[4], vv[4];
 #pragma unroll
-      for (int j = 0; j < MAXC; ++j) {
+      for (int j = 0; j < 4; ++j) {
         acc[j] = 0.0f;
-        vv[j] = has_c ? s_cur[lane * MAXC + j] : 0.0f;
+        vv[j] = has_c ? s_cur[cl * 4 + j] : 0.0f;
       }
       for (int base = 0; base < rpw; base += 64) {
         const int r_l = row0 + base + lane;  // this lane prepares row r_l
@@ -231,52 +216,57 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
             }
           }
         }
-        unsigned long long m = __ballot(touch_l);
-        while (m) {
-          int ls[kFlight];
+        const unsigned long long m = __ballot(touch_l);
+        const int count = __popcll(m);
+        if (touch_l) s_list[wave][__popcll(m & ((1ull << lane) - 1ull))] = (unsigned char)lane;
+        // (LDS operations of one wave execute in order: the list is read back below without a barrier)
+        for (int i0 = 0; i0 < count; i0 += kFlight * RPI) {
+          int src[kFlight];
           bool ok[kFlight];
-          float rv[kFlight][MAXC];
+          float4 rv[kFlight];
 #pragma unroll
           for (int u = 0; u < kFlight; ++u) {
-            ok[u] = m != 0ull;
-            ls[u] = ok[u] ? __builtin_ctzll(m) : 0;
-            if (ok[u]) m &= m - 1;
+            const int idx = i0 + u * RPI + sub;
+            const int listed = s_list[wave][idx & 63];  // read whether or not the slot is used: no branch
+            ok[u] = idx < count;
+            src[u] = ok[u] ? listed : 0;
           }
+          // unconditional loads (an unused slot reads the wave's first row again): loads under a branch are not
+          // issued back to back
+#pragma unroll
+          for (int u = 0; u < kFlight; ++u)
+            rv[u] = *reinterpret_cast<const float4 *>(rho + (size_t)(row0 + base + src[u]) * d + coff);
 #pragma unroll
           for (int u = 0; u < kFlight; ++u) {
-            // unconditional (an unused slot reads the wave's first row again): loads under a branch are not
-            // issued back to back
-            const float *row = rho + (size_t)(row0 + base + ls[u]) * d;
-            load_vec<MAXC>(row + (has_c ? lane * MAXC : 0), rv[u]);
-          }
+            const float q_src = __shfl(q_l, src[u], 64);
+            const float scale = __shfl(scale_l, src[u], 64);
+            const float qn = ok[u] ? q_src : 0.0f;
+            float r[4] = {rv[u].x, rv[u].y, rv[u].z, rv[u].w};
 #pragma unroll
-          for (int u = 0; u < kFlight; ++u) {
-            const int lu = __builtin_amdgcn_readfirstlane(ls[u]);  // the row list is the same in every lane
-            const float qn = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(q_l), lu));
-            const float scale = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(scale_l), lu));
-            if (ok[u]) {
-              float *row = rho + (size_t)(row0 + base + ls[u]) * d;
-              if (has_c) {
-#pragma unroll
-                for (int j = 0; j < MAXC; ++j) {
-                  float r = rv[u][j];
-                  if (lazy) r = r * scale;
-                  acc[j] = __builtin_fmaf(r, qn, acc[j]);
-                  const float outer = qn * vv[j];
-                  r = r + outer;
-                  if (alibi) r = r * dec;  // src/model/bdh.rs:299-301
-                  rv[u][j] = r;
-                }
-                store_vec<MAXC>(row + lane * MAXC, rv[u]);
-              }
+            for (int j = 0; j < 4; ++j) {
+              float e = ok[u] ? r[j] : 0.0f;
+              if (lazy) e = e * scale;
+              acc[j] = __builtin_fmaf(e, qn, acc[j]);
+              const float outer = qn * vv[j];
+              e = e + outer;
+              if (alibi) e = e * dec;  // src/model/bdh.rs:299-301
+              r[j] = e;
             }
+            if (ok[u] && has_c)
+              *reinterpret_cast<float4 *>(rho + (size_t)(row0 + base + src[u]) * d + coff) = make_float4(r[0], r[1], r[2], r[3]);
           }
         }
         if (lazy && touch_l) st[r_l] = (int32_t)min(pos + 1, 0x7fffffffL);
       }
+      // the rows of one instruction sit side by side in the wave: fold them onto the first LPR lanes
 #pragma unroll
-      for (int j = 0; j < MAXC; ++j)
-        if (has_c) s_red[wave][lane * MAXC + j] = acc[j];
+      for (int o = LPR; o < 64; o <<= 1)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] += __shfl_xor(acc[j], o, 64);
+      if (sub == 0 && has_c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s_red[wave][cl * 4 + j] = acc[j];
+      }
     }
     __syncthreads();
     for (int i = tid; i < h * d; i += kThreads) {  // the waves of a head, in order
@@ -409,11 +399,11 @@ int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, float *rh
       a.log_decay[i] = (float)log((double)a.decay[i]);  // of the rounded factor, as the lazy state step
     }
   if (a.d <= 64)
-    hipLaunchKernelGGL(k_model_step_small<1>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
+    hipLaunchKernelGGL(k_model_step_small<16>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
   else if (a.d <= 128)
-    hipLaunchKernelGGL(k_model_step_small<2>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
+    hipLaunchKernelGGL(k_model_step_small<32>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
   else
-    hipLaunchKernelGGL(k_model_step_small<4>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
+    hipLaunchKernelGGL(k_model_step_small<64>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
   BDH_LAUNCH_CHECK(ctx, "k_model_step_small");
   return BDH_OK;
 }
