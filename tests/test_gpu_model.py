@@ -382,7 +382,7 @@ def test_decode_equals_prefill_on_device(bda):
     assert torch.equal(torch.cat(rows, 1), la)
     assert torch.equal(sa.storage, sb.storage) and sa.position == sb.position == 6
     try:
-        ctx.set_option("model.one_launch", 2)  # by default only from 8 sequences on for a model of this size
+        ctx.set_option("model.one_launch", 2)  # whatever the size and the batch
         one = torch.cat([model.forward_with_state(tokens[:, t : t + 1], sc) for t in range(6)], 1)
     finally:
         ctx.set_option("model.one_launch", 1)
