@@ -102,29 +102,40 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank(const float *__restrict__
   }
 }
 
-// One input row against a SMALL weight matrix (a few MiB: it sits in the L2): with one thread per column there
-// are only a handful of workgroups and each thread walks k in rounds of 64 loads.  Here NW waves share 64
+// A few input rows against a SMALL weight matrix (a few MiB: it sits in the L2): with one thread per column there
+// are only a handful of workgroups and each thread walks k in rounds of loads.  Here NW waves share 64
 // columns: each wave asks for its own 64-row span of k at once, so every weight of the matrix is in flight
 // together, and the waves then extend the column's fmaf chain one after the other in k order (the accumulator
 // is handed on through LDS) -- the same k-sequential chain per output as k_relu_lowrank.  Measured per decode
 // step of a whole model: 4 x 1 MiB (d=256) 141 -> 132 us, 8 x 4 MiB (d=512) 389 -> 317 us; 32 MiB a tie; at
 // 256 MiB the column-per-thread kernel is 1 % ahead, hence the size limit at the call site.
-template <int NW>
-__global__ __launch_bounds__(NW * 64) void k_relu_lowrank_row(const float *__restrict__ in, int h_in, int d,
+template <int NW, int RT>
+__global__ __launch_bounds__(NW * 64) void k_relu_lowrank_row(const float *__restrict__ in, int h_in, int T, int d,
                                                              const float *__restrict__ w, int h, int N,
                                                              const float *__restrict__ bias, float thr,
                                                              const unsigned char *__restrict__ block_active,
                                                              int block_size, int n_blocks,
-                                                             const float *__restrict__ gate, float *__restrict__ out) {
-  __shared__ float s_in[NW * 64];
-  __shared__ float s_acc[64];
+                                                             const float *__restrict__ gate, float *__restrict__ out,
+                                                             int M) {
+  __shared__ float s_in[RT][NW * 64];
+  __shared__ float s_acc[RT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int hh = blockIdx.y;
   const int n = blockIdx.x * 64 + lane;
+  const int m0 = blockIdx.z * RT;
   const bool valid = n < N;
   const int k_lo = wave * 64;
-  // loads return in issue order: the input row first, it is needed first
-  const float xin = (int)threadIdx.x < d ? in[(long)(h_in == 1 ? 0 : hh) * d + threadIdx.x] : 0.0f;
+  // loads return in issue order: the input rows first, they are needed first
+  float xin[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int m = m0 + r;
+    xin[r] = 0.0f;
+    if ((int)threadIdx.x < d && m < M) {
+      const int b = m / T, t = m - b * T;
+      xin[r] = in[(((long)b * h_in + (h_in == 1 ? 0 : hh)) * T + t) * d + threadIdx.x];
+    }
+  }
   // unconditional loads (rows past d are clamped to the last one and not used): a load under a branch would
   // be waited for before the next one is issued
   const float *wp = w + (long)hh * d * N + (valid ? n : 0);
@@ -134,36 +145,62 @@ __global__ __launch_bounds__(NW * 64) void k_relu_lowrank_row(const float *__res
     const float t = wp[(long)min(k_lo + u, d - 1) * N];
     wv[u] = k_lo + u < d ? t : 0.0f;  // a select, not a branch; s_in is zero there too, so the term is +0
   }
-  float gv = 1.0f, bv = 0.0f;
-  if (wave == NW - 1 && valid) {
-    if (gate) gv = gate[(long)hh * N + n];
-    if (bias) bv = bias[(long)hh * N + n];
+  float gv[RT], bv = 0.0f;
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int m = m0 + r;
+    gv[r] = 1.0f;
+    if (wave == NW - 1 && valid && gate && m < M) {
+      const int b = m / T, t = m - b * T;
+      gv[r] = gate[(((long)b * h + hh) * T + t) * N + n];
+    }
   }
-  s_in[threadIdx.x] = xin;
+  if (wave == NW - 1 && valid && bias) bv = bias[(long)hh * N + n];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) s_in[r][threadIdx.x] = xin[r];
   __syncthreads();
-  float acc = 0.0f;
+  float acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = 0.0f;
 #pragma unroll
   for (int stage = 0; stage < NW; ++stage) {
     if (wave == stage) {
-      if (stage > 0) acc = s_acc[lane];
+      if (stage > 0) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) acc[r] = s_acc[r][lane];
+      }
       // unconditional, so that the LDS reads of the inputs are issued together
 #pragma unroll
-      for (int u = 0; u < 64; ++u) acc = __builtin_fmaf(s_in[k_lo + u], wv[u], acc);
-      if (stage < NW - 1) s_acc[lane] = acc;
+      for (int u = 0; u < 64; ++u)
+#pragma unroll
+        for (int r = 0; r < RT; ++r) acc[r] = __builtin_fmaf(s_in[r][k_lo + u], wv[u], acc[r]);
+      if (stage < NW - 1) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) s_acc[r][lane] = acc[r];
+      }
     }
     if (stage < NW - 1) __syncthreads();
   }
   if (wave != NW - 1 || !valid) return;
-  float p = acc;
-  if (bias) p = p + bv;
-  if (thr != 0.0f) p = p - thr;
-  float y = p > 0.0f ? p : 0.0f;
+  float maskv = 1.0f;
   if (block_active) {
     const int blk = n / block_size;
-    y = y * ((blk < n_blocks && block_active[blk]) ? 1.0f : 0.0f);
+    maskv = (blk < n_blocks && block_active[blk]) ? 1.0f : 0.0f;
   }
-  if (gate) y = gv * y;
-  out[(long)hh * N + n] = y;
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    const int m = m0 + r;
+    if (m < M) {
+      const int b = m / T, t = m - b * T;
+      float p = acc[r];
+      if (bias) p = p + bv;
+      if (thr != 0.0f) p = p - thr;
+      float y = p > 0.0f ? p : 0.0f;
+      if (block_active) y = y * maskv;
+      if (gate) y = gv[r] * y;
+      out[(((long)b * h + hh) * T + t) * N + n] = y;
+    }
+  }
 }
 
 // A few input rows (a batch of 8 to 63 sequences decoding together) without LDS: the inputs of a row tile
@@ -688,6 +725,37 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
     BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_tile");
     return BDH_OK;
   }
+  // A matrix of up to 16 MiB (it sits in the L2) whose column-per-thread grid would leave most CUs idle, or a single
+  // row: 64 columns per workgroup, every weight in flight at once, as many rows per workgroup (1, 2, 4, 8) as still
+  // give a workgroup per CU
+  const int n_cu_rl = ctx->n_cu > 0 ? ctx->n_cu : 256;
+  if (p.d >= 128 && p.d <= 512 && ctx->opt_lowrank_row != 0 &&
+      sizeof(float) * (size_t)p.h * p.d * p.N <= (size_t(16) << 20) &&
+      (M == 1 || (long)((p.N + 255) / 256) * p.h * ((M + 15) / 16) < n_cu_rl)) {
+    const long col_blocks = (p.N + 63) / 64;
+    int rt = 1;
+    if (M > 1) {
+      rt = 8;
+      while (rt > 1 && col_blocks * p.h * ((M + rt - 1) / rt) < n_cu_rl) rt >>= 1;
+      while (rt > M) rt >>= 1;
+    }
+    const long row_tiles = (M + rt - 1) / rt;
+    if (row_tiles > 65535 || p.h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (row tiles %ld)", row_tiles);
+    const dim3 grid((unsigned)col_blocks, p.h, (unsigned)row_tiles);
+#define BDH_ROW(NW_, RT_)                                                                                             \
+  hipLaunchKernelGGL((k_relu_lowrank_row<NW_, RT_>), grid, dim3(NW_ * 64), 0, ctx->stream, p.in, p.h_in, p.T, p.d,   \
+                     p.weight, p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M)
+#define BDH_ROW_RT(NW_)                                                                           \
+  do {                                                                                            \
+    if (rt == 8) BDH_ROW(NW_, 8); else if (rt == 4) BDH_ROW(NW_, 4); else if (rt == 2) BDH_ROW(NW_, 2); \
+    else BDH_ROW(NW_, 1);                                                                         \
+  } while (0)
+    if (p.d <= 128) BDH_ROW_RT(2); else if (p.d <= 256) BDH_ROW_RT(4); else BDH_ROW_RT(8);
+#undef BDH_ROW_RT
+#undef BDH_ROW
+    BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_row");
+    return BDH_OK;
+  }
   if (M >= 8 && ctx->opt_lowrank_scalar != 0) {
     // 8 to 63 rows: inputs through the scalar cache, 16 rows (two SGPR batches of 8 k) or 8 rows per pass
     const int rt = M >= 16 ? 16 : 8;
@@ -701,19 +769,6 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
       hipLaunchKernelGGL((k_relu_lowrank_sc<8, 8>), grid, dim3(256), 0, ctx->stream, p.in, p.h_in, p.T, p.d, p.weight,
                          p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M);
     BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_sc");
-    return BDH_OK;
-  }
-  if (M == 1 && p.d >= 128 && p.d <= 512 && ctx->opt_lowrank_row != 0 &&
-      sizeof(float) * (size_t)p.h * p.d * p.N <= (size_t(16) << 20)) {
-    // a single row against a matrix of up to 16 MiB: every weight in flight at once
-    if (p.h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (heads %d)", p.h);
-    const dim3 grid((p.N + 63) / 64, p.h);
-#define BDH_ROW(NW_)                                                                                                 \
-  hipLaunchKernelGGL((k_relu_lowrank_row<NW_>), grid, dim3(NW_ * 64), 0, ctx->stream, p.in, p.h_in, p.d, p.weight, p.h, \
-                     p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out)
-    if (p.d <= 128) BDH_ROW(2); else if (p.d <= 256) BDH_ROW(4); else BDH_ROW(8);
-#undef BDH_ROW
-    BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_row");
     return BDH_OK;
   }
   const int RT = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1));
