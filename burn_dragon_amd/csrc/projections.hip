@@ -820,7 +820,9 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
     BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
     return BDH_OK;
   }
-  if (T == 1 && M >= ctx->opt_decoder_splitk_rows && (K % 1024) == 0) {
+  // (only when its 32 x 64 tiles over k-blocks of 1024 are enough workgroups for half the chip: not for a small model)
+  if (T == 1 && M >= ctx->opt_decoder_splitk_rows && (K % 1024) == 0 &&
+      (K / 1024) * ((d + 63) / 64) * ((M + 31) / 32) >= (ctx->n_cu > 0 ? ctx->n_cu : 256) / 2) {
     // a batch of decoding sequences: split-K product on the f32 matrix cores, KB = 1024
     const int KB = 1024;
     const int KBN = (int)(K / KB);
@@ -839,6 +841,8 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   // about two workgroups per CU: more k-blocks only add partials for the second stage to read
   int KB = 1024;
   while (KB > 128 && ((K + KB - 1) / KB) * row_tiles < 2L * (ctx->n_cu > 0 ? ctx->n_cu : 256)) KB >>= 1;
+  // a small model: down to 32 rows of E per workgroup, until there is a workgroup per CU
+  while (KB > 32 && ((K + KB - 1) / KB) * row_tiles < (ctx->n_cu > 0 ? ctx->n_cu : 256)) KB >>= 1;
   const int KBN = (int)((K + KB - 1) / KB);
   size_t lds = sizeof(float) * (size_t)RT * KB;
   if (lds < sizeof(float) * 4u * d) lds = sizeof(float) * 4u * d;
