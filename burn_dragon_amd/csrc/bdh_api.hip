@@ -143,7 +143,7 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     return BDH_OK;
   }
   if (strcmp(name, "decoder.splitk_rows") == 0) {
-    if (value < 1) return bdh_fail(ctx, BDH_E_INVAL, "decoder.splitk_rows takes a positive row count");
+    if (value == 0) return bdh_fail(ctx, BDH_E_INVAL, "decoder.splitk_rows takes a non-zero row count");
     ctx->opt_decoder_splitk_rows = value;
     return BDH_OK;
   }

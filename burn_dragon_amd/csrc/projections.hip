@@ -821,8 +821,10 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
     return BDH_OK;
   }
   // (only when its 32 x 64 tiles over k-blocks of 1024 are enough workgroups for half the chip: not for a small model)
-  if (T == 1 && M >= ctx->opt_decoder_splitk_rows && (K % 1024) == 0 &&
-      (K / 1024) * ((d + 63) / 64) * ((M + 31) / 32) >= (ctx->n_cu > 0 ? ctx->n_cu : 256) / 2) {
+  // (a negative option value -r takes it from r rows on whatever the grid)
+  const int sk_rows = ctx->opt_decoder_splitk_rows;
+  const bool sk_grid = (K / 1024) * ((d + 63) / 64) * ((M + 31) / 32) >= (ctx->n_cu > 0 ? ctx->n_cu : 256) / 2;
+  if (T == 1 && (K % 1024) == 0 && (sk_rows > 0 ? (M >= sk_rows && sk_grid) : M >= -(long)sk_rows)) {
     // a batch of decoding sequences: split-K product on the f32 matrix cores, KB = 1024
     const int KB = 1024;
     const int KBN = (int)(K / KB);

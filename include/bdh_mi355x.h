@@ -85,7 +85,9 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       the f32 matrix cores, 0 = always the VALU kernel.
  *   "decoder.splitk_rows": 24 (default) a decode step (T = 1) of this many or more sequences runs the
  *                       encoder E as a split-K product on the f32 matrix cores (all of E is streamed
- *                       once); fewer sequences take the VALU kernel that skips inactive rows of E.
+ *                       once) when its tiles cover half the chip; fewer sequences, and small models, take
+ *                       the VALU kernel that skips inactive rows of E.  A negative value -r takes the
+ *                       matrix-core form from r sequences on whatever the size.
  *   "model.one_launch": 1 (default) a decode step (T = 1, f32 state, no x_tap / viz) of a small model
  *                       (d <= 256 and d % 4 == 0, h * N <= 2048 and a multiple of 32, h in {1,2,4,8,16},
  *                       V <= 1024, RoPE or ALiBi) runs as one launch, a workgroup per sequence, when the
