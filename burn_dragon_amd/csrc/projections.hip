@@ -369,12 +369,32 @@ __global__ __launch_bounds__(256) void k_relu_lowrank_tile(const float *__restri
 // every thread walks it in index order, so mean and variance are the same left-to-right f32
 // sums a scalar loop produces, independent of the launch shape.
 // ------------------------------------------------------------------------------------
+// (s_row is 16-byte aligned; four values per LDS read, added one after the other in index order)
 __device__ __forceinline__ void ln_stats_in_order(const float *s_row, int d, float &mean, float &den) {
   float sum = 0.0f;
-  for (int i = 0; i < d; ++i) sum += s_row[i];
+  int i = 0;
+#pragma unroll 4
+  for (; i + 4 <= d; i += 4) {
+    const float4 v = *reinterpret_cast<const float4 *>(s_row + i);
+    sum += v.x;
+    sum += v.y;
+    sum += v.z;
+    sum += v.w;
+  }
+  for (; i < d; ++i) sum += s_row[i];
   mean = sum / (float)d;
   float sq = 0.0f;
-  for (int i = 0; i < d; ++i) {
+  i = 0;
+#pragma unroll 4
+  for (; i + 4 <= d; i += 4) {
+    const float4 v = *reinterpret_cast<const float4 *>(s_row + i);
+    float c;
+    c = v.x - mean; sq += c * c;
+    c = v.y - mean; sq += c * c;
+    c = v.z - mean; sq += c * c;
+    c = v.w - mean; sq += c * c;
+  }
+  for (; i < d; ++i) {
     const float c = s_row[i] - mean;
     sq += c * c;
   }
