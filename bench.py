@@ -370,6 +370,10 @@ def bench_chunks(args):
     }))
 
 
+# (n_layer, n_embd, n_head, mlp_internal_dim_multiplier) of the reference's config/{tiny,small,base,large}.toml
+SHIPPED_SIZES = {"tiny": (4, 128, 4, 4), "small": (4, 192, 4, 4), "base": (4, 256, 4, 4), "large": (8, 512, 8, 4)}
+
+
 def bench_model(args):
     """Full-model greedy decode (BDH::forward_with_state per token, argmax on the device).
     c1 = BASELINE config 1 (V=256, d=256, h=4, N=8192, L=6, B=1, 64-byte prompt, 256 tokens);
@@ -393,6 +397,17 @@ def bench_model(args):
         text = ("First Citizen:\nBefore we proceed any further, hear me speak.\n\nAll:\nSpeak, speak.\n" * 8)[:args.prompt]
         prompt = torch.tensor([tok.encode(text)] * B)
         weights_note = "trained tiny_shakespeare checkpoint (ALiBi, lazily decayed state)"
+    elif args.model_config in SHIPPED_SIZES:
+        # the sizes of the reference's config/*.toml (ALiBi, eagerly decayed f32 state), random-init weights
+        L_, d_, h_, mult_ = SHIPPED_SIZES[args.model_config]
+        cfg = bda.BDHConfig(n_layer=L_, n_embd=d_, n_head=h_, mlp_internal_dim_multiplier=mult_, vocab_size=256)
+        cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ALIBI)
+        B = 1 if args.batch == 32 else args.batch
+        steps = 256 if args.steps == 1000 else args.steps
+        model = bda.BDH(cfg, dev, seed=7, rho_dtype=rho_dtype, alibi_lazy=args.alibi_lazy)
+        if args.alibi_lazy:
+            weights_note += ", lazily decayed state"
+        prompt = torch.randint(0, 256, (B, args.prompt), generator=torch.Generator().manual_seed(1))
     else:
         if args.model_config == "c1":
             cfg = bda.BDHConfig(n_layer=6, n_embd=256, n_head=4, mlp_internal_dim_multiplier=128, vocab_size=256)
@@ -470,8 +485,10 @@ def main():
                          "alibi = ALiBi state step, lazily decayed state beside the eager dense decay; "
                          "parallel = fused_state_aligned in f32 at the config-3 shape; chunks = many-token state step "
                          "(f32 dense products) beside the token loop at the config-2 shape; copy = counter calibration")
-    ap.add_argument("--model-config", choices=["c1", "c4", "ckpt"], default="c1",
-                    help="model: config 1, config 4, or the trained tiny_shakespeare checkpoint of the test fixtures")
+    ap.add_argument("--model-config", choices=["c1", "c4", "ckpt", *SHIPPED_SIZES], default="c1",
+                    help="model: config 1, config 4, the trained tiny_shakespeare checkpoint of the test fixtures, or one "
+                         "of the sizes the reference ships configurations for (random-init, ALiBi)")
+    ap.add_argument("--alibi-lazy", action="store_true", help="model, shipped sizes: keep the ALiBi state lazily decayed")
     ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
     ap.add_argument("--graph", action="store_true", help="model: replay one captured HIP graph per token")
     ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")

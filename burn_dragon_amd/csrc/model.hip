@@ -134,10 +134,11 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
 
   // a decode step of a small model with no by-products: the whole step in one launch, a workgroup per sequence
   // (one CU streams all the weights of a step, W bytes: measured on the reference's tiny / small / base sizes, W = 3,
-  // 6.75 and 12 MiB, the launch wins from 1, 1 and 4 sequences on)
+  // 6.75 and 12 MiB, the launch wins always, from 8 to 64 and from 64 to 256 sequences on, depending on how sparse
+  // the state step is)
   if (T == 1 && !x_tap && !viz && rho_dtype == BDH_F32 && ctx->opt_model_one_launch != 0 && bdh_model_small_fits(c)) {
     const size_t w_bytes = sizeof(float) * (size_t)3 * h * N * d * L;
-    const int b_min = w_bytes <= (size_t(8) << 20) ? 1 : 4;
+    const int b_min = w_bytes <= (size_t(4) << 20) ? 1 : (w_bytes <= (size_t(8) << 20) ? 16 : 128);
     if (ctx->opt_model_one_launch == 2 || B >= b_min)
       return bdh_launch_model_small(m, tokens, B, static_cast<float *>(rho), stamps, position, positions_dev, logits,
                                     next_tokens);

@@ -91,8 +91,9 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *   "model.one_launch": 1 (default) a decode step (T = 1, f32 state, no x_tap / viz) of a small model
  *                       (d <= 256 and d % 4 == 0, h * N <= 2048 and a multiple of 32, h in {1,2,4,8,16},
  *                       V <= 1024, RoPE or ALiBi) runs as one launch, a workgroup per sequence, when the
- *                       batch is large enough for that to pay (always for up to 8 MiB of projection weights per
- *                       step, from 4 sequences on for more); 2 = whenever the model fits; 0 = kernel
+ *                       batch is large enough for that to pay (always for up to 4 MiB of projection weights per
+ *                       step, from 16 sequences on for up to 8 MiB, from 128 on for more); 2 = whenever the
+ *                       model fits; 0 = kernel
  *                       by kernel like any other call (values agree to 1e-5: other summation trees).
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
  *                       1 = the two products on the f32 matrix cores (T >= 128 by default). */
