@@ -694,7 +694,7 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
                        (long)h * N, (long)(p.position + T), p.positions_dev, T);
     BDH_LAUNCH_CHECK(ctx, "k_set_stamps");
   }
-  if (out_ln) return bdh_launch_layer_norm(ctx, (int64_t)S * T, d, p.out, out_ln);
+  if (out_ln) return bdh_launch_layer_norm_rows(ctx, (int64_t)S * T, d, p.out, out_ln);
   return BDH_OK;
 }
 

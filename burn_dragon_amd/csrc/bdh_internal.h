@@ -109,6 +109,8 @@ struct ReluLowrankParams {
 };
 int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p);
 int bdh_launch_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);
+// the same for internal many-row use: statistics by wave reduction, not bit-identical to the index-order sums
+int bdh_launch_layer_norm_rows(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);
 
 // embed gather + LN (src/model/bdh.rs:319-322); tokens validated on the device: an id
 // outside [0,V) writes NaN rows (the reference would panic in the gather).

@@ -412,6 +412,38 @@ __global__ __launch_bounds__(256) void k_layer_norm(const float *__restrict__ in
   for (int c = threadIdx.x; c < d; c += 256) y[c] = (s_row[c] - mean) / den;
 }
 
+// LayerNorm of many rows for internal use (the readout of a many-token state step): one wave per row, the
+// statistics by wave reduction instead of the index-order sums above (d <= 1024)
+__global__ __launch_bounds__(256) void k_layer_norm_wave(const float *__restrict__ in, float *__restrict__ out, int d,
+                                                         long rows) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long row = (long)blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  const float *x = in + row * d;
+  float *y = out + row * d;
+  float v[16], s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int c = j * 64 + lane;
+    v[j] = c < d ? x[c] : 0.0f;
+    s += v[j];
+  }
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  const float mean = s / (float)d;
+  float q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    if (j * 64 + lane < d) {
+      const float c = v[j] - mean;
+      q += c * c;
+    }
+  for (int o = 32; o > 0; o >>= 1) q += __shfl_xor(q, o);
+  const float den = sqrtf(q / (float)d + kLnEps);
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    if (j * 64 + lane < d) y[j * 64 + lane] = (v[j] - mean) / den;
+}
+
 // embed gather + LayerNorm (src/model/bdh.rs:319-322)
 __global__ __launch_bounds__(256) void k_embed_ln(const int64_t *__restrict__ tokens, int d, int V,
                                                   const float *__restrict__ embed, float *__restrict__ out) {
@@ -812,6 +844,16 @@ int bdh_launch_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, fl
   if (d > 16384) return bdh_fail(ctx, BDH_E_SHAPE, "LayerNorm row of %d floats does not fit in LDS", d);
   hipLaunchKernelGGL(k_layer_norm, dim3((unsigned)rows), dim3(256), sizeof(float) * (size_t)d, ctx->stream, in, out, d);
   BDH_LAUNCH_CHECK(ctx, "k_layer_norm");
+  return BDH_OK;
+}
+
+int bdh_launch_layer_norm_rows(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out) {
+  if (d > 1024) return bdh_launch_layer_norm(ctx, rows, d, in, out);
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many rows");
+  if (rows == 0) return BDH_OK;
+  hipLaunchKernelGGL(k_layer_norm_wave, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, out, d, (long)rows);
+  BDH_LAUNCH_CHECK(ctx, "k_layer_norm_wave");
   return BDH_OK;
 }
 
