@@ -610,8 +610,12 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
   const int nt_d = (d + 127) / 128;
   if ((long)groups * 8 * ((Nq + 127) / 128) * nt_d > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
 
+  const int n_cu = ctx->n_cu > 0 ? ctx->n_cu : 256;
   for (int t0 = 0; t0 < T; t0 += (int)Tc) {
     const int tc = (int)std::min<long>(Tc, T - t0);
+    // a small model or a short call: with 128 x 128 tiles the products would run on a few CUs, each a chain of
+    // load latencies; 32 x 64 tiles give sixteen times the workgroups
+    const bool small_tiles = (long)8 * groups * ((tc + 127) / 128) * nt_d < n_cu;
     const float *qc = q;           // this chunk's rotated activations [S][tc][Nq]
     long q_batch = (long)tc * Nq;
     if (alibi) {
@@ -635,7 +639,11 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
       g.block_size = 1; g.tb = tc; g.h = h; g.use_alibi = 0; g.dense = 1;
       with_decay(g, FSA_DECAY_SCORES);
       const bool big = S * ((tc + 255) / 256) * ((tc + 255) / 256) >= 256;
-      if (big) {
+      if (small_tiles) {
+        g.mt = (tc + 31) / 32; g.nt = (tc + 63) / 64;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128),
+                           0, ctx->stream, g);
+      } else if (big) {
         g.mt = g.nt = (tc + 255) / 256;
         hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 256, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512),
                            0, ctx->stream, g);
@@ -653,9 +661,15 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
       g.lda = Nq; g.ldb = d; g.ldc = d; g.M = tc; g.N = d; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
       g.block_size = 1; g.h = h; g.dense = 0; g.beta = 0;
       with_decay(g, FSA_DECAY_ROWS);
-      g.mt = (tc + 127) / 128; g.nt = nt_d;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
-                         ctx->stream, g);
+      if (small_tiles) {
+        g.mt = (tc + 31) / 32; g.nt = (d + 63) / 64;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128), 0,
+                           ctx->stream, g);
+      } else {
+        g.mt = (tc + 127) / 128; g.nt = nt_d;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                           ctx->stream, g);
+      }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q rho>");
     }
     {  // out += S V   (K limited to the causal prefix of each row tile)
@@ -664,9 +678,15 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
       g.a_batch = (long)Tc * Tcp; g.b_batch = (long)T * d; g.c_batch = (long)T * d;
       g.lda = Tcp; g.ldb = d; g.ldc = d; g.M = tc; g.N = d; g.K = tc; g.b_div = h; g.n_slices = (int)S;
       g.block_size = 1; g.h = h; g.dense = 1; g.beta = 1;
-      g.mt = (tc + 127) / 128; g.nt = nt_d;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
-                         ctx->stream, g);
+      if (small_tiles) {
+        g.mt = (tc + 31) / 32; g.nt = (d + 63) / 64;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128), 0,
+                           ctx->stream, g);
+      } else {
+        g.mt = (tc + 127) / 128; g.nt = nt_d;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                           ctx->stream, g);
+      }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<S V>");
     }
     {  // rho += Q^T V   (both operands k-major: the reduction runs over the tokens)
@@ -677,9 +697,15 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
       g.lda = Nq; g.ldb = d; g.ldc = d; g.M = Nq; g.N = d; g.K = tc; g.b_div = h; g.n_slices = (int)S;
       g.block_size = 1; g.h = h; g.dense = 0; g.beta = 1;
       with_decay(g, FSA_DECAY_STATE);
-      g.mt = (Nq + 127) / 128; g.nt = nt_d;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
-                         ctx->stream, g);
+      if (small_tiles) {
+        g.mt = (Nq + 31) / 32; g.nt = (d + 63) / 64;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128), 0,
+                           ctx->stream, g);
+      } else {
+        g.mt = (Nq + 127) / 128; g.nt = nt_d;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                           ctx->stream, g);
+      }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q^T V>");
     }
   }

@@ -1035,7 +1035,7 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   // From 24 tokens on where the token loop has nothing to gain from sparsity: an f32 state that every token
   // streams in full anyway (PoPE, eager ALiBi), or one so small (up to 64 MiB) that the loop is a chain of launch
   // and barrier latencies (a 64-token prompt of the reference's tiny / base / large sizes: 1.5 / 1.4 / 3.5 ms
-  // token by token, 0.50 / 0.62 / 1.6 ms as dense products; a tie at 16 tokens).
+  // token by token, 0.27 / 0.34 / 0.95 ms as dense products; a tie at 16 tokens).
   const bool streamed = p.rho_dtype == BDH_F32 && (p.rotary == BDH_POPE || (p.rotary == BDH_ALIBI && !p.stamps));
   const bool small_state = p.rho_dtype == BDH_F32 && !loop_is_cheap &&
                            sizeof(float) * (size_t)slices * Nq * d <= (size_t(64) << 20);
