@@ -1027,20 +1027,21 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   // (not when even a 128-token chunk of rotated activations would pass 16 GiB of workspace)
   const bool chunk_fits = sizeof(float) * (size_t)slices * Nq * 128 <= (size_t(16) << 30) &&
                           (p.rho_dtype == BDH_F32 || sizeof(float) * (size_t)slices * Nq * d <= (size_t(64) << 30));
-  // By default from 128 tokens on (from 24 for the cases below); where the token loop is cheap (the f32 RoPE kernel walks many tokens per
+  // By default from 128 tokens on (from 8 for the cases below); where the token loop is cheap (the f32 RoPE kernel walks many tokens per
   // launch) only once the products have enough tiles to cover the chip (measured at N=8192, d=256, T=512:
   // B*h = 4 or 8 slices lose to the loop at 5 % density, 16 slices win at any density).
   const bool loop_is_cheap = fast && p.rho_dtype == BDH_F32;
   const long state_tiles = (long)slices * ((std::min(T, 512) + 127) / 128) * ((d + 127) / 128);
-  // From 24 tokens on where the token loop has nothing to gain from sparsity: an f32 state that every token
+  // From 8 tokens on where the token loop has nothing to gain from sparsity: an f32 state that every token
   // streams in full anyway (PoPE, eager ALiBi), or one so small (up to 64 MiB) that the loop is a chain of launch
   // and barrier latencies (a 64-token prompt of the reference's tiny / base / large sizes: 1.5 / 1.4 / 3.5 ms
-  // token by token, 0.27 / 0.34 / 0.95 ms as dense products; a tie at 16 tokens).
+  // token by token, 0.27 / 0.34 / 0.95 ms as dense products; at 8 tokens 0.30 / 0.29 / 0.69 against 0.22 / 0.27 /
+  // 0.59 ms, at 4 tokens the loop is ahead).
   const bool streamed = p.rho_dtype == BDH_F32 && (p.rotary == BDH_POPE || (p.rotary == BDH_ALIBI && !p.stamps));
   const bool small_state = p.rho_dtype == BDH_F32 && !loop_is_cheap &&
                            sizeof(float) * (size_t)slices * Nq * d <= (size_t(64) << 20);
   const bool dense_auto = (T >= 128 && (!loop_is_cheap || state_tiles >= n_cu / 2)) ||
-                          (T >= 24 && (streamed || small_state));
+                          (T >= 8 && (streamed || small_state));
   if (!p.bitmask && !p.rows_touched && chunk_fits && (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : dense_auto))
     return bdh_launch_state_chunks_f32(ctx, p, out_ln);
   // tokens per launch: the f32 RoPE kernel, the generic and the dense streaming kernel walk several, as many as

@@ -71,7 +71,7 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *   "state_step.dense_chunks": -1 (default) a call of 128+ tokens without
  *                       bitmask / row-count outputs runs as dense products on the f32 matrix cores
  *                       (with only a few (sequence, head) slices an f32 RoPE state keeps the token loop;
- *                       from 24 tokens on for an f32 state that every token streams in full -- PoPE,
+ *                       from 8 tokens on for an f32 state that every token streams in full -- PoPE,
  *                       eager ALiBi -- or that is at most 64 MiB),
  *                       0 = always token by token, 1 = dense products for any T.
  *   "state_step.dense_kernel": 1 (default) PoPE and eagerly decayed ALiBi steps at d in {256,512} take
