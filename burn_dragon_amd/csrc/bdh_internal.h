@@ -43,7 +43,7 @@ struct bdh_model {
 
 int bdh_fail(bdh_ctx *ctx, int status, const char *fmt, ...);
 
-// model_small.hip: the one-launch decode step of a small model (T = 1, f32 state, RoPE or ALiBi)
+// model_small.hip: the one-launch decode step of a small model (T = 1, f32 state)
 bool bdh_model_small_fits(const bdh_model_config &c);
 int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, float *rho, int32_t *stamps, int64_t position,
                            const int32_t *positions_dev, float *logits, int64_t *next_tokens);

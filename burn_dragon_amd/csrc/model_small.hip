@@ -161,11 +161,13 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
   }
   __syncthreads();
 
-  const int rpw = cols / kWaves;       // state rows per wave, all of one head
+  const bool alibi = a.rotary == BDH_ALIBI, pope = a.rotary == BDH_POPE;
+  const int Nq = pope ? 2 * N : N;     // PoPE: rows N..2N-1 of a head are the imaginary parts
+  const int srows = h * Nq;            // state rows of a sequence
+  const int rpw = srows / kWaves;      // state rows per wave, all of one head
   const int row0 = wave * rpw;
-  const int hh_w = row0 / N;
+  const int hh_w = row0 / Nq;
   const int wph = kWaves / h;          // waves per head
-  const bool alibi = a.rotary == BDH_ALIBI;
 
   for (int l = 0; l < a.L; ++l) {  // src/model/bdh.rs:336 -- the same weights in every layer
     // x = relu(cur . encoder - thr)
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
     // recurrent attention with value = cur (src/model/bdh.rs:353-359, 232-306): readout with the old rows,
     // then the rank-1 update (and the ALiBi decay); only visited rows are touched
     {
-      float *rho = a.rho + (size_t)l * a.rho_layer_stride + (size_t)b * cols * d;
+      float *rho = a.rho + (size_t)l * a.rho_layer_stride + (size_t)b * srows * d;
       int32_t *st = a.stamps ? a.stamps + (size_t)l * a.stamps_layer_stride + (size_t)b * cols : nullptr;
       const bool lazy = alibi && st != nullptr;
       const float dec = alibi ? a.decay[hh_w] : 1.0f;
@@ -201,6 +203,14 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
               const long k = pos - (long)st[r_l];
               if (k > 0) scale_l = expf((float)k * a.log_decay[hh_w]);
             }
+          } else if (pope) {  // PoPE (src/model/attention.rs:323-330): every row is visited
+            const int n = r_l - hh_w * Nq;
+            const int m = n < N ? n : n - N;
+            const float mag = logf(expf(s_x[hh_w * N + m] * 1.0f) + 1.0f) / 1.0f;  // softplus, beta = 1
+            const float raw = posf * a.freqs[m];
+            const float ph = (raw - floorf(raw)) * kTwoPi;
+            q_l = n < N ? mag * cosf(ph) : mag * sinf(ph);
+            touch_l = true;
           } else {  // RoPE (src/model/attention.rs:305-321)
             const int n = r_l - hh_w * N;
             const float xn = s_x[r_l], xo = s_x[r_l ^ 1];
@@ -356,11 +366,11 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
 bool bdh_model_small_fits(const bdh_model_config &c) {
   const long cols = (long)c.n_head * c.latent;
   const int h = c.n_head;
-  if (c.rotary != BDH_ROPE && c.rotary != BDH_ALIBI) return false;
+  if (c.rotary != BDH_ROPE && c.rotary != BDH_ALIBI && c.rotary != BDH_POPE) return false;
   if ((c.n_embd & 3) != 0) return false;  // a lane reads up to four adjacent columns of a state row at once
   if (c.n_embd < 1 || c.n_embd > kMaxD || c.vocab < 1 || c.vocab > kThreads || c.n_layer < 1) return false;
   if (h != 1 && h != 2 && h != 4 && h != 8 && h != 16) return false;
-  if (cols < 32 || cols > kMaxCols || (cols % (2 * kWaves)) != 0) return false;  // whole RoPE pairs per wave
+  if (cols < 32 || cols > kMaxCols || (cols % (2 * kWaves)) != 0) return false;  // whole RoPE pairs per wave; PoPE doubles the rows, not the columns
   return true;
 }
 
@@ -391,7 +401,7 @@ int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, float *rh
   a.L = c.n_layer;
   a.rotary = c.rotary;
   a.thr = c.relu_threshold;
-  a.rho_layer_stride = (size_t)B * c.n_head * c.latent * c.n_embd;
+  a.rho_layer_stride = (size_t)B * c.n_head * (c.rotary == BDH_POPE ? 2 : 1) * c.latent * c.n_embd;
   a.stamps_layer_stride = (size_t)B * c.n_head * c.latent;
   if (c.rotary == BDH_ALIBI)
     for (int i = 0; i < c.n_head; ++i) {

@@ -92,7 +92,7 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       matrix-core form from r sequences on whatever the size.
  *   "model.one_launch": 1 (default) a decode step (T = 1, f32 state, no x_tap / viz) of a small model
  *                       (d <= 256 and d % 4 == 0, h * N <= 2048 and a multiple of 32, h in {1,2,4,8,16},
- *                       V <= 1024, RoPE or ALiBi) runs as one launch, a workgroup per sequence, when the
+ *                       V <= 1024, any rotary mode) runs as one launch, a workgroup per sequence, when the
  *                       batch is large enough for that to pay (always for up to 4 MiB of projection weights per
  *                       step, from 16 sequences on for up to 8 MiB, from 128 on for more); 2 = whenever the
  *                       model fits; 0 = kernel

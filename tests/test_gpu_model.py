@@ -392,7 +392,7 @@ def test_decode_equals_prefill_on_device(bda):
     assert rel_err(sc.storage.cpu().numpy(), sa.storage.cpu().numpy()) < 1e-5 and sc.position == 6
 
 
-@pytest.mark.parametrize("rotary,lazy", [("rope", False), ("alibi", False), ("alibi", True)])
+@pytest.mark.parametrize("rotary,lazy", [("rope", False), ("pope", False), ("alibi", False), ("alibi", True)])
 @pytest.mark.parametrize("d,h,mult,L,V", [(64, 1, 4, 2, 40), (128, 4, 4, 3, 69), (256, 8, 8, 2, 256), (32, 16, 16, 2, 17)])
 def test_one_launch_decode_step(bda, corc, rotary, lazy, d, h, mult, L, V):
     """A small model's decode step (one token per sequence, no by-products) runs as ONE launch, a workgroup per
@@ -408,8 +408,7 @@ def test_one_launch_decode_step(bda, corc, rotary, lazy, d, h, mult, L, V):
     B, T0, steps = 3, 5, 4
     rng = np.random.default_rng(7 * d + h)
     prompt = rng.integers(0, V, (B, T0))
-    N = one.latent
-    rho_ref = np.zeros((L, B, h, N, d), np.float32)
+    rho_ref = np.zeros((L, B, h, one.latent_q, d), np.float32)
     logits_ref, pos, _, _ = corc.forward_with_state(shape, w, prompt, rho_ref, 0, sparse_state=False)
     s_one, s_ref = one.init_state(), ref.init_state()
     ctx = bda.ffi.default_context(0)
