@@ -132,6 +132,11 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     ctx->opt_model_one_launch = value;
     return BDH_OK;
   }
+  if (strcmp(name, "model.phase_batch") == 0) {
+    if (value < 0) return bdh_fail(ctx, BDH_E_INVAL, "model.phase_batch takes a batch size >= 0");
+    ctx->opt_model_phase_batch = value;
+    return BDH_OK;
+  }
   if (strcmp(name, "relu_lowrank.row") == 0) {
     if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "relu_lowrank.row takes 0 or 1");
     ctx->opt_lowrank_row = value;

@@ -23,6 +23,7 @@ struct bdh_ctx {
   int opt_decoder_mfma = 1;  // 0: the encoder E never takes the f32 matrix-core form
   int opt_model_one_launch = 1;  // small model's decode step in one launch: 1 when it pays, 2 whenever it fits, 0 never
   int opt_lowrank_row = 1;     // 0: relu_lowrank with one input row and a small matrix uses the column-per-thread kernel
+  int opt_model_phase_batch = 1 << 30;  // two launches per layer for a decode step of at most this many sequences (0: never)
   int opt_lowrank_scalar = 1;  // 0: relu_lowrank with 8 to 63 rows stages its inputs in LDS instead of scalar loads
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on
@@ -42,6 +43,14 @@ struct bdh_model {
 };
 
 int bdh_fail(bdh_ctx *ctx, int status, const char *fmt, ...);
+
+// model_phase.hip: a decode step in two launches per layer (T = 1, f32 state, 128 <= d <= 512, N a multiple of 64)
+bool bdh_model_phase_fits(const bdh_model_config &c);
+size_t bdh_model_phase_scratch_floats(const bdh_model_config &c, int B);
+int bdh_launch_model_phases(bdh_model *m, int B, float *scratch, float *rho, int32_t *stamps, int64_t position,
+                            const int32_t *positions_dev, float **cur_final, float **dec_partial, int *G_out);
+// projections.hip: cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))
+int bdh_launch_decoder_finalize(bdh_ctx *ctx, const float *partial, int KBN, int M, int d, float *cur);
 
 // model_small.hip: the one-launch decode step of a small model (T = 1, f32 state)
 bool bdh_model_small_fits(const bdh_model_config &c);

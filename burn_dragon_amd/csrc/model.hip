@@ -132,16 +132,42 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
   const size_t Nq = c.rotary == BDH_POPE ? 2 * (size_t)N : (size_t)N;
   const size_t M = (size_t)B * T;
 
-  // a decode step of a small model with no by-products: the whole step in one launch, a workgroup per sequence
-  // (one CU streams all the weights of a step, W bytes: measured on the reference's tiny / small / base sizes, W = 3,
-  // 6.75 and 12 MiB, the launch wins always, from 8 to 64 and from 64 to 256 sequences on, depending on how sparse
-  // the state step is)
-  if (T == 1 && !x_tap && !viz && rho_dtype == BDH_F32 && ctx->opt_model_one_launch != 0 && bdh_model_small_fits(c)) {
-    const size_t w_bytes = sizeof(float) * (size_t)3 * h * N * d * L;
-    const int b_min = w_bytes <= (size_t(4) << 20) ? 1 : (w_bytes <= (size_t(8) << 20) ? 16 : 128);
-    if (ctx->opt_model_one_launch == 2 || B >= b_min)
+  // A decode step (one token per sequence, f32 state, no by-products) need not run kernel by kernel:
+  //  * a small model (d <= 256, h*N <= 2048) can run the whole step in ONE launch, a workgroup per sequence; one CU then
+  //    streams all the projection weights of the step, W bytes;
+  //  * a mid-size model (128 <= d <= 512, up to 64 blocks of 64 neurons) can run TWO launches per layer, a workgroup
+  //    per block; every workgroup streams its share of the layer's weights once per sequence.
+  // Measured at the sizes of the reference's configurations (W = 3 / 6.75 / 12 / 96 MiB; us per step, one launch | two
+  // per layer | kernel by kernel): tiny 77|77|112 at B=1, 84|100|145 at B=64; small 152|82|130 at B=1, 168|127|195 at
+  // B=64, 323|442|478 at B=256; base 223|83|123 at B=1, 273|210|240 at B=64, 559|-|654 at B=256; large -|210|308 at
+  // B=1, -|519|554 at B=16, -|1092|981 at B=33.
+  if (T == 1 && !x_tap && !viz && rho_dtype == BDH_F32 && ctx->opt_model_one_launch != 0) {
+    const size_t w_layer = sizeof(float) * (size_t)3 * h * N * d;
+    const size_t w_bytes = w_layer * L;
+    const bool small_fits = bdh_model_small_fits(c);
+    const bool forced = ctx->opt_model_one_launch == 2;
+    const bool one_first = small_fits && (forced || w_bytes <= (size_t(4) << 20));
+    const bool phases = !one_first && bdh_model_phase_fits(c) && B <= ctx->opt_model_phase_batch &&
+                        (size_t)B * w_layer <= (size_t(256) << 20);
+    const int b_min = w_bytes <= (size_t(8) << 20) ? 16 : 128;
+    if (one_first || (!phases && small_fits && B >= b_min))
       return bdh_launch_model_small(m, tokens, B, static_cast<float *>(rho), stamps, position, positions_dev, logits,
                                     next_tokens);
+    if (phases) {
+      int rc2 = ensure_act(m, sizeof(float) * bdh_model_phase_scratch_floats(c, B));
+      if (rc2 != BDH_OK) return rc2;
+      float *scratch = static_cast<float *>(m->act);
+      rc2 = bdh_launch_embed_ln(ctx, tokens, (int64_t)B, d, V, m->w.embed, scratch);  // :319-322
+      if (rc2 != BDH_OK) return rc2;
+      float *cur_final = nullptr, *dpart = nullptr;
+      int G = 0;
+      rc2 = bdh_launch_model_phases(m, B, scratch, static_cast<float *>(rho), stamps, position, positions_dev, &cur_final,
+                                    &dpart, &G);
+      if (rc2 != BDH_OK) return rc2;
+      rc2 = bdh_launch_decoder_finalize(ctx, dpart, G, B, d, cur_final);  // the last layer's second stage (:436-441)
+      if (rc2 != BDH_OK) return rc2;
+      return bdh_launch_lm_head(ctx, B, 1, d, V, cur_final, m->w.lm_head, logits, next_tokens);  // :446-449
+    }
   }
 
   // activation scratch: cur [M,d] | x [B,h,T,N] | xy [B,h,T,N] | attn [B,h,T,d] | attn_ln [B,h,T,d] | last [h,d]

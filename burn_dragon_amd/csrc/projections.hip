@@ -939,6 +939,13 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   return BDH_OK;
 }
 
+int bdh_launch_decoder_finalize(bdh_ctx *ctx, const float *partial, int KBN, int M, int d, float *cur) {
+  if (d > 1024 || (d & 3) != 0) return bdh_fail(ctx, BDH_E_SHAPE, "encoder second stage needs d %% 4 == 0 and d <= 1024");
+  hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur);
+  BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
+  return BDH_OK;
+}
+
 int bdh_launch_lm_head(bdh_ctx *ctx, int B, int T, int d, int V, const float *cur, const float *lm_head,
                        float *logits, int64_t *next_tokens) {
   const int M = B * T;

@@ -90,13 +90,17 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       once) when its tiles cover half the chip; fewer sequences, and small models, take
  *                       the VALU kernel that skips inactive rows of E.  A negative value -r takes the
  *                       matrix-core form from r sequences on whatever the size.
- *   "model.one_launch": 1 (default) a decode step (T = 1, f32 state, no x_tap / viz) of a small model
- *                       (d <= 256 and d % 4 == 0, h * N <= 2048 and a multiple of 32, h in {1,2,4,8,16},
- *                       V <= 1024, any rotary mode) runs as one launch, a workgroup per sequence, when the
- *                       batch is large enough for that to pay (always for up to 4 MiB of projection weights per
- *                       step, from 16 sequences on for up to 8 MiB, from 128 on for more); 2 = whenever the
- *                       model fits; 0 = kernel
- *                       by kernel like any other call (values agree to 1e-5: other summation trees).
+ *   "model.one_launch": 1 (default) a decode step (T = 1, f32 state, no x_tap / viz) of a model that is
+ *                       small enough does not run kernel by kernel: a small model (d <= 256 and d % 4 == 0,
+ *                       h * N <= 2048 and a multiple of 32, h in {1,2,4,8,16}, V <= 1024) can take ONE launch
+ *                       for the whole step, a workgroup per sequence (always for up to 4 MiB of projection
+ *                       weights per step, else only for large batches); a mid-size model (128 <= d <= 512,
+ *                       N a multiple of 64, at most 64 blocks of 64 neurons) takes TWO launches per layer, a
+ *                       workgroup per block, while batch x weights of a layer stay under 256 MiB.
+ *                       2 = the one-launch step whenever the model fits it; 0 = kernel by kernel like any
+ *                       other call (values agree to 1e-5: other summation trees).
+ *   "model.phase_batch": the two-launch layer only for at most this many sequences (default: no limit
+ *                       beyond the one above; 0 = never).
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
  *                       1 = the two products on the f32 matrix cores (T >= 128 by default). */
 int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);

@@ -441,6 +441,56 @@ def test_one_launch_decode_step(bda, corc, rotary, lazy, d, h, mult, L, V):
         assert torch.equal(s_one.stamps, s_ref.stamps)
 
 
+@pytest.mark.parametrize("rotary,lazy", [("rope", False), ("pope", False), ("alibi", False), ("alibi", True)])
+@pytest.mark.parametrize("d,h,mult,L,V", [(128, 4, 32, 2, 40), (192, 3, 4, 3, 69), (256, 4, 16, 2, 256), (512, 8, 4, 2, 17)])
+def test_two_launch_layer_decode_step(bda, corc, rotary, lazy, d, h, mult, L, V):
+    """A decode step of a mid-size model at a small batch runs two launches per layer (a workgroup per 64 neurons of a
+    head of a sequence).  Logits, state and greedy tokens against the C oracle (1e-3) and against the same steps run
+    kernel by kernel (1e-5: only the summation trees differ), after a prompt that went through the many-token path."""
+    cfg = bda.BDHConfig(n_layer=L, n_embd=d, n_head=h, mlp_internal_dim_multiplier=mult, vocab_size=V, dropout=0.0)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse(rotary))
+    shape = _shape_from_cfg(cfg)
+    w = orc.init_weights(shape, seed=d + h)
+    weights = {"embed": w.embed, "encoder": w.encoder, "encoder_v": w.encoder_v, "decoder": w.decoder, "lm_head": w.lm_head}
+    fused = bda.BDH(cfg, DEV, weights=weights, alibi_lazy=lazy)
+    ref = bda.BDH(cfg, DEV, weights=weights, alibi_lazy=lazy)
+    assert fused.latent % 64 == 0
+    B, T0, steps = 3, 5, 4
+    rng = np.random.default_rng(7 * d + h)
+    prompt = rng.integers(0, V, (B, T0))
+    rho_ref = np.zeros((L, B, h, fused.latent_q, d), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, prompt, rho_ref, 0, sparse_state=False)
+    s_fused, s_ref = fused.init_state(), ref.init_state()
+    ctx = bda.ffi.default_context(0)
+    fused.forward_with_state(torch.from_numpy(prompt), s_fused)
+    ref.forward_with_state(torch.from_numpy(prompt), s_ref)
+    feed = logits_ref[:, -1].argmax(-1)
+    for step in range(steps):
+        tok = feed.reshape(B, 1)
+        logits_ref, pos, _, _ = corc.forward_with_state(shape, w, tok, rho_ref, pos, sparse_state=False)
+        got, nxt = fused.forward_with_state(torch.from_numpy(tok), s_fused, want_next=True)  # B <= 8: two launches per layer
+        try:
+            ctx.set_option("model.one_launch", 0)
+            kbk = ref.forward_with_state(torch.from_numpy(tok), s_ref)
+        finally:
+            ctx.set_option("model.one_launch", 1)
+        torch.cuda.synchronize()
+        got_np = got.cpu().numpy()
+        assert rel_err(got_np, logits_ref) < 1e-3, f"step {step} against the oracle"
+        assert rel_err(got_np, kbk.cpu().numpy()) < 1e-5, f"step {step} against the kernel-by-kernel step"
+        assert not np.array_equal(got_np, kbk.cpu().numpy()), "the two-launch layer was not taken"
+        assert np.array_equal(nxt.cpu().numpy(), got_np[:, 0].argmax(-1))
+        feed = logits_ref[:, -1].argmax(-1)
+    assert s_fused.position == T0 + steps == pos
+    fused.materialize_state(s_fused)
+    ref.materialize_state(s_ref)
+    torch.cuda.synchronize()
+    assert rel_err(s_fused.storage.cpu().numpy(), rho_ref) < 1e-3
+    assert rel_err(s_fused.storage.cpu().numpy(), s_ref.storage.cpu().numpy()) < 1e-5
+    if lazy:
+        assert torch.equal(s_fused.stamps, s_ref.stamps)
+
+
 def test_bad_token_poisons_only_its_row(bda):
     cfg = bda.BDHConfig(n_layer=1, n_embd=16, n_head=2, mlp_internal_dim_multiplier=4, vocab_size=32)
     cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
