@@ -511,10 +511,12 @@ def test_model_create_rejects_bad_configs(bda):
     assert err.value.status == ffi.E_SHAPE
 
 
-def test_decode_graph_replays_match_eager_steps(bda):
+@pytest.mark.parametrize("d,mult", [(256, 16), (256, 128), (128, 4)], ids=["two-launch-layer", "kernel-by-kernel", "one-launch"])
+def test_decode_graph_replays_match_eager_steps(bda, d, mult):
     """A captured decode step is replayed several times, with eager work and synchronisations of the
-    same program between the replays, and every replay is checked against the eager path."""
-    cfg = bda.BDHConfig(n_layer=3, n_embd=256, n_head=4, mlp_internal_dim_multiplier=16, vocab_size=64)
+    same program between the replays, and every replay is checked against the eager path -- for each of
+    the three forms a decode step can take."""
+    cfg = bda.BDHConfig(n_layer=3, n_embd=d, n_head=4, mlp_internal_dim_multiplier=mult, vocab_size=64)
     cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
     model = bda.BDH(cfg, DEV, seed=21)
     prompt = torch.randint(0, 64, (2, 5), generator=torch.Generator().manual_seed(2))
