@@ -17,7 +17,6 @@ namespace {
 
 constexpr float kLnEps = 1e-5f;                    // src/model/bdh.rs:17
 constexpr float kTwoPi = 6.28318530717958647692f;  // f32(2*PI), src/model/attention.rs:343
-constexpr int kFlight = 8;                         // state rows in flight per wave
 
 struct PhaseArgs {
   const float *cur_in;        // [B][d] the layer's input (before the pending encoder second stage, if any)
@@ -98,6 +97,7 @@ __device__ __forceinline__ float chain_spans(const float *s_in, const float *wv,
 template <int NW>
 __global__ __launch_bounds__(NW * 64) void k_layer_phase_a(PhaseArgs a) {
   constexpr int VPL = (NW + 3) / 4;  // float4 per lane per state row: columns (j*64 + lane)*4
+  constexpr int kFlight = 64 / NW < 16 ? 64 / NW : 16;  // state rows in flight per wave: all of its share of a dense block
   __shared__ __align__(16) float s_cur[NW * 64];
   __shared__ float s_x[64];
   __shared__ float s_acc[64];
