@@ -47,8 +47,11 @@ int bdh_fail(bdh_ctx *ctx, int status, const char *fmt, ...);
 // model_phase.hip: a decode step in two launches per layer (T = 1, f32 state, 128 <= d <= 512, N a multiple of 64)
 bool bdh_model_phase_fits(const bdh_model_config &c);
 size_t bdh_model_phase_scratch_floats(const bdh_model_config &c, int B);
-int bdh_launch_model_phases(bdh_model *m, int B, float *scratch, float *rho, int32_t *stamps, int64_t position,
+int bdh_launch_model_phases(bdh_model *m, const int64_t *tokens, int B, float *scratch, float *rho, int32_t *stamps,
+                            int64_t position,
                             const int32_t *positions_dev, float **cur_final, float **dec_partial, int *G_out);
+int bdh_launch_phase_head(bdh_model *m, int B, const float *cur, const float *dec_partial, int G, float *logits,
+                          int64_t *next_tokens);
 // projections.hip: cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))
 int bdh_launch_decoder_finalize(bdh_ctx *ctx, const float *partial, int KBN, int M, int d, float *cur);
 

@@ -157,16 +157,16 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
       int rc2 = ensure_act(m, sizeof(float) * bdh_model_phase_scratch_floats(c, B));
       if (rc2 != BDH_OK) return rc2;
       float *scratch = static_cast<float *>(m->act);
-      rc2 = bdh_launch_embed_ln(ctx, tokens, (int64_t)B, d, V, m->w.embed, scratch);  // :319-322
-      if (rc2 != BDH_OK) return rc2;
       float *cur_final = nullptr, *dpart = nullptr;
       int G = 0;
-      rc2 = bdh_launch_model_phases(m, B, scratch, static_cast<float *>(rho), stamps, position, positions_dev, &cur_final,
-                                    &dpart, &G);
+      rc2 = bdh_launch_model_phases(m, tokens, B, scratch, static_cast<float *>(rho), stamps, position, positions_dev,
+                                    &cur_final, &dpart, &G);
       if (rc2 != BDH_OK) return rc2;
-      rc2 = bdh_launch_decoder_finalize(ctx, dpart, G, B, d, cur_final);  // the last layer's second stage (:436-441)
+      if (V <= 1024)  // the last layer's second stage (:436-441) and the head (:446-449) in one launch
+        return bdh_launch_phase_head(m, B, cur_final, dpart, G, logits, next_tokens);
+      rc2 = bdh_launch_decoder_finalize(ctx, dpart, G, B, d, cur_final);
       if (rc2 != BDH_OK) return rc2;
-      return bdh_launch_lm_head(ctx, B, 1, d, V, cur_final, m->w.lm_head, logits, next_tokens);  // :446-449
+      return bdh_launch_lm_head(ctx, B, 1, d, V, cur_final, m->w.lm_head, logits, next_tokens);
     }
   }
 

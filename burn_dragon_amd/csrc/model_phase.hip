@@ -19,8 +19,11 @@ constexpr float kLnEps = 1e-5f;                    // src/model/bdh.rs:17
 constexpr float kTwoPi = 6.28318530717958647692f;  // f32(2*PI), src/model/attention.rs:343
 
 struct PhaseArgs {
+  const int64_t *tokens;      // first layer only: [B] tokens, the layer's input is LN(embed[token]) (else null)
+  const float *embed;         // [V][d]
+  int V;
   const float *cur_in;        // [B][d] the layer's input (before the pending encoder second stage, if any)
-  float *cur_out;             // [B][d] written by the first workgroup of a sequence when a second stage is pending
+  float *cur_out;             // [B][d] written by the first workgroup of a sequence when it computed the input itself
   const float *dec_partial;   // [G][B][d] encoder partials of the previous layer, or null
   float *x;                   // [B][h*N]
   float *attn_partial;        // [B][h][N/64][d]
@@ -123,7 +126,18 @@ __global__ __launch_bounds__(NW * 64) void k_layer_phase_a(PhaseArgs a) {
   // (src/model/bdh.rs:383, 436-441: cur = LN(cur + LN(mixed . decoder)))
   {
     const bool has = tid < d;
-    float cur = has ? a.cur_in[(long)b * d + tid] : 0.0f;
+    float cur = 0.0f;
+    if (a.tokens) {  // embedding row and its LayerNorm (src/model/bdh.rs:319-322); a bad token poisons the row
+      const int64_t tok = a.tokens[b];
+      const bool bad = tok < 0 || tok >= a.V;
+      const float v = has ? (bad ? __int_as_float(0x7fc00000) : a.embed[(long)tok * d + tid]) : 0.0f;
+      float mean, den;
+      block_ln_stats<NW>(v, has, d, s_st, mean, den);
+      cur = has ? (v - mean) / den : 0.0f;
+      if (has && hh == 0 && nblk == 0) a.cur_out[(long)b * d + tid] = cur;
+    } else if (has) {
+      cur = a.cur_in[(long)b * d + tid];
+    }
     if (a.dec_partial) {
       const int G = h * nblk_n;
       float mlp = 0.0f;
@@ -351,6 +365,103 @@ __global__ __launch_bounds__(NW * 64) void k_layer_phase_b(PhaseArgs a) {
   }
 }
 
+// ---- head -----------------------------------------------------------------------------------------------------
+// The last layer's pending second stage, then the logits and the greedy token (src/model/bdh.rs:436-449): one
+// workgroup of 16 waves per sequence.  logits[v] = sum_k cur[k] * lm_head[k][v]: 1024 / pad64(V) groups split k,
+// each one fmaf chain over its span with 32 rows in flight; the groups are added in order; the lowest index wins ties.
+__global__ __launch_bounds__(1024) void k_phase_head(const float *__restrict__ cur_in, const float *__restrict__ dec_partial,
+                                                     int G, int B, int d, const float *__restrict__ lm_head, int V,
+                                                     float *__restrict__ logits, int64_t *__restrict__ next) {
+  __shared__ float s_cur[512];
+  __shared__ float s_st[32];
+  __shared__ float s_grp[1024];
+  __shared__ float s_best[16];
+  __shared__ int s_arg[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = blockIdx.x;
+  {
+    const bool has = tid < d;
+    float mlp = 0.0f;
+    if (has) {
+      int g = 0;
+      for (; g + 8 <= G; g += 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = dec_partial[((long)(g + u) * B + b) * d + tid];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) mlp += t[u];
+      }
+      for (; g < G; ++g) mlp += dec_partial[((long)g * B + b) * d + tid];
+    }
+    const float base = has ? cur_in[(long)b * d + tid] : 0.0f;
+    float mean, den;
+    block_ln_stats<16>(mlp, has, d, s_st, mean, den);
+    const float z = has ? base + (mlp - mean) / den : 0.0f;
+    block_ln_stats<16>(z, has, d, s_st, mean, den);
+    if (tid < 512) s_cur[tid] = has ? (z - mean) / den : 0.0f;
+  }
+  __syncthreads();
+  const int Vp = (V + 63) & ~63;
+  const int GK = 1024 / Vp;
+  const int g = tid / Vp, c = tid - g * Vp;
+  const int per = (d + GK - 1) / GK;
+  if (g < GK && c < V) {
+    const int k0 = min(d, g * per), k1 = min(d, k0 + per);
+    float acc = 0.0f;
+    int k = k0;
+    for (; k + 32 <= k1; k += 32) {
+      float wv[32];
+#pragma unroll
+      for (int u = 0; u < 32; ++u) wv[u] = lm_head[(long)(k + u) * V + c];
+#pragma unroll
+      for (int u = 0; u < 32; ++u) acc = __builtin_fmaf(s_cur[k + u], wv[u], acc);
+    }
+    for (; k + 8 <= k1; k += 8) {
+      float wv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) wv[u] = lm_head[(long)(k + u) * V + c];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc = __builtin_fmaf(s_cur[k + u], wv[u], acc);
+    }
+    for (; k < k1; ++k) acc = __builtin_fmaf(s_cur[k], lm_head[(long)k * V + c], acc);
+    s_grp[g * Vp + c] = acc;
+  }
+  __syncthreads();
+  float best = -INFINITY;
+  int arg = 0x7fffffff;
+  if (tid < V) {
+    float v = s_grp[tid];
+    for (int gg = 1; gg < GK; ++gg) v += s_grp[gg * Vp + tid];
+    logits[(long)b * V + tid] = v;
+    if (v > best) {
+      best = v;
+      arg = tid;
+    }
+  }
+  if (!next) return;  // uniform
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o);
+    const int oa = __shfl_xor(arg, o);
+    if (ob > best || (ob == best && oa < arg)) {
+      best = ob;
+      arg = oa;
+    }
+  }
+  if (lane == 0) {
+    s_best[wave] = best;
+    s_arg[wave] = arg;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; ++w)
+      if (s_best[w] > best || (s_best[w] == best && s_arg[w] < arg)) {
+        best = s_best[w];
+        arg = s_arg[w];
+      }
+    next[b] = arg == 0x7fffffff ? 0 : arg;
+  }
+}
+
 }  // namespace
 
 bool bdh_model_phase_fits(const bdh_model_config &c) {
@@ -370,9 +481,10 @@ size_t bdh_model_phase_scratch_floats(const bdh_model_config &c, int B) {
          bdh_align_up(G * (size_t)B * d, 64);
 }
 
-// cur0 holds LN(embed[token]) on entry; on return cur_final points at the buffer holding the last layer's input
-// and dec_partial at its encoder partials [G][B][d]: the caller runs the encoder's second stage and the head.
-int bdh_launch_model_phases(bdh_model *m, int B, float *scratch, float *rho, int32_t *stamps, int64_t position,
+// On return cur_final points at the buffer holding the last layer's input and dec_partial at its encoder partials
+// [G][B][d]: the caller runs the encoder's second stage and the head.
+int bdh_launch_model_phases(bdh_model *m, const int64_t *tokens, int B, float *scratch, float *rho, int32_t *stamps,
+                            int64_t position,
                             const int32_t *positions_dev, float **cur_final, float **dec_partial, int *G_out) {
   bdh_ctx *ctx = m->ctx;
   const bdh_model_config &c = m->cfg;
@@ -409,9 +521,12 @@ int bdh_launch_model_phases(bdh_model *m, int B, float *scratch, float *rho, int
     }
   const int nw = (d + 63) / 64;
   int in = 0;  // cur[in] is the layer's input; a layer with a pending second stage writes cur[in ^ 1]
+  a.embed = m->w.embed;
+  a.V = c.vocab;
   for (int l = 0; l < L; ++l) {
+    a.tokens = l == 0 ? tokens : nullptr;  // the first layer makes its own input and leaves it in cur[0]
     a.cur_in = cur[in];
-    a.cur_out = cur[in ^ 1];
+    a.cur_out = l == 0 ? cur[0] : cur[in ^ 1];
     a.dec_partial = l > 0 ? dpart : nullptr;
     a.rho = rho + (size_t)l * B * h * Nq * d;
     a.stamps = stamps ? stamps + (size_t)l * B * h * N : nullptr;
@@ -426,5 +541,17 @@ int bdh_launch_model_phases(bdh_model *m, int B, float *scratch, float *rho, int
   *cur_final = cur[in];
   *dec_partial = dpart;
   *G_out = (int)G;
+  return BDH_OK;
+}
+
+// The last layer's second stage and the output head in one launch (V <= 1024).
+int bdh_launch_phase_head(bdh_model *m, int B, const float *cur, const float *dec_partial, int G, float *logits,
+                          int64_t *next_tokens) {
+  bdh_ctx *ctx = m->ctx;
+  const bdh_model_config &c = m->cfg;
+  if (c.vocab > 1024 || c.n_embd > 512) return bdh_fail(ctx, BDH_E_SHAPE, "head kernel needs V <= 1024 and d <= 512");
+  hipLaunchKernelGGL(k_phase_head, dim3((unsigned)B), dim3(1024), 0, ctx->stream, cur, dec_partial, G, B, c.n_embd,
+                     m->w.lm_head, c.vocab, logits, next_tokens);
+  BDH_LAUNCH_CHECK(ctx, "k_phase_head");
   return BDH_OK;
 }
