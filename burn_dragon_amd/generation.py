@@ -96,12 +96,20 @@ def prefill_state(model: BDH, prompt_tokens) -> Tuple[ModelState, torch.Tensor]:
     return state, logits[0, -1]
 
 
+def uniform_variate(device, generator: Optional[torch.Generator] = None) -> torch.Tensor:
+    """One uniform variate in [0, 1) as a [1] tensor on `device`, drawn on the generator's own device (a CPU
+    generator serves a GPU model)."""
+    if generator is not None and generator.device.type != torch.device(device).type:
+        return torch.rand((1,), device=generator.device, generator=generator).to(device)
+    return torch.rand((1,), device=device, generator=generator)
+
+
 def sample_next_token(model: BDH, state: ModelState, last_logits: torch.Tensor, temperature: float,
                       top_k: Optional[int], generator: Optional[torch.Generator] = None
                       ) -> Tuple[torch.Tensor, torch.Tensor]:
     """src/generation.rs:107-128: draws from last_logits [V], feeds the token and returns
     (token [1] int64 on the device, logits of the new token [V])."""
-    u = torch.rand((1,), device=last_logits.device, generator=generator)
+    u = uniform_variate(last_logits.device, generator)
     nxt = sample_from_logits(model, last_logits.reshape(1, -1), temperature, top_k, u)
     logits = model.forward_with_state(nxt.reshape(1, 1), state)
     return nxt, logits[0, -1]

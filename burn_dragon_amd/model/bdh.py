@@ -183,9 +183,9 @@ class BDH:
         out = [indices]
         for _ in range(max_new_tokens):
             if not greedy:
-                from ..generation import sample_from_logits
+                from ..generation import sample_from_logits, uniform_variate
 
-                u = torch.rand((1,), device=self.device, generator=generator)
+                u = uniform_variate(self.device, generator)
                 nxt = sample_from_logits(self, logits[:, -1], temperature, top_k, u)
             tok = nxt.reshape(1, 1)
             out.append(tok)
