@@ -96,20 +96,39 @@ def prefill_state(model: BDH, prompt_tokens) -> Tuple[ModelState, torch.Tensor]:
     return state, logits[0, -1]
 
 
-def uniform_variate(device, generator: Optional[torch.Generator] = None) -> torch.Tensor:
-    """One uniform variate in [0, 1) as a [1] tensor on `device`, drawn on the generator's own device (a CPU
+def uniform_variates(n: int, device, generator: Optional[torch.Generator] = None) -> torch.Tensor:
+    """n uniform variates in [0, 1) as an [n] tensor on `device`, drawn on the generator's own device (a CPU
     generator serves a GPU model)."""
     if generator is not None and generator.device.type != torch.device(device).type:
-        return torch.rand((1,), device=generator.device, generator=generator).to(device)
-    return torch.rand((1,), device=device, generator=generator)
+        return torch.rand((n,), device=generator.device, generator=generator).to(device)
+    return torch.rand((n,), device=device, generator=generator)
+
+
+class VariateStream:
+    """The uniform variates of one generation run, drawn from `generator` a block at a time so that no host work
+    is done per token.  Every consumer draws blocks of the same size: two runs from equal seeds see the same
+    sequence whichever entry point they go through."""
+
+    BLOCK = 256
+
+    def __init__(self, device, generator: Optional[torch.Generator] = None):
+        self.device, self.generator = device, generator
+        self._buf, self._at = None, 0
+
+    def next(self) -> torch.Tensor:
+        if self._buf is None or self._at == self.BLOCK:
+            self._buf, self._at = uniform_variates(self.BLOCK, self.device, self.generator), 0
+        self._at += 1
+        return self._buf[self._at - 1:self._at]
 
 
 def sample_next_token(model: BDH, state: ModelState, last_logits: torch.Tensor, temperature: float,
-                      top_k: Optional[int], generator: Optional[torch.Generator] = None
-                      ) -> Tuple[torch.Tensor, torch.Tensor]:
+                      top_k: Optional[int], generator: Optional[torch.Generator] = None,
+                      variates: Optional[VariateStream] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """src/generation.rs:107-128: draws from last_logits [V], feeds the token and returns
-    (token [1] int64 on the device, logits of the new token [V])."""
-    u = uniform_variate(last_logits.device, generator)
+    (token [1] int64 on the device, logits of the new token [V]).  The variate comes from `variates` when a
+    run keeps a stream, else from a draw of its own."""
+    u = variates.next() if variates is not None else uniform_variates(1, last_logits.device, generator)
     nxt = sample_from_logits(model, last_logits.reshape(1, -1), temperature, top_k, u)
     logits = model.forward_with_state(nxt.reshape(1, 1), state)
     return nxt, logits[0, -1]
@@ -129,10 +148,11 @@ def generate_tokens(model: BDH, prompt_tokens: List[int], settings: GenerationSe
         state.trim(window)
     produced: List[torch.Tensor] = []
     generated = 0
+    variates = VariateStream(last_logits.device, generator)
     try:
         while settings.max_new_tokens is None or generated < settings.max_new_tokens:
             nxt, last_logits = sample_next_token(model, state, last_logits, settings.temperature, settings.top_k,
-                                                 generator)
+                                                 generator, variates)
             generated += 1
             if on_token is not None:
                 tok = int(nxt[0])

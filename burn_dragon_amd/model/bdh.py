@@ -181,12 +181,13 @@ class BDH:
         greedy = top_k == 1
         logits, nxt = self.forward_with_state(indices, state, want_next=True)
         out = [indices]
+        if not greedy:  # the variates come a block at a time: no host work per token
+            from ..generation import VariateStream, sample_from_logits
+
+            variates = VariateStream(self.device, generator)
         for _ in range(max_new_tokens):
             if not greedy:
-                from ..generation import sample_from_logits, uniform_variate
-
-                u = uniform_variate(self.device, generator)
-                nxt = sample_from_logits(self, logits[:, -1], temperature, top_k, u)
+                nxt = sample_from_logits(self, logits[:, -1], temperature, top_k, variates.next())
             tok = nxt.reshape(1, 1)
             out.append(tok)
             logits, nxt = self.forward_with_state(tok, state, want_next=True)
