@@ -291,7 +291,43 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
     const bool a_vec = (g.lda % 4 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0);
     const bool b_vec = (g.ldb % 4 == 0) && (reinterpret_cast<uintptr_t>(Bm) % 16 == 0);
     float4 ra[1][CA], rb[1][CB];
+    // a tile that lies inside both operands, 16-byte aligned: its loads need no checks, and loads that sit
+    // under no branch are issued back to back
+    const bool tile_full = a_vec && b_vec && m0 + BM <= g.M && n0 + BN <= g.N;
     auto load = [&](float4 *pa, float4 *pb, int k0) {
+      if (tile_full && k0 + FK <= K) {
+#pragma unroll
+        for (int c = 0; c < CA; ++c) {
+          const int chunk = c * NT + tid;
+          if (!A_KMAJOR) {
+            const int row = chunk >> 2, kc = (chunk & 3) * 4;
+            pa[c] = *reinterpret_cast<const float4 *>(A + (long)(m0 + row) * g.lda + k0 + kc);
+          } else {
+            const int kr = chunk / (BM / 4), mc = (chunk % (BM / 4)) * 4;
+            pa[c] = *reinterpret_cast<const float4 *>(A + (long)(k0 + kr) * g.lda + m0 + mc);
+          }
+        }
+#pragma unroll
+        for (int c = 0; c < CB; ++c) {
+          const int chunk = c * NT + tid;
+          if (!B_KMAJOR) {
+            const int row = chunk >> 2, kc = (chunk & 3) * 4;
+            pb[c] = *reinterpret_cast<const float4 *>(Bm + (long)(n0 + row) * g.ldb + k0 + kc);
+          } else {
+            const int kr = chunk / (BN / 4), nc = (chunk % (BN / 4)) * 4;
+            pb[c] = *reinterpret_cast<const float4 *>(Bm + (long)(k0 + kr) * g.ldb + n0 + nc);
+          }
+        }
+        if (A_KMAJOR && EPI == 2 && (g.decay_mode & FSA_DECAY_STATE)) {
+#pragma unroll
+          for (int c = 0; c < CA; ++c) {
+            const int kr = (c * NT + tid) / (BM / 4);
+            const float f = expf((float)(K - (k0 + kr)) * ld);
+            pa[c].x *= f; pa[c].y *= f; pa[c].z *= f; pa[c].w *= f;
+          }
+        }
+        return;
+      }
 #pragma unroll
       for (int c = 0; c < CA; ++c) {
         const int chunk = c * NT + tid;
