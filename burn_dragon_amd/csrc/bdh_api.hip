@@ -72,6 +72,11 @@ int bdh_ctx_create(int device_id, void *hip_stream, bdh_ctx **out) {
     return BDH_E_HIP;
   }
   ctx->n_cu = prop.multiProcessorCount;
+  // the device is current: resolve this device's copy of the fixed scratch array of bdh_state_step_noalloc
+  if (bdh_step_scratch_resolve(ctx) != BDH_OK) {
+    delete ctx;
+    return BDH_E_HIP;
+  }
   *out = ctx;
   return BDH_OK;
 }
@@ -296,6 +301,27 @@ int bdh_state_step(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const f
   return bdh_recurrent_attention(ctx, B, h, 1, N, d, rotary, x, v, freqs, position, positions_dev,
                                  alibi_slopes_host, rho, rho_dtype, out, active_bitmask,
                                  rows_touched);
+}
+
+int bdh_state_step_noalloc(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const float *x,
+                           const float *v, const float *freqs, int64_t position,
+                           const int32_t *positions_dev, const float *alibi_slopes_host, void *rho,
+                           int rho_dtype, float *out, uint64_t *active_bitmask, int32_t *rows_touched) {
+  int rc = validate_state_args(ctx, B, h, 1, N, d, rotary, x, v, freqs, position, rho, rho_dtype, out);
+  if (rc != BDH_OK) return rc;
+  if (B == 0 || h == 0) return BDH_OK;
+  void *fixed = bdh_step_scratch_ptr(ctx);
+  if (!fixed) return bdh_fail(ctx, BDH_E_UNSUPPORTED, "no fixed scratch array was resolved for device %d", ctx->device);
+  float slopes[64];
+  if (rotary == BDH_ALIBI) {
+    if (alibi_slopes_host)
+      memcpy(slopes, alibi_slopes_host, sizeof(float) * h);
+    else
+      bdh_default_alibi_slopes(h, slopes);
+  }
+  StateStepParams p{B, h, 1, N, d, rotary, rho_dtype, x, v, freqs, position, positions_dev,
+                    rotary == BDH_ALIBI ? slopes : nullptr, rho, out, active_bitmask, rows_touched};
+  return bdh_launch_state_steps_in(ctx, p, nullptr, fixed, bdh_step_scratch_bytes());
 }
 
 int bdh_relu_lowrank(bdh_ctx *ctx, int B, int h_in, int T, int d, int h, int N, const float *in,

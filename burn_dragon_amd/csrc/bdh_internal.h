@@ -102,6 +102,13 @@ int bdh_launch_state_steps(bdh_ctx *ctx, const StateStepParams &p);
 // Variant used inside the fused model step: the readout is LayerNorm-ed on the fly
 // (src/model/bdh.rs:359) when out_ln != nullptr.
 int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
+// The same with the partials in a caller-given buffer (nothing is allocated; fails when they do not fit).
+int bdh_launch_state_steps_in(bdh_ctx *ctx, const StateStepParams &p, float *out_ln, void *fixed, size_t fixed_bytes);
+// The fixed scratch array of the allocation-free decode step: resolve its address on the context's device
+// (that device must be current), read it back, and its size.
+int bdh_step_scratch_resolve(bdh_ctx *ctx);
+void *bdh_step_scratch_ptr(const bdh_ctx *ctx);
+size_t bdh_step_scratch_bytes();
 // The same T steps as four dense products per chunk on the f32 matrix cores (attention_parallel.hip):
 // RoPE / PoPE, f32 state, no bitmask or row counts.
 int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);

@@ -17,6 +17,7 @@
 #include <hip/hip_bf16.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include "bdh_internal.h"
 
@@ -985,7 +986,45 @@ void launch_fast(hipStream_t st, int blocks, const StepPtrs &a, float *rho) {
 
 }  // namespace
 
+// ------------------------------------------------------------------------------------
+// Scratch of the allocation-free decode step (bdh_state_step_noalloc): the readout partials
+// [slices, S, d] and the per-workgroup pair counts live in this array instead of the context's
+// growable workspace.  Every device the library runs on holds its own copy at its own address
+// until the process ends; the address is resolved once per device, with that device current,
+// and only that address (never the array's name) is handed to kernels.
+// ------------------------------------------------------------------------------------
+constexpr size_t kStepScratchBytes = (size_t(32) << 20) + (size_t(256) << 10);
+static __device__ __align__(256) unsigned char scratch[kStepScratchBytes];
+constexpr int kStepScratchDevices = 64;
+static void *g_step_scratch[kStepScratchDevices];
+static std::mutex g_step_scratch_mutex;
+
+size_t bdh_step_scratch_bytes() { return kStepScratchBytes; }
+
+int bdh_step_scratch_resolve(bdh_ctx *ctx) {
+  if (ctx->device < 0 || ctx->device >= kStepScratchDevices) return BDH_OK;  // such a device has no allocation-free step
+  std::lock_guard<std::mutex> lock(g_step_scratch_mutex);
+  if (g_step_scratch[ctx->device]) return BDH_OK;
+  void *ptr = nullptr;
+  BDH_HIP_CHECK(ctx, hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr) return bdh_fail(ctx, BDH_E_HIP, "hipGetSymbolAddress gave a null scratch address");
+  g_step_scratch[ctx->device] = ptr;
+  return BDH_OK;
+}
+
+void *bdh_step_scratch_ptr(const bdh_ctx *ctx) {
+  if (ctx->device < 0 || ctx->device >= kStepScratchDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_step_scratch_mutex);
+  return g_step_scratch[ctx->device];
+}
+
 int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out_ln) {
+  return bdh_launch_state_steps_in(ctx, p, out_ln, nullptr, 0);
+}
+
+// fixed != nullptr: partials and counts go to that buffer of fixed_bytes instead of the context's workspace,
+// and nothing is allocated (the call fails when they do not fit)
+int bdh_launch_state_steps_in(bdh_ctx *ctx, const StateStepParams &p, float *out_ln, void *fixed, size_t fixed_bytes) {
   const int B = p.B, h = p.h, T = p.T, N = p.N, d = p.d;
   const int Nq = p.rotary == BDH_POPE ? 2 * N : N;
   const int slices = B * h;
@@ -1042,7 +1081,8 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
                            sizeof(float) * (size_t)slices * Nq * d <= (size_t(64) << 20);
   const bool dense_auto = (T >= 128 && (!loop_is_cheap || state_tiles >= n_cu / 2)) ||
                           (T >= 8 && (streamed || small_state));
-  if (!p.bitmask && !p.rows_touched && chunk_fits && (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : dense_auto))
+  if (!fixed && !p.bitmask && !p.rows_touched && chunk_fits &&
+      (ctx->opt_step_dense >= 0 ? ctx->opt_step_dense == 1 : dense_auto))
     return bdh_launch_state_chunks_f32(ctx, p, out_ln);
   // tokens per launch: the f32 RoPE kernel, the generic and the dense streaming kernel walk several, as many as
   // 64 MiB of partials allow
@@ -1053,12 +1093,21 @@ int bdh_launch_state_steps_ln(bdh_ctx *ctx, const StateStepParams &p, float *out
   int group = 1;
   if (T > 1 && ((fast && p.rho_dtype == BDH_F32) || (generic && !p.bitmask && !p.rows_touched)))
     group = (int)std::max<size_t>(1, std::min<size_t>((size_t)T, (size_t(64) << 20) / partial_one));
+  if (fixed) group = 1;
   const size_t partial_bytes = partial_one * group;
   const size_t cnt_bytes = cnt_one * group;
-  int rc = bdh_ws_reserve(ctx, partial_bytes + cnt_bytes);
-  if (rc != BDH_OK) return rc;
-  float *partial = static_cast<float *>(ctx->ws);
-  int *pair_cnt = reinterpret_cast<int *>(static_cast<char *>(ctx->ws) + partial_bytes);
+  if (fixed) {
+    if (partial_bytes + cnt_bytes > fixed_bytes)
+      return bdh_fail(ctx, BDH_E_SHAPE,
+                      "the allocation-free step needs %zu bytes of scratch for B*h=%d, N=%d, d=%d; the fixed array holds %zu",
+                      partial_bytes + cnt_bytes, slices, N, d, fixed_bytes);
+  } else {
+    int rc = bdh_ws_reserve(ctx, partial_bytes + cnt_bytes);
+    if (rc != BDH_OK) return rc;
+  }
+  char *ws = static_cast<char *>(fixed ? fixed : ctx->ws);
+  float *partial = reinterpret_cast<float *>(ws);
+  int *pair_cnt = reinterpret_cast<int *>(ws + partial_bytes);
 
   HeadScalars decay{}, log_decay{};
   const int has_decay = p.rotary == BDH_ALIBI;

@@ -165,6 +165,23 @@ int bdh_state_step(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const f
                    int rho_dtype, float *out, uint64_t *active_bitmask,
                    int32_t *rows_touched);
 
+/* bdh_state_step for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments,
+ * same kernels and bit-identical results, but the readout partials [B*h, S, d] and the per-workgroup
+ * row counts go to a fixed 32.25 MiB array in device memory that the library holds on every device it
+ * runs on (resolved at bdh_ctx_create) instead of the context's growable workspace, and the call makes
+ * no hipMalloc / hipFree.  A shape whose partials do not fit returns BDH_E_SHAPE and bdh_last_error
+ * names the bytes needed: about 4*B*h*S*(d+1) with S workgroups per (sequence, head) slice (S = N/512
+ * for RoPE at d in {256,512}, N/128 when that grid would leave CUs idle, N/64 for the other kernels).
+ * BASELINE configs 2 and 4 need 2 and 16 MiB.  All calls on one device share the array: calls that overlap on one device (two streams, two
+ * contexts) race; calls ordered on one stream do not.  Nothing in the array has to start at zero: every
+ * element that is read was written by the same call. */
+int bdh_state_step_noalloc(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const float *x,
+                           const float *v, const float *freqs, int64_t position,
+                           const int32_t *positions_dev, const float *alibi_slopes_host, void *rho,
+                           int rho_dtype, float *out, uint64_t *active_bitmask,
+                           int32_t *rows_touched);
+
 /* ---- a3 / a7: ReLU low-rank projection ------------------------------------------- */
 /*
  * Replaces kernel::relu_lowrank::fused_forward (src/kernel/relu_lowrank.rs:7-37) and the
