@@ -194,6 +194,63 @@ def bench_copy(args):
                                  "bytes_read_per_step": n * 4, "bytes_written_per_step": n * 4}}))
 
 
+def measure_rmw_ceiling(region_bytes=1 << 30, chunk_kib=2, density=0.0975, lists=16, iters=64, workgroups=8192,
+                        modes=(0,)):
+    """What the decode step's access pattern reaches with the arithmetic taken away (bdh_probe_chunks):
+    random chunk_kib-KiB chunks covering `density` of a region, read, scaled by 1 and written back in place,
+    a different ready-made chunk list on every launch.  At the defaults this is the traffic of the config-2
+    step (2 KiB = both rows of a lane pair, 9.75 % of 1 GiB = the pair-closed rows at 5 % active neurons).
+    Returns {mode: (microseconds per launch, GB/s over bytes read + bytes written)}."""
+    import torch
+
+    from burn_dragon_amd import ffi
+
+    dev = torch.device("cuda:0")
+    ctx = ffi.default_context(0)
+    region = torch.zeros(region_bytes // 4, device=dev)
+    n_region = region_bytes // (chunk_kib << 10)
+    g = torch.Generator(device=dev).manual_seed(11)
+    idx = [torch.nonzero(torch.rand(n_region, device=dev, generator=g) < density).flatten().to(torch.int32).contiguous()
+           for _ in range(lists)]
+    moved = float(np.mean([i.numel() for i in idx])) * (chunk_kib << 10)
+    out = {}
+    for mode in modes:
+        def launch(i):
+            ctx.check(ctx.lib.bdh_probe_chunks(ctx.handle, region.data_ptr(), region_bytes, idx[i % lists].data_ptr(),
+                                               idx[i % lists].numel(), chunk_kib, mode, workgroups))
+        for i in range(lists):
+            launch(i)
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(iters):
+            launch(i)
+        stop.record()
+        torch.cuda.synchronize()
+        us = start.elapsed_time(stop) / iters * 1e3
+        out[mode] = (us, (2.0 if mode == 0 else 1.0) * moved / (us * 1e-6) / 1e9)
+    return out, moved
+
+
+def bench_rmw_probe(args):
+    """The bandwidth ceiling of the decode step's access pattern, measured on this box."""
+    res, moved = measure_rmw_ceiling(modes=(0, 1, 2), iters=256 if args.steps == 1000 else args.steps)
+    us, gbs = res[0]
+    print(json.dumps({
+        "metric": "in-place read-modify-write bandwidth of random 2 KiB chunks (decode-step access pattern)",
+        "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": 256 if args.steps == 1000 else args.steps, "warmup": 16,
+        "ms_per_step": us * 1e-3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "bdh_probe_chunks: random 2 KiB chunks, 9.75 % of a 1 GiB region, ready-made chunk "
+                               "lists (16, rotating), 8192 workgroups of 4 waves, one wave per KiB",
+                   "bytes_read_per_launch": moved, "bytes_written_per_launch": moved,
+                   "read_only_us": res[1][0], "read_only_gbs": res[1][1],
+                   "write_only_us": res[2][0], "write_only_gbs": res[2][1]},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "kernel": "k_probe_chunks<0>", "launch_us": us},
+    }))
+
+
 F32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense f32 matrix, published
 
 
@@ -479,12 +536,13 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--prefill-chunk", type=int, default=0,
                     help="model workload: feed the prompt in calls of this many tokens (0 = one call)")
-    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy", "alibi", "parallel", "chunks"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy", "alibi", "parallel", "chunks", "rmw_probe"], default="decode",
                     help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA); "
                          "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4); "
                          "alibi = ALiBi state step, lazily decayed state beside the eager dense decay; "
                          "parallel = fused_state_aligned in f32 at the config-3 shape; chunks = many-token state step "
-                         "(f32 dense products) beside the token loop at the config-2 shape; copy = counter calibration")
+                         "(f32 dense products) beside the token loop at the config-2 shape; copy = counter calibration; "
+                         "rmw_probe = the bandwidth the decode step's access pattern reaches without its arithmetic")
     ap.add_argument("--model-config", choices=["c1", "c4", "ckpt", *SHIPPED_SIZES], default="c1",
                     help="model: config 1, config 4, the trained tiny_shakespeare checkpoint of the test fixtures, or one "
                          "of the sizes the reference ships configurations for (random-init, ALiBi)")
@@ -526,6 +584,8 @@ def main():
         return bench_parallel(args)
     if args.workload == "chunks":
         return bench_chunks(args)
+    if args.workload == "rmw_probe":
+        return bench_rmw_probe(args)
     B, h, N, d = args.batch, args.heads, args.latent, args.embd
     ctx = ffi.default_context(0)
     lib = ctx.lib
@@ -575,8 +635,12 @@ def main():
     ctx.check(rc_bad)
     gpu_ms = start.elapsed_time(stop)
     ms_per_step = max(gpu_ms, wall * 1e3) / args.steps  # the slower of the two clocks
-    kernel_us = gpu_ms / args.steps * 1e3
-    achieved = bytes_per_step / (kernel_us * 1e-6) / 1e9
+    event_us = gpu_ms / args.steps * 1e3
+    achieved = bytes_per_step / (ms_per_step * 1e-3) / 1e9  # on the same clock as ms_per_step and value
+    ceiling = None
+    if default_workload:  # the same pattern without the arithmetic, measured in this run
+        probe, _ = measure_rmw_ceiling(iters=64)
+        ceiling = probe[0][1]
 
     result = {
         "metric": "decode tokens/sec at batch B (single-layer state step) + achieved HBM GB/s",
@@ -605,10 +669,20 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain copy of
-            # known size (profiles/state_step_config2_f32_pmc_traffic.md); measured for the default workload only
+            # known size; measured for the default workload only, by the profile named in traffic_source
             "traffic": 216.06e6 if default_workload else None,
-            "kernel": f"k_step_rope_{args.rho_dtype} (+ k_step_finalize); duration = HIP-event time of the timed region / steps",
-            "launch_us": kernel_us,
+            "traffic_source": "profiles/state_step_config2_f32_pmc_traffic.md" if default_workload else None,
+            "kernel": f"k_step_rope_{args.rho_dtype} (+ k_step_finalize); achieved = algorithmic bytes / ms_per_step "
+                      "(both kernels of the step, the slower of the HIP-event and the host clock)",
+            "launch_us": ms_per_step * 1e3,
+            "event_us": event_us,
+            # the dominant kernel alone, from the committed rocprofv3 kernel trace of this command
+            "kernel_us": 42.3 if default_workload else None,
+            "kernel_us_source": "profiles/state_step_config2_f32_kernel_trace.md" if default_workload else None,
+            # bdh_probe_chunks in this run: in-place read-modify-write of random 2 KiB chunks (9.75 % of 1 GiB)
+            # from ready-made lists: what this access pattern reaches with no arithmetic at all
+            "ceiling_measured_gbs": ceiling,
+            "frac_of_measured_ceiling": (achieved / ceiling) if ceiling else None,
         },
     }
     if not args.no_cpu_baseline:

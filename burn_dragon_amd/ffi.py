@@ -27,7 +27,7 @@ EXPORTS = [
     "bdh_model_state_bytes", "bdh_model_forward", "bdh_model_forward_ex", "bdh_advance_positions",
     "bdh_sample_top_k", "bdh_recurrent_attention_lazy_alibi", "bdh_alibi_materialize", "bdh_model_forward_lazy",
     "bdh_rho_energy", "bdh_model_forward_viz", "bdh_rotate",
-    "bdh_model_forward_fast", "bdh_state_step_noalloc",
+    "bdh_model_forward_fast", "bdh_state_step_noalloc", "bdh_probe_chunks",
 ]
 
 
@@ -85,6 +85,7 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
                                             c_int, P, P, P]
     lib.bdh_state_step.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, P, P, P, c_int, P, P, P]
     lib.bdh_state_step_noalloc.argtypes = lib.bdh_state_step.argtypes
+    lib.bdh_probe_chunks.argtypes = [P, P, c_size_t, P, c_int, c_int, c_int, c_int]
     lib.bdh_relu_lowrank.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_float, c_int, P, c_int,
                                      P, P]
     lib.bdh_layer_norm.argtypes = [P, c_int64, c_int, P, P]

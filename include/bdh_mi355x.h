@@ -380,6 +380,15 @@ int bdh_model_forward_viz(bdh_model *model, const int64_t *tokens, int B, int T,
 int bdh_sample_top_k(bdh_ctx *ctx, int B, int V, const float *logits, int64_t row_stride,
                      float temperature, int top_k, const float *uniforms, int64_t *next_tokens);
 
+/* Measurement aid, no counterpart in the reference: the memory traffic of the decode state step without
+ * its arithmetic.  Reads, scales by 1 and writes back in place (mode 0), only reads (1) or only writes
+ * zeros (2) the listed chunks of `region`: chunk c covers bytes [chunk_index[c] * chunk_kib KiB, + chunk_kib
+ * KiB); one wavefront moves 1 KiB at a time, `workgroups` workgroups of 256 threads stride over the list.
+ * Listed chunks that do not lie inside region_bytes are skipped.  bench.py --workload rmw_probe times it on the
+ * config-2 pattern (random 2 KiB chunks, 9.75 % of 1 GiB) to report the bandwidth that pattern can reach. */
+int bdh_probe_chunks(bdh_ctx *ctx, void *region, size_t region_bytes, const int32_t *chunk_index, int n_chunks,
+                     int chunk_kib, int mode, int workgroups);
+
 #ifdef __cplusplus
 }
 #endif
