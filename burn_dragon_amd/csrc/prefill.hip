@@ -18,7 +18,9 @@
 // k-major (Q [T,N] with the reduction over T): that tile is also copied as is, [k][m], and the
 // fragments are read with the transposing LDS load of gfx950 (ds_read_b64_tr_b16); a 64-byte
 // column swizzle on every other group of eight k rows keeps the two half-waves on different banks.
+#include <algorithm>
 #include <atomic>
+#include <type_traits>
 
 #include "bdh_internal.h"
 
@@ -26,6 +28,8 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr float kTwoPi = 6.28318530717958647692f;
 constexpr int BM = 256, BN = 256, BK = 64;
@@ -45,13 +49,12 @@ __device__ __forceinline__ float bf16_bits_to_f32(unsigned short v) { return __u
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_rope_bf16(const uint4 *__restrict__ x, uint4 *__restrict__ q,
                                                    const float *__restrict__ freqs, int S, int T, int N,
-                                                   float pos0_f, long pos0) {
+                                                   long x_slice_groups, long pos0) {
   const int groups = N >> 3;  // 8 elements (4 pairs) per thread
   const long gid = (long)blockIdx.x * 256 + threadIdx.x;
   if (gid >= (long)T * groups) return;
   const int t = (int)(gid / groups), g = (int)(gid - (long)t * groups);
   const float pos = (float)(pos0 + t);
-  (void)pos0_f;
   float cs[8], sn[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
@@ -80,13 +83,12 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint4 *__restrict__ x, 
   for (; s + 8 <= S; s += 8) {
     uint4 in[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) in[u] = x[((long)(s + u) * T + t) * groups + g];
+    for (int u = 0; u < 8; ++u) in[u] = x[(long)(s + u) * x_slice_groups + (long)t * groups + g];
 #pragma unroll
     for (int u = 0; u < 8; ++u) q[((long)(s + u) * T + t) * groups + g] = rotate(in[u]);
   }
   for (; s < S; ++s) {
-    const long off = ((long)s * T + t) * groups + g;
-    q[off] = rotate(x[off]);
+    q[((long)s * T + t) * groups + g] = rotate(x[(long)s * x_slice_groups + (long)t * groups + g]);
   }
 }
 
@@ -96,11 +98,11 @@ __global__ __launch_bounds__(256) void k_rope_bf16(const uint4 *__restrict__ x, 
 // ------------------------------------------------------------------------------------
 template <typename TIn>
 __global__ __launch_bounds__(256) void k_transpose_to_bf16(const TIn *__restrict__ in, unsigned short *__restrict__ out,
-                                                          int R, int C, int ldo) {
+                                                          int R, int C, int ldo, long in_batch) {
   __shared__ unsigned short tile[64][66];
   const long batch = blockIdx.z;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  const TIn *src = in + batch * (long)R * C;
+  const TIn *src = in + batch * in_batch;
   unsigned short *dst = out + batch * (long)C * ldo;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   for (int rr = ty; rr < 64; rr += 4) {
@@ -425,6 +427,520 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
     }
 }
 
+// ====================================================================================
+// Chunk-recurrent form for aligned shapes (T a multiple of 256, N a multiple of 256, d = 256):
+//   per 256-token chunk c of a (b,h) slice, with rho_c the state before the chunk,
+//     out_c = tril(-1)(Q_c Q_c^T) V_c + Q_c rho_c        rho_{c+1} = rho_c + Q_c^T V_c
+// It executes 45 % of the matrix work of the all-scores form at T = 2048 (one 256x256 score tile and
+// one 256x256 state product per chunk instead of (T/256+1)/2 score tiles), and its workspace is linear
+// in T.  Two kernels:
+//   k_state_update  one workgroup per (slice, 256 neurons): walks all tokens, keeps its 256x256 tile of
+//                   rho in the accumulators (f32, started from the caller's state), rotates x on the way
+//                   in (RoPE; Q = bf16(rope(x)) is also written out for the second kernel) and, at every
+//                   chunk boundary, writes bf16(rho_c) transposed ([d][N], the k-contiguous B operand of
+//                   Q_c rho_c).
+//   k_chunk_out     one workgroup per (slice, chunk): S = Q_c Q_c^T on the matrix cores (operands straight
+//                   from global memory into LDS), mask + round to bf16 into LDS, out = S V_c, then
+//                   out += Q_c bf16(rho_c) with the same accumulators, written once.
+// ====================================================================================
+
+// The k loop of k_gemm_direct as a function: acc += A[0..255, k] * B[0..255, k] over K (a multiple of 64);
+// A_rows / B_rows point at the first row of the 256-row operand panels.  Ends with every wave past its last
+// LDS read.  SAME: B is A (a diagonal score tile), loaded once.
+template <bool SAME>
+__device__ __forceinline__ void direct_mainloop(f32x16 (&acc)[4][2], const unsigned short *A_rows, long lda,
+                                                const unsigned short *B_rows, long ldb, int K,
+                                                unsigned short *s_dyn, int wave, int lane) {
+  constexpr int TILE = 256 * 64;
+  constexpr int BUF = 2 * TILE;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int lr = lane >> 3, lc = (lane & 7) ^ ((lr >> 1) | ((wave & 1) << 2));
+  const unsigned short *pa[4], *pb[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int bi = c * 8 + wave;
+    pa[c] = A_rows + (long)(bi * 8 + lr) * lda + lc * 8;
+    pb[c] = B_rows + (long)(bi * 8 + lr) * ldb + lc * 8;
+  }
+#define BDH_ISSUE(buf, k0)                                                                                          \
+  _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                                   \
+    const int bi = c * 8 + wave;                                                                                    \
+    __builtin_amdgcn_global_load_lds((gptr_t)(pa[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + bi * 512), 16, 0, 0);     \
+    if (!SAME)                                                                                                      \
+      __builtin_amdgcn_global_load_lds((gptr_t)(pb[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, 0); \
+  }
+  BDH_ISSUE(0, 0)
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  int cur = 0;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    if (k0 + BK < K) { BDH_ISSUE(cur ^ 1, k0 + BK) }
+    const unsigned short *sa = s_dyn + cur * BUF, *sb = SAME ? sa : sa + TILE;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 16) {
+      bf16x8 fa[4], fb[2];
+      const int C = (kk >> 3) + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int R = wm * 128 + i * 32 + (lane & 31);
+        fa[i] = *reinterpret_cast<const bf16x8 *>(sa + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ ((R >> 1) & 7))) * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int R = wn * 64 + j * 32 + (lane & 31);
+        fb[j] = *reinterpret_cast<const bf16x8 *>(sb + (R >> 3) * 512 + (((R & 7) << 3) + (C ^ ((R >> 1) & 7))) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    cur ^= 1;
+  }
+#undef BDH_ISSUE
+}
+
+// Workgroup barrier that orders LDS accesses only: global loads and stores issued before it stay in flight
+// (__syncthreads also waits for every outstanding global access).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at "no wait")
+#define BDH_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+struct ChunkOutArgs {
+  const unsigned short *Q;   // [S][Tc][N] rotated activations of this pass
+  long q_slice;
+  const unsigned short *P;   // [slot][S][256][N]: bf16(rho_c)^T, slot c = the state before chunk c
+  long p_slot, p_slice;
+  const unsigned short *Vt;  // [B][256][ldv]: V^T of this pass
+  long vt_batch;
+  float *out;                // row 0 of this pass in out [S][T][256]
+  long out_slice;
+  int N, ldv, nc, n_slices, h;
+  int has_state;             // chunk 0 has a state term as well
+  int lo_slot;               // >= 0: chunk 0 also adds Q_0 * P[lo_slot] (the rounding remainder of the carried state)
+};
+
+constexpr int S_ROW = 256 + 8;  // bf16 elements per row of the score tile in LDS (528 bytes: 16-byte reads of 16
+                                // consecutive rows cover the 64 banks once)
+constexpr int CHUNK_OUT_LDS = 256 * S_ROW * 2;  // 135168 bytes >= the 128 KiB of the operand buffers
+
+__global__ __launch_bounds__(512) void k_chunk_out(ChunkOutArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned short s_dyn[];
+  const int xcd = blockIdx.x & 7;
+  const int r = blockIdx.x >> 3;
+  const int slice = xcd + 8 * (r / g.nc);
+  if (slice >= g.n_slices) return;
+  const int c = g.nc - 1 - r % g.nc;  // later chunks first: they all have a state term
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const unsigned short *Qc = g.Q + (long)slice * g.q_slice + (long)c * 256 * g.N;
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  // 1. S = Q_c Q_c^T
+  direct_mainloop<true>(acc, Qc, g.N, Qc, g.N, g.N, s_dyn, wave, lane);
+
+  // 2. tril(-1), rounded to bf16, into LDS as the A operand of S V (the operand buffers are free now)
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        s_dyn[row * S_ROW + col] = col < row ? f32_to_bf16_bits(acc[i][j][e]) : (unsigned short)0;
+        acc[i][j][e] = 0.0f;
+      }
+    }
+  __syncthreads();
+
+  // 3. out = S V_c: A fragments from LDS, B fragments (V^T rows = value columns, k = token) straight from
+  //    global memory (128 KiB per workgroup, shared by the heads of a sequence).  Rows 0..127 (wm = 0) see
+  //    only the first 128 tokens of the chunk.
+  {
+    const unsigned short *vt = g.Vt + (long)(slice / g.h) * g.vt_batch + (long)c * 256 + (lane >> 5) * 8;
+    const unsigned short *vrow[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) vrow[j] = vt + (long)(wn * 64 + j * 32 + (lane & 31)) * g.ldv;
+    const int kend = wm == 0 ? 128 : 256;
+    for (int k0 = 0; k0 < kend; k0 += 64) {
+      bf16x8 fb[4][2];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[q][j] = *reinterpret_cast<const bf16x8 *>(vrow[j] + k0 + q * 16);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        bf16x8 fa[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int R = wm * 128 + i * 32 + (lane & 31);
+          fa[i] = *reinterpret_cast<const bf16x8 *>(s_dyn + R * S_ROW + k0 + q * 16 + (lane >> 5) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[q][j], acc[i][j], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();  // the score tile is overwritten by the operand buffers of the next product
+
+  // 4. out += Q_c bf16(rho_c)   (+ Q_0 times the rounding remainder of a carried state)
+  if (c > 0 || g.has_state) {
+    const unsigned short *Pc = g.P + (long)c * g.p_slot + (long)slice * g.p_slice;
+    direct_mainloop<false>(acc, Qc, g.N, Pc, g.N, g.N, s_dyn, wave, lane);
+    if (c == 0 && g.lo_slot >= 0) {
+      const unsigned short *Pl = g.P + (long)g.lo_slot * g.p_slot + (long)slice * g.p_slice;
+      direct_mainloop<false>(acc, Qc, g.N, Pl, g.N, g.N, s_dyn, wave, lane);
+    }
+  }
+
+  float *o = g.out + (long)slice * g.out_slice + (long)c * 256 * 256;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        o[(long)row * 256 + col] = acc[i][j][e];
+      }
+    }
+}
+
+struct StateUpdArgs {
+  const unsigned short *X;   // x bf16, token 0 of this pass; rows of N
+  long x_slice;
+  unsigned short *Q;         // [S][Tc][N] out: bf16(rope(x))
+  long q_slice;
+  const unsigned short *Vt;  // [B][256][ldv]
+  long vt_batch;
+  const float *freqs;        // [N]
+  float *rho;                // [S][N][256] in/out
+  unsigned short *P;         // [slot][S][256][N]
+  long p_slot, p_slice;
+  long pos0;                 // position of token 0 of this pass
+  int N, Tc, ldv, h, n_slices, nt;  // nt = N / 256 neuron tiles per slice
+  int has_state;             // the accumulators start from rho, and slot 0 is written
+  int lo_slot;               // >= 0: bf16(rho_0 - float(bf16(rho_0))) goes to that slot
+  const int *pairs_equal;    // device flag written by k_freq_pairs_equal
+};
+
+constexpr int UPD_A_TILE = 64 * KM_STRIDE;       // k-major activations tile: 64 tokens x (256+32) neurons
+constexpr int UPD_B_TILE = 256 * LDS_STRIDE;     // V^T tile: 256 value columns x (64+8) tokens
+constexpr int UPD_BUF = UPD_A_TILE + UPD_B_TILE;  // elements per stage (73728 bytes)
+constexpr int UPD_LDS = 2 * UPD_BUF * 2 + 256 * 2 * 4;  // two stages + the per-neuron 16-token rotation steps
+#ifndef BDH_UPD_SCHED
+#define BDH_UPD_SCHED 1
+#endif
+constexpr int DUMP_ROW = 256 + 8;                 // bf16 elements per staged row of a state dump
+static_assert(128 * DUMP_ROW <= UPD_BUF, "half a dump must fit the free stage");
+
+template <bool EQ>  // EQ: the two elements of every lane pair share a frequency (what build_freqs makes)
+__device__ __forceinline__ void state_update_body(const StateUpdArgs &g, unsigned short *s_dyn) {
+  float *s_step = reinterpret_cast<float *>(s_dyn + 2 * UPD_BUF);  // [256][2]: cos, sin of 16 tokens' phase advance
+  const int xcd = blockIdx.x & 7;
+  const int r = blockIdx.x >> 3;
+  const int slice = xcd + 8 * (r / g.nt);
+  if (slice >= g.n_slices) return;
+  const int m0 = (r % g.nt) * 256;  // first neuron of this workgroup
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+
+  const unsigned short *X = g.X + (long)slice * g.x_slice + m0;
+  unsigned short *Qo = g.Q + (long)slice * g.q_slice + m0;
+  const unsigned short *Vt = g.Vt + (long)(slice / g.h) * g.vt_batch;
+  float *rho = g.rho + ((long)slice * g.N + m0) * 256;
+
+  // rotation state of this thread: neurons mc..mc+7 of the tile, tokens (tid >> 5) + 16 j, j = 0, 1, ...
+  // (cos, sin) of the even element of each of the four lane pairs, and of the odd one when the table gives
+  // the two elements of a pair different frequencies (build_freqs gives them the same: then the whole
+  // wavefront keeps four states instead of eight)
+  const int mc = (tid & 31) * 8, tk = tid >> 5;
+  float cse[4], sne[4], cso[EQ ? 1 : 4], sno[EQ ? 1 : 4];
+  constexpr bool eq = EQ;
+  if (tid < 256) {
+    // the phase advance of 16 tokens: 16 f is exact in binary32, the fraction is taken as the reference takes it
+    const float raw = 16.0f * g.freqs[m0 + tid];
+    float s16, c16;
+    sincosf((raw - floorf(raw)) * kTwoPi, &s16, &c16);
+    s_step[2 * tid] = c16;
+    s_step[2 * tid + 1] = s16;
+  }
+  // exact phases (src/model/attention.rs:338-343) at the first token of a chunk; 16-token steps inside it
+  auto seed = [&](int token) {
+    const float pos = (float)(g.pos0 + token);
+    const float4 f0 = *reinterpret_cast<const float4 *>(g.freqs + m0 + mc);
+    const float4 f1 = *reinterpret_cast<const float4 *>(g.freqs + m0 + mc + 4);
+    const float fre[4] = {f0.x, f0.z, f1.x, f1.z}, fro[4] = {f0.y, f0.w, f1.y, f1.w};
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const float raw = pos * fre[p];
+      sincosf((raw - floorf(raw)) * kTwoPi, &sne[p], &cse[p]);
+      if constexpr (!eq) {
+        const float rawo = pos * fro[p];
+        sincosf((rawo - floorf(rawo)) * kTwoPi, &sno[p], &cso[p]);
+      }
+    }
+  };
+  auto advance = [&]() {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const float4 st = *reinterpret_cast<const float4 *>(s_step + 2 * (mc + 2 * p));  // c16, s16 of 2p and 2p + 1
+      const float c0 = cse[p] * st.x - sne[p] * st.y, s0 = sne[p] * st.x + cse[p] * st.y;
+      cse[p] = c0; sne[p] = s0;
+      if constexpr (!eq) {
+        const float c1 = cso[p] * st.z - sno[p] * st.w, s1 = sno[p] * st.z + cso[p] * st.w;
+        cso[p] = c1; sno[p] = s1;
+      }
+    }
+  };
+  // q[2j] = x[2j] cos + (-x[2j+1]) sin ; q[2j+1] = x[2j+1] cos + x[2j] sin  (src/model/attention.rs:305-321),
+  // rounded to bf16 (nearest even) by the conversion instruction
+  auto rotate = [&](const uint4 in) -> uint4 {
+    const unsigned int w[4] = {in.x, in.y, in.z, in.w};
+    unsigned int o[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const float xe = __uint_as_float(w[p] << 16), xo = __uint_as_float(w[p] & 0xffff0000u);
+      const float co = eq ? cse[p] : cso[eq ? 0 : p], so = eq ? sne[p] : sno[eq ? 0 : p];
+      const float a0 = xe * cse[p], r0 = (-xo) * sne[p];
+      const float a1 = xo * co, r1 = xe * so;
+      const f32x2 qv = {a0 + r0, a1 + r1};
+      o[p] = __builtin_bit_cast(unsigned int, __builtin_convertvector(qv, bf16x2));
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+  };
+
+  f32x16 acc[4][2];
+  if (g.has_state) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int col = wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          acc[i][j][e] = rho[(long)row * 256 + col];
+        }
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  }
+
+  uint4 ra[4];
+  // addresses = a wavefront-uniform row pointer + this lane's 32-bit offset (scalar base + vector offset form)
+  const int lane_off = tk * g.N + mc;
+  auto load_piece = [&](int step, int c) {  // activations of 16 tokens of a step into registers
+    const unsigned short *rowp = X + (long)(step * 64 + c * 16) * g.N;
+    ra[c] = *reinterpret_cast<const uint4 *>(rowp + lane_off);
+  };
+  // The V^T tile of a step (256 value columns x 64 tokens, L2-resident) goes through registers, half a tile at a
+  // time.  (A direct global->LDS copy would save the registers, but the compiler then makes every LDS access that
+  // might alias its destination wait for ALL outstanding global accesses, the prefetched activations included.)
+  uint4 rb[2];
+  const int v_lane_off = (tid >> 3) * g.ldv + (tid & 7) * 8;
+  auto load_v = [&](int step, int half) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      // chunk = (half*2 + c)*512 + tid: row = chunk >> 3 = (half*2 + c)*64 + (tid >> 3), k-chunk = tid & 7
+      const unsigned short *vp = Vt + (long)((half * 2 + c) * 64) * g.ldv + step * 64;
+      rb[c] = *reinterpret_cast<const uint4 *>(vp + v_lane_off);
+    }
+  };
+  auto store_v = [&](int step, int half) {
+    unsigned short *sb = s_dyn + (step & 1) * UPD_BUF + UPD_A_TILE;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int chunk = (half * 2 + c) * 512 + tid;
+      const int row = chunk >> 3, kc = (chunk & 7) * 8;
+      *reinterpret_cast<uint4 *>(sb + row * LDS_STRIDE + kc) = rb[c];
+    }
+  };
+  // piece c of a staged step: rotate, write Q, put both operands into the stage's LDS buffers
+  auto stage_piece = [&](int step, int c) {
+    unsigned short *sa = s_dyn + (step & 1) * UPD_BUF;
+    const uint4 q = rotate(ra[c]);
+    advance();
+    const int kr = c * 16 + tk;
+    unsigned short *qrow = Qo + (long)(step * 64 + c * 16) * g.N;
+    *reinterpret_cast<uint4 *>(qrow + lane_off) = q;
+    *reinterpret_cast<uint4 *>(sa + kr * KM_STRIDE + (mc ^ (((kr >> 3) & 1) << 5))) = q;
+  };
+  // bf16 of the accumulators, transposed to [value column][neuron], through the free stage buffer
+  auto dump = [&](unsigned short *stage, int slot, bool remainder) {
+    // per-lane bases laundered through the register file: every access below is base + constant, and the
+    // compiler cannot hoist 70 precomputed addresses out of the token loop (that spilled the accumulators)
+    unsigned short *wbase = stage + ((wn & 1) * 64 + (lane & 31)) * DUMP_ROW + wm * 128 + (lane >> 5) * 4;
+    unsigned short *rbase = stage + (tid >> 5) * DUMP_ROW + (tid & 31) * 8;
+    unsigned short *dst = g.P + (long)slot * g.p_slot + (long)slice * g.p_slice + m0 + (long)(tid >> 5) * g.N + (tid & 31) * 8;
+    asm volatile("" : "+v"(wbase), "+v"(rbase), "+v"(dst));
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      if ((wn >> 1) == half) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+              unsigned short b[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float v = acc[i][j][e4 * 4 + e];
+                const unsigned short hi = f32_to_bf16_bits(v);
+                b[e] = remainder ? f32_to_bf16_bits(v - bf16_bits_to_f32(hi)) : hi;
+              }
+              *reinterpret_cast<uint2 *>(wbase + j * 32 * DUMP_ROW + i * 32 + e4 * 8) =
+                  make_uint2((unsigned int)b[0] | ((unsigned int)b[1] << 16), (unsigned int)b[2] | ((unsigned int)b[3] << 16));
+            }
+          }
+      }
+      lds_barrier();
+#pragma unroll
+      for (int pass = 0; pass < 8; ++pass)
+        *reinterpret_cast<uint4 *>(dst + (long)(half * 128 + pass * 16) * g.N) =
+            *reinterpret_cast<const uint4 *>(rbase + pass * 16 * DUMP_ROW);
+      lds_barrier();
+    }
+  };
+
+  const int nk = g.Tc / 64;
+  __syncthreads();  // s_step
+#pragma unroll
+  for (int c = 0; c < 4; ++c) load_piece(0, c);
+  load_v(0, 0);
+  seed(tk);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    stage_piece(0, c);
+    if (nk > 1) load_piece(1, c);
+  }
+  store_v(0, 0);
+  load_v(0, 1);
+  store_v(0, 1);
+  lds_barrier();
+  // One step: the matrix products of step kt from one LDS stage and, between them and 16 tokens at a time,
+  // {rotate step kt+1's activations, store Q, fill the other stage, fetch step kt+2}; step kt+1's V^T tile
+  // follows in two halves.  MORE / MORE2 (is there a step kt+1 / kt+2) are compile-time so that the body is one
+  // straight block the scheduler can interleave; barriers order LDS only, global accesses stay in flight.
+  auto step = [&](int kt, auto more_t, auto more2_t) {
+    constexpr bool MORE = decltype(more_t)::value, MORE2 = decltype(more2_t)::value;
+    const unsigned short *s_a = s_dyn + (kt & 1) * UPD_BUF, *s_b = s_a + UPD_A_TILE;
+    if ((kt & 3) == 0 && (kt > 0 || g.has_state)) {
+      unsigned short *stage = s_dyn + ((kt + 1) & 1) * UPD_BUF;
+      dump(stage, kt >> 2, false);
+      if (kt == 0 && g.lo_slot >= 0) dump(stage, g.lo_slot, true);
+    }
+    if (MORE && (kt & 3) == 3) seed((kt + 1) * 64 + tk);  // the next step opens a chunk: exact phases
+    if (MORE) load_v(kt + 1, 0);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 16) {
+      if (MORE) {
+        stage_piece(kt + 1, kk >> 4);
+        if (MORE2) load_piece(kt + 2, kk >> 4);
+        if (kk == 32) {
+          store_v(kt + 1, 0);
+          load_v(kt + 1, 1);
+        }
+      }
+      bf16x8 fa[4], fb[2];
+      const int kof = kk + (lane >> 5) * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        // transposing LDS read: see k_gemm
+        const int j16 = lane & 15;
+        const int mcol = (wm * 128 + i * 32 + ((lane >> 4) & 1) * 16) ^ ((lane >> 5) << 5);
+        const unsigned short *src = s_a + (kof + (j16 >> 2)) * KM_STRIDE + mcol + (j16 & 3) * 4;
+        typedef short s16x4 __attribute__((ext_vector_type(4)));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_t;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(src));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(src + 4 * KM_STRIDE));
+        const s16x8 pk = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        fa[i] = __builtin_bit_cast(bf16x8, pk);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        fb[j] = *reinterpret_cast<const bf16x8 *>(s_b + (wn * 64 + j * 32 + (lane & 31)) * LDS_STRIDE + kof);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+#if BDH_UPD_SCHED
+      if (MORE) {
+#pragma unroll
+        for (int q8 = 0; q8 < 8; ++q8) {  // the rotation arithmetic in the shadow of the matrix instructions
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 9, 0);
+        }
+      }
+#endif
+    }
+    if (MORE) store_v(kt + 1, 1);
+    lds_barrier();
+  };
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
+  if (kt + 1 < nk) step(kt++, std::true_type{}, std::false_type{});
+  step(kt, std::false_type{}, std::false_type{});
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        rho[(long)row * 256 + col] = acc[i][j][e];
+      }
+    }
+}
+
+// flag[0] = 1 when the two elements of every lane pair share a frequency (what build_freqs makes), else 0
+__global__ __launch_bounds__(256) void k_freq_pairs_equal(const float *__restrict__ freqs, int N, int *__restrict__ flag) {
+  int ok = 1;
+  for (int p = threadIdx.x; p < N / 2; p += 256) {
+    const float2 f = reinterpret_cast<const float2 *>(freqs)[p];
+    ok &= f.x == f.y;
+  }
+  ok = __syncthreads_and(ok);
+  if (threadIdx.x == 0) flag[0] = ok;
+}
+
+// Both instantiations are launched; the one the frequency table does not call for returns at once (the choice
+// is made on the device, so no host synchronisation is needed, and each body gets its own register allocation).
+template <bool EQ>
+__global__ __launch_bounds__(512) void k_state_update(StateUpdArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned short s_dyn[];
+  if ((g.pairs_equal[0] != 0) != EQ) return;
+  state_update_body<EQ>(g, s_dyn);
+}
+
 template <bool AK, int EPI>
 hipError_t launch_gemm(hipStream_t st, const GemmArgs &g) {
   const int groups = (g.n_slices + 7) / 8;
@@ -453,20 +969,11 @@ hipError_t launch_gemm(hipStream_t st, const GemmArgs &g) {
   return hipSuccess;
 }
 
-}  // namespace
-
-extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
-                                   const uint16_t *v_bf16, const float *freqs, int64_t position,
-                                   int state_is_zero, float *rho, float *out) {
-  if (!ctx) return BDH_E_INVAL;
-  if (B < 0 || h < 0 || T < 0 || N < 0 || d < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
-  if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
-  if (B == 0 || h == 0 || T == 0) return BDH_OK;
-  if ((N & 7) || (d & 7) || N == 0 || d == 0)
-    return bdh_fail(ctx, BDH_E_SHAPE, "chunked prefill needs N and d to be positive multiples of 8 (N=%d d=%d)", N, d);
-  if (!x_bf16 || !v_bf16 || !freqs || !rho || !out) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
-  if (!bdh_aligned(x_bf16, 16) || !bdh_aligned(v_bf16, 16) || !bdh_aligned(rho, 16) || !bdh_aligned(out, 16))
-    return bdh_fail(ctx, BDH_E_ALIGN, "x, v, rho and out need 16-byte alignment");
+// One pass of the all-scores form (any T, N, d that are multiples of 8): tokens [0, T) of the pointers given,
+// x / out slices x_slice / out_slice elements apart.
+static int prefill_pass_scores(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16, long x_slice,
+                               const uint16_t *v_bf16, long v_batch, const float *freqs, int64_t position,
+                               int state_is_zero, float *rho, float *out, long out_slice) {
   const int S = B * h;
   const int Tp = (T + 7) / 8 * 8;  // leading dimension of the score matrix
   const int mt = (T + BM - 1) / BM;  // row/col tiles of the score matrix
@@ -488,15 +995,14 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
   unsigned short *Rt = reinterpret_cast<unsigned short *>(ws + q_bytes + s_bytes + vt_bytes);
   if ((long)S * n_score_tiles > 0x7fffffffL / 16 || (long)S * n_rho_tiles > 0x7fffffffL / 16)
     return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles (T=%d N=%d)", T, N);
-  if (B > 65535 || S > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "batch too large for the transpose grid");
 
   // 0. V^T (and rho0^T): make every B operand k-contiguous
   hipLaunchKernelGGL(k_transpose_to_bf16<unsigned short>, dim3((d + 63) / 64, (Tp + 63) / 64, B), dim3(256), 0,
-                     ctx->stream, v_bf16, Vt, T, d, Tp);
+                     ctx->stream, v_bf16, Vt, T, d, Tp, v_batch);
   BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<V>");
   if (!state_is_zero) {
     hipLaunchKernelGGL(k_transpose_to_bf16<float>, dim3((d + 63) / 64, (N + 63) / 64, S), dim3(256), 0, ctx->stream,
-                       rho, Rt, N, d, N);
+                       rho, Rt, N, d, N, (long)N * d);
     BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<rho0>");
   }
   // 1. rotation
@@ -504,7 +1010,7 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
     const long work = (long)T * (N / 8);
     hipLaunchKernelGGL(k_rope_bf16, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, ctx->stream,
                        reinterpret_cast<const uint4 *>(x_bf16), reinterpret_cast<uint4 *>(Q), freqs, S, T, N,
-                       (float)position, (long)position);
+                       x_slice / 8, (long)position);
     BDH_LAUNCH_CHECK(ctx, "k_rope_bf16");
   }
   // 2. scores = tril(-1)(Q Q^T), lower tiles only
@@ -522,7 +1028,7 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
   if (!state_is_zero) {
     GemmArgs g{};
     g.A = Q; g.B = Rt; g.C = out;
-    g.a_batch = (long)T * N; g.b_batch = (long)d * N; g.c_batch = (long)T * d;
+    g.a_batch = (long)T * N; g.b_batch = (long)d * N; g.c_batch = out_slice;
     g.lda = N; g.ldb = N; g.ldc = d;
     g.M = T; g.N = d; g.K = N; g.b_div = 1; g.beta = 0; g.causal_k = 0;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
@@ -533,7 +1039,7 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
   {
     GemmArgs g{};
     g.A = Sc; g.B = Vt; g.C = out;
-    g.a_batch = (long)T * Tp; g.b_batch = (long)d * Tp; g.c_batch = (long)T * d;
+    g.a_batch = (long)T * Tp; g.b_batch = (long)d * Tp; g.c_batch = out_slice;
     g.lda = Tp; g.ldb = Tp; g.ldc = d;
     g.M = T; g.N = d; g.K = T; g.b_div = h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 1;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
@@ -550,6 +1056,126 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
     g.tri = 0; g.mt = nt_rho; g.nt = nt_d; g.n_tiles = n_rho_tiles; g.n_slices = S;
     BDH_HIP_CHECK(ctx, (launch_gemm<true, EPI_ACC>(ctx->stream, g)));
     BDH_LAUNCH_CHECK(ctx, "k_gemm<Q^T V>");
+  }
+  return BDH_OK;
+}
+
+// dynamic LDS beyond 64 KiB must be allowed per (kernel, device)
+template <typename K>
+static hipError_t allow_lds(K kernel, int bytes, std::atomic<uint64_t> &configured) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (configured.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) configured.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
+// One pass of the chunk-recurrent form: Tc tokens (a multiple of 256), N a multiple of 256, d = 256.
+static int prefill_pass_chunks(bdh_ctx *ctx, int B, int h, int Tc, int N, const uint16_t *x_bf16, long x_slice,
+                               const uint16_t *v_bf16, long v_batch, const float *freqs, int64_t position,
+                               int state_is_zero, int hilo, float *rho, float *out, long out_slice) {
+  constexpr int d = 256;
+  const int S = B * h, nc = Tc / 256, nt = N / 256;
+  const int lo_slot = (!state_is_zero && hilo) ? nc : -1;
+  const int slots = nc + (lo_slot >= 0 ? 1 : 0);
+  // workspace: Q bf16 [S,Tc,N] | P bf16 [slots,S,d,N] | V^T bf16 [B,d,Tc]
+  const size_t q_bytes = bdh_align_up((size_t)S * Tc * N * 2, 256);
+  const size_t p_bytes = bdh_align_up((size_t)slots * S * d * N * 2, 256);
+  const size_t vt_bytes = bdh_align_up((size_t)B * d * Tc * 2, 256);
+  int rc = bdh_ws_reserve(ctx, q_bytes + p_bytes + vt_bytes + 256);
+  if (rc != BDH_OK) return rc;
+  char *ws = static_cast<char *>(ctx->ws);
+  unsigned short *Q = reinterpret_cast<unsigned short *>(ws);
+  unsigned short *P = reinterpret_cast<unsigned short *>(ws + q_bytes);
+  unsigned short *Vt = reinterpret_cast<unsigned short *>(ws + q_bytes + p_bytes);
+  int *flag = reinterpret_cast<int *>(ws + q_bytes + p_bytes + vt_bytes);
+  const int groups = (S + 7) / 8;
+  if ((long)groups * 8 * std::max(nt, nc) > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
+
+  hipLaunchKernelGGL(k_transpose_to_bf16<unsigned short>, dim3(d / 64, Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16,
+                     Vt, Tc, d, Tc, v_batch);
+  BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<V>");
+  hipLaunchKernelGGL(k_freq_pairs_equal, dim3(1), dim3(256), 0, ctx->stream, freqs, N, flag);
+  BDH_LAUNCH_CHECK(ctx, "k_freq_pairs_equal");
+  {
+    static std::atomic<uint64_t> configured_eq{0}, configured_ne{0};
+    BDH_HIP_CHECK(ctx, allow_lds(k_state_update<true>, UPD_LDS, configured_eq));
+    BDH_HIP_CHECK(ctx, allow_lds(k_state_update<false>, UPD_LDS, configured_ne));
+    StateUpdArgs g{};
+    g.X = x_bf16; g.x_slice = x_slice;
+    g.Q = Q; g.q_slice = (long)Tc * N;
+    g.Vt = Vt; g.vt_batch = (long)d * Tc; g.ldv = Tc;
+    g.freqs = freqs; g.rho = rho;
+    g.P = P; g.p_slot = (long)S * d * N; g.p_slice = (long)d * N;
+    g.pos0 = (long)position;
+    g.N = N; g.Tc = Tc; g.h = h; g.n_slices = S; g.nt = nt;
+    g.has_state = state_is_zero ? 0 : 1; g.lo_slot = lo_slot;
+    g.pairs_equal = flag;
+    hipLaunchKernelGGL(k_state_update<true>, dim3(8 * groups * nt), dim3(512), UPD_LDS, ctx->stream, g);
+    hipLaunchKernelGGL(k_state_update<false>, dim3(8 * groups * nt), dim3(512), UPD_LDS, ctx->stream, g);
+    BDH_LAUNCH_CHECK(ctx, "k_state_update");
+  }
+  {
+    static std::atomic<uint64_t> configured{0};
+    BDH_HIP_CHECK(ctx, allow_lds(k_chunk_out, CHUNK_OUT_LDS, configured));
+    ChunkOutArgs g{};
+    g.Q = Q; g.q_slice = (long)Tc * N;
+    g.P = P; g.p_slot = (long)S * d * N; g.p_slice = (long)d * N;
+    g.Vt = Vt; g.vt_batch = (long)d * Tc; g.ldv = Tc;
+    g.out = out; g.out_slice = out_slice;
+    g.N = N; g.nc = nc; g.n_slices = S; g.h = h;
+    g.has_state = state_is_zero ? 0 : 1; g.lo_slot = lo_slot;
+    hipLaunchKernelGGL(k_chunk_out, dim3(8 * groups * nc), dim3(512), CHUNK_OUT_LDS, ctx->stream, g);
+    BDH_LAUNCH_CHECK(ctx, "k_chunk_out");
+  }
+  return BDH_OK;
+}
+
+}  // namespace
+
+extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
+                                   const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk,
+                                   int flags, float *rho, float *out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (B < 0 || h < 0 || T < 0 || N < 0 || d < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
+  if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
+  if (chunk < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative chunk length");
+  if (flags & ~(BDH_PREFILL_STATE_IS_ZERO | BDH_PREFILL_STATE_HILO | BDH_PREFILL_ALL_SCORES))
+    return bdh_fail(ctx, BDH_E_INVAL, "unknown flag bits 0x%x", flags);
+  if (B == 0 || h == 0 || T == 0) return BDH_OK;
+  if ((N & 7) || (d & 7) || N == 0 || d == 0)
+    return bdh_fail(ctx, BDH_E_SHAPE, "chunked prefill needs N and d to be positive multiples of 8 (N=%d d=%d)", N, d);
+  if (!x_bf16 || !v_bf16 || !freqs || !rho || !out) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  if (!bdh_aligned(x_bf16, 16) || !bdh_aligned(v_bf16, 16) || !bdh_aligned(rho, 16) || !bdh_aligned(out, 16))
+    return bdh_fail(ctx, BDH_E_ALIGN, "x, v, rho and out need 16-byte alignment");
+  if (B > 65535 || B * h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "batch too large for the transpose grid");
+  // tokens per pass: the workspace holds the rotated activations (and, in the all-scores form, the score
+  // matrix) of one pass only; the state is carried from pass to pass in the caller's f32 rho
+  const int pass_default = 2048;
+  int pass = chunk > 0 ? chunk : pass_default;
+  const bool aligned = !(flags & BDH_PREFILL_ALL_SCORES) && d == 256 && N % 256 == 0;
+  int zero = (flags & BDH_PREFILL_STATE_IS_ZERO) ? 1 : 0;
+  const int hilo = (flags & BDH_PREFILL_STATE_HILO) ? 1 : 0;
+  for (int t0 = 0; t0 < T;) {
+    int Tc = std::min(pass, T - t0);
+    const uint16_t *xp = x_bf16 + (long)t0 * N;
+    const uint16_t *vp = v_bf16 + (long)t0 * d;
+    float *op = out + (long)t0 * d;
+    int rc;
+    if (aligned && Tc >= 256) {
+      Tc -= Tc % 256;  // a ragged tail goes to the all-scores form below
+      rc = prefill_pass_chunks(ctx, B, h, Tc, N, xp, (long)T * N, vp, (long)T * d, freqs, position + t0, zero, hilo, rho,
+                               op, (long)T * d);
+    } else {
+      rc = prefill_pass_scores(ctx, B, h, Tc, N, d, xp, (long)T * N, vp, (long)T * d, freqs, position + t0, zero, rho,
+                               op, (long)T * d);
+    }
+    if (rc != BDH_OK) return rc;
+    zero = 0;
+    t0 += Tc;
   }
   return BDH_OK;
 }

@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(PKG, "libbdh_mi355x.so")
 OK, E_INVAL, E_SHAPE, E_ALIGN, E_HIP, E_NOMEM, E_UNSUPPORTED = 0, -1, -2, -3, -4, -5, -6
 ROPE, ALIBI, POPE = 0, 1, 2
 F32, BF16 = 0, 1
+PREFILL_STATE_IS_ZERO, PREFILL_STATE_HILO, PREFILL_ALL_SCORES = 1, 2, 4
 
 # every symbol include/bdh_mi355x.h declares
 EXPORTS = [
@@ -91,7 +92,7 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_layer_norm.argtypes = [P, c_int64, c_int, P, P]
     lib.bdh_fused_state_aligned.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, P, c_int, P, c_int, c_int,
                                             c_int, P]
-    lib.bdh_prefill_chunked.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, c_int, P, P]
+    lib.bdh_prefill_chunked.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, c_int, c_int, P, P]
     lib.bdh_model_create.argtypes = [P, POINTER(ModelConfigC), POINTER(ModelWeightsC), POINTER(P)]
     lib.bdh_model_destroy.argtypes = [P]
     lib.bdh_model_state_bytes.restype = c_size_t

@@ -119,10 +119,13 @@ def layer_norm(x: torch.Tensor, ctx: Optional[ffi.Context] = None) -> torch.Tens
 
 
 def prefill_chunked(x_bf16: torch.Tensor, v_bf16: torch.Tensor, rho: torch.Tensor, freqs: torch.Tensor,
-                    position: int, state_is_zero: bool = False, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
+                    position: int, state_is_zero: bool = False, chunk: int = 0, hilo: bool = False,
+                    all_scores: bool = False, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
     """The recurrent path (src/model/bdh.rs:258-307, RoPE) for T tokens at once on the bf16 matrix
     cores.  x_bf16 [B,h,T,N] bfloat16 un-rotated, v_bf16 [B,T,d] bfloat16, rho [B,h,N,d] float32
-    (updated in place).  Returns out [B,h,T,d] float32."""
+    (updated in place).  chunk = tokens per internal pass (0 = 2048; the workspace grows with it, not
+    with T); hilo = the state carried into the call enters its product as a bf16 pair; all_scores = never the
+    chunk-recurrent form.  Returns out [B,h,T,d] float32."""
     ctx = ctx or ffi.default_context(x_bf16.device.index or 0)
     B, h, T, N = x_bf16.shape
     d = v_bf16.shape[-1]
@@ -132,7 +135,9 @@ def prefill_chunked(x_bf16: torch.Tensor, v_bf16: torch.Tensor, rho: torch.Tenso
     assert rho.dtype == torch.float32 and rho.is_contiguous() and tuple(rho.shape) == (B, h, N, d)
     out = torch.empty((B, h, T, d), device=x_bf16.device, dtype=torch.float32)
     freqs = freqs.reshape(-1)
+    flags = ((ffi.PREFILL_STATE_IS_ZERO if state_is_zero else 0) | (ffi.PREFILL_STATE_HILO if hilo else 0) |
+             (ffi.PREFILL_ALL_SCORES if all_scores else 0))
     ctx.check(ctx.lib.bdh_prefill_chunked(ctx.handle, B, h, T, N, d, ffi.ptr(x_bf16), ffi.ptr(v_bf16),
-                                          ffi.ptr(freqs), int(position), int(bool(state_is_zero)), ffi.ptr(rho),
+                                          ffi.ptr(freqs), int(position), int(chunk), flags, ffi.ptr(rho),
                                           ffi.ptr(out)))
     return out

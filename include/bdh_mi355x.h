@@ -236,14 +236,30 @@ int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N, int dv,
  *   x   [B,h,T,N] bf16 (raw 16-bit patterns) un-rotated activations
  *   v   [B,T,d]   bf16, shared by the heads of a batch entry
  *   position      start position of token 0
- *   state_is_zero non-zero: the caller promises rho holds zeros (a fresh state, src/model/
- *                 state.rs:27-45); the Q rho0 product is skipped and rho is overwritten
+ *   chunk         tokens per internal pass (0 = 2048).  The call walks the T tokens in passes of this
+ *                 many; the workspace holds one pass (rotated activations [B*h, chunk, N] in bf16 and, for
+ *                 shapes that take the chunk-recurrent form, one bf16 copy of the state per 256 tokens of
+ *                 the pass), so it is linear in chunk and independent of T.  Between passes the state is
+ *                 carried in the caller's f32 rho, never rounded.  The chunk-recurrent form (d = 256, N a
+ *                 multiple of 256, passes of 256+ tokens) wants a multiple of 256; a remainder of fewer
+ *                 than 256 tokens takes the all-scores form.
+ *   flags         BDH_PREFILL_STATE_IS_ZERO: the caller promises rho holds zeros (a fresh state,
+ *                 src/model/state.rs:27-45): the Q rho0 product is skipped and rho is overwritten.
+ *                 BDH_PREFILL_STATE_HILO: the state carried INTO the call enters the Q rho0 product as
+ *                 bf16(rho0) + bf16(rho0 - bf16(rho0)) (two products; chunk-recurrent form only), i.e. with 16
+ *                 mantissa bits instead of 8.  Inside a call the state between 256-token chunks enters its
+ *                 product rounded to bf16 once, like the scores and the activations do; the f32 state
+ *                 itself accumulates without rounding either way.
+ *                 BDH_PREFILL_ALL_SCORES: always the all-scores form (every causal 256x256 score tile of
+ *                 the pass, no state copies).
  *   rho [B,h,N,d] f32 in/out,  out [B,h,T,d] f32
- * N and d must be multiples of 8.
+ * N and d must be multiples of 8.  There is no row-normalised variant: the normaliser of
+ * kernel::linear_attention::fused_state_aligned needs whole score rows (bdh_fused_state_aligned).
  */
+enum bdh_prefill_flags { BDH_PREFILL_STATE_IS_ZERO = 1, BDH_PREFILL_STATE_HILO = 2, BDH_PREFILL_ALL_SCORES = 4 };
 int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
-                        const uint16_t *v_bf16, const float *freqs, int64_t position,
-                        int state_is_zero, float *rho, float *out);
+                        const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk,
+                        int flags, float *rho, float *out);
 
 /* ---- a1: the whole cached step ------------------------------------------------------- */
 /* src/model/config.rs:113-164 (BDHConfig) + :10-31 (FusedKernelConfig), as plain scalars */

@@ -184,6 +184,70 @@ def test_prefill_chunked_equals_sequential_recurrence(bda, corc, T, N, d, rho0_s
     assert not out[:, :, 0].any() or rho0_scale != 0.0  # token 0 reads only the initial state
 
 
+@pytest.mark.parametrize("T,N,chunk,rho0_scale,position,hilo", [
+    (256, 256, 0, 0.0, 0, False), (512, 512, 0, 0.05, 77, False), (1024, 256, 512, 0.0, 3000, False),
+    (768, 512, 256, 0.05, 5, True), (600, 256, 512, 0.05, 9, False), (1280, 256, 0, 0.05, 1, True)])
+def test_prefill_chunk_recurrent_form(bda, corc, T, N, chunk, rho0_scale, position, hilo):
+    """Shapes that take the chunk-recurrent kernels (d = 256, N a multiple of 256, passes of 256+ tokens; a ragged tail
+    of the last pass falls to the all-scores form): several 256-token chunks per pass, several passes per call, a
+    carried-in state with and without the bf16 pair, against the sequential oracle (2e-2) and against the all-scores
+    form of the same call."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h, d = 2, 2, 256
+    x, v, rho0 = _prefill_case(T + N + chunk, B, h, T, N, d, 0.2, rho0_scale)
+    freqs = corc.build_freqs(N)
+    q = corc.rotate(x.float().numpy(), freqs, orc.ROPE, position)
+    out_ref, rho_ref = corc.recurrent_attention(q, v.float().numpy(), rho0.numpy(), sparse=True)
+    ft = torch.from_numpy(freqs).to(DEV)
+    rho = rho0.clone().to(DEV)
+    print(f"chunk-recurrent prefill T={T} N={N} chunk={chunk} hilo={hilo}", flush=True)
+    out = prefill_chunked(x.to(DEV), v.to(DEV), rho, ft, position, state_is_zero=(rho0_scale == 0.0), chunk=chunk,
+                          hilo=hilo)
+    torch.cuda.synchronize()
+    e_out, e_rho = rel_err(out.cpu().numpy(), out_ref), rel_err(rho.cpu().numpy(), rho_ref)
+    print(f"   out rel err {e_out:.2e}, state rel err {e_rho:.2e}")
+    assert e_out < 2e-2 and e_rho < 2e-2
+    rho_s = rho0.clone().to(DEV)
+    out_s = prefill_chunked(x.to(DEV), v.to(DEV), rho_s, ft, position, state_is_zero=(rho0_scale == 0.0), chunk=chunk,
+                            all_scores=True)
+    d_out, d_rho = rel_err(out.cpu().numpy(), out_s.cpu().numpy()), rel_err(rho.cpu().numpy(), rho_s.cpu().numpy())
+    # both accumulate Q^T V in f32; their Q differ by a bf16 rounding step here and there (inside a chunk the
+    # chunk-recurrent kernel steps the rotation by angle addition from the chunk's exact phase)
+    assert d_out < 2e-2 and d_rho < 5e-3, (d_out, d_rho)
+
+
+def test_prefill_in_four_calls_equals_one_call(bda, corc):
+    """One prompt fed as four successive calls (the state carried in the caller's f32 rho, entering each call's
+    product as a bf16 pair) against the sequential oracle and against the single call: T = 4096 in chunks of 512."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h, T, N, d = 1, 2, 4096, 512, 256
+    x, v, _ = _prefill_case(21, B, h, T, N, d, 0.1, 0.0)
+    freqs = corc.build_freqs(N)
+    q = corc.rotate(x.float().numpy(), freqs, orc.ROPE, 0)
+    out_ref, rho_ref = corc.recurrent_attention(q, v.float().numpy(), np.zeros((B, h, N, d), np.float32), sparse=True)
+    ft = torch.from_numpy(freqs).to(DEV)
+    xd, vd = x.to(DEV), v.to(DEV)
+    rho1 = torch.zeros((B, h, N, d), device=DEV)
+    out1 = prefill_chunked(xd, vd, rho1, ft, 0, state_is_zero=True, chunk=512)
+    rho4 = torch.zeros((B, h, N, d), device=DEV)
+    outs = []
+    for k in range(4):
+        sl = slice(k * 1024, (k + 1) * 1024)
+        outs.append(prefill_chunked(xd[:, :, sl].contiguous(), vd[:, sl].contiguous(), rho4, ft, k * 1024,
+                                    state_is_zero=(k == 0), chunk=512, hilo=True))
+    out4 = torch.cat(outs, dim=2)
+    torch.cuda.synchronize()
+    errs = (rel_err(out1.cpu().numpy(), out_ref), rel_err(rho1.cpu().numpy(), rho_ref),
+            rel_err(out4.cpu().numpy(), out_ref), rel_err(rho4.cpu().numpy(), rho_ref),
+            rel_err(out4.cpu().numpy(), out1.cpu().numpy()))
+    print("one call / four calls against the oracle (out, rho, out, rho), four against one (out):", errs)
+    assert max(errs) < 2e-2, errs
+    d_rho = rel_err(rho4.cpu().numpy(), rho1.cpu().numpy())
+    assert d_rho < 1e-5, d_rho  # the f32 state never passes through bf16
+
+
 def test_prefill_chunked_then_decode_steps_continue_the_state(bda, corc):
     """Prefill T tokens on the matrix cores, then decode 3 tokens with bdh_state_step: the
     readouts must match the all-sequential oracle (2e-2: the prefilled state carries bf16 error)."""
@@ -232,6 +296,8 @@ def test_prefill_chunked_argument_errors(bda):
     ctx = ffi.default_context(0)
     t = torch.zeros(4096, device=DEV)
     p = t.data_ptr()
-    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 12, 8, p, p, p, 0, 1, p, p) == ffi.E_SHAPE  # N % 8
-    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 16, 8, None, p, p, 0, 1, p, p) == ffi.E_INVAL
-    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 0, 1, 8, 16, 8, None, None, None, 0, 1, None, None) == ffi.OK
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 12, 8, p, p, p, 0, 0, 1, p, p) == ffi.E_SHAPE  # N % 8
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 16, 8, None, p, p, 0, 0, 1, p, p) == ffi.E_INVAL
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 16, 8, p, p, p, 0, -1, 1, p, p) == ffi.E_INVAL  # chunk < 0
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 16, 8, p, p, p, 0, 0, 64, p, p) == ffi.E_INVAL  # flag bits
+    assert ctx.lib.bdh_prefill_chunked(ctx.handle, 0, 1, 8, 16, 8, None, None, None, 0, 0, 1, None, None) == ffi.OK
