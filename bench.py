@@ -110,24 +110,20 @@ def cpu_baseline_model(cfg, B, prompt, budget_s=20.0, max_tokens=256):
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
-def bench_prefill(args):
+def measure_prefill(B=8, h=4, N=8192, d=256, T=2048, density=0.05, steps=10, warmup=3):
     """BASELINE config 3: chunked prefill, B=8, T=2048, h=4, N=8192, d=256, bf16 inputs, f32
-    accumulate, 5 % density, positions 0..T, fresh state.  One step = one bdh_prefill_chunked."""
+    accumulate, 5 % density, positions 0..T, fresh state.  One step = one bdh_prefill_chunked.
+    Returns (ms per call, algorithmic FLOP per call)."""
     import torch
     from scipy.stats import norm
 
-    from burn_dragon_amd import ffi
     from burn_dragon_amd.kernel.linear_attention import build_freqs
     from burn_dragon_amd.positional import RotaryEmbedding
     from burn_dragon_amd.recurrent import prefill_chunked
 
     dev = torch.device("cuda:0")
-    B = 8 if args.batch == 32 else args.batch
-    h, N, d, T = args.heads, args.latent, args.embd, args.time
-    steps = min(args.steps, 20) if args.steps == 1000 else args.steps
-    warmup = min(args.warmup, 3) if args.warmup == 50 else args.warmup
     g = torch.Generator(device=dev).manual_seed(4)
-    mu = float(norm.ppf(args.density))
+    mu = float(norm.ppf(density))
     x = torch.empty((B, h, T, N), device=dev, dtype=torch.bfloat16)
     for b in range(B):  # generated per batch entry to bound the f32 temporary
         x[b] = torch.relu(torch.randn((h, T, N), device=dev, generator=g) + mu).to(torch.bfloat16)
@@ -145,10 +141,30 @@ def bench_prefill(args):
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    gpu_ms = start.elapsed_time(stop)
-    ms = max(gpu_ms, wall * 1e3) / steps
+    ms = max(start.elapsed_time(stop), wall * 1e3) / steps
     flop = float(B * h) * (T * (T - 1.0) * N + T * (T - 1.0) * d + 2.0 * T * N * d)
+    return ms, flop
+
+
+def prefill_executed_flop(B, h, N, d, T):
+    """Matrix-core FLOP the chunk-recurrent form executes (d = 256, N % 256 == 0, T % 256 == 0): per 256-token chunk a
+    full 256x256 score tile (K = N), scores x V (K = 256, half of it for the upper row block), the state term
+    (K = N, absent for the first chunk of a fresh state) and the state update."""
+    nc = T // 256
+    per_slice = nc * 2.0 * 256 * 256 * N + nc * 2.0 * 256 * 256 * 192 + (nc - 1) * 2.0 * 256 * d * N + 2.0 * T * N * d
+    return B * h * per_slice
+
+
+def bench_prefill(args):
+    """BASELINE config 3 (see measure_prefill)."""
+    B = 8 if args.batch == 32 else args.batch
+    h, N, d, T = args.heads, args.latent, args.embd, args.time
+    steps = min(args.steps, 20) if args.steps == 1000 else args.steps
+    warmup = min(args.warmup, 3) if args.warmup == 50 else args.warmup
+    ms, flop = measure_prefill(B, h, N, d, T, args.density, steps, warmup)
     achieved = flop / (ms * 1e-3) / 1e12
+    chunked = d == 256 and N % 256 == 0 and T % 256 == 0
+    executed = prefill_executed_flop(B, h, N, d, T) if chunked else None
     print(json.dumps({
         "metric": "prefill tokens/sec (chunked dense linear attention) + bf16 MFMA utilisation",
         "value": B * T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -156,14 +172,14 @@ def bench_prefill(args):
         "data": "synthetic",
         "config": {"workload": f"BASELINE config 3: chunked prefill B={B} T={T} h={h} N={N} d={d}, bf16 in / f32 "
                                f"accumulate, {args.density:.0%} active, RoPE positions 0..T, fresh state",
-                   "algorithmic_flop_per_step": flop},
+                   "algorithmic_flop_per_step": flop, "executed_flop_per_step": executed},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     # HBM bytes of one call, all kernels: FETCH_SIZE (scaled x2 as for a copy of known size) +
-                     # WRITE_SIZE from profiles/prefill_config3_bf16_kernel_trace.md; measured at the default shape only
-                     "traffic": 7.56e9 if (B, T, h, N, d) == (8, 2048, 4, 8192, 256) else None,
-                     "kernel": "whole bdh_prefill_chunked call (k_rope_bf16 + 3 k_gemm launches); algorithmic FLOP "
-                               "= B*h*[T(T-1)N + T(T-1)d + 2TNd]"},
+                     "executed_tflops": (executed / (ms * 1e-3) / 1e12) if executed else None,
+                     "traffic": None,
+                     "kernel": "whole bdh_prefill_chunked call (k_state_update + k_chunk_out); algorithmic FLOP "
+                               "= B*h*[T(T-1)N + T(T-1)d + 2TNd], the all-scores count of the workload; the "
+                               "chunk-recurrent form executes executed_flop_per_step of them"},
     }))
 
 
@@ -685,6 +701,21 @@ def main():
             "frac_of_measured_ceiling": (achieved / ceiling) if ceiling else None,
         },
     }
+    if default_workload:
+        # BASELINE config 3 beside the headline: the chunked prefill, bf16 matrix cores (its own roofline)
+        del rho, xs, vs
+        torch.cuda.empty_cache()
+        p_ms, p_flop = measure_prefill(steps=5, warmup=2)
+        p_exec = prefill_executed_flop(8, 4, 8192, 256, 2048)
+        result["prefill_config3"] = {
+            "workload": "BASELINE config 3: bdh_prefill_chunked B=8 T=2048 h=4 N=8192 d=256, bf16 in / f32 accumulate, "
+                        "5% active, fresh state, 5 timed calls",
+            "ms": p_ms, "tokens_per_s": 8 * 2048 / (p_ms * 1e-3),
+            "algorithmic_flop": p_flop, "tflops": p_flop / (p_ms * 1e-3) / 1e12,
+            "frac": p_flop / (p_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
+            "executed_flop": p_exec, "executed_tflops": p_exec / (p_ms * 1e-3) / 1e12,
+            "kernel_us_source": "profiles/prefill_config3_bf16_kernel_trace.md",
+        }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(B, h, N, d, freqs_host.numpy())
     print(json.dumps(result))

@@ -16,6 +16,11 @@
 
 namespace {
 
+struct FsaSlopes {
+  float v[64];
+};
+
+
 constexpr float kTwoPi = 6.28318530717958647692f;
 constexpr float kRowNormEps = 1e-6f;  // src/kernel/linear_attention.rs:9
 
@@ -123,7 +128,7 @@ __global__ __launch_bounds__(256) void k_narrow_bf16(const float *__restrict__ i
 
 // one workgroup per (slice, query row i)
 __global__ __launch_bounds__(256) void k_fsa_row(const float *__restrict__ q, const float *__restrict__ v,
-                                                 const float *__restrict__ slopes_dev, int use_alibi, int h,
+                                                 FsaSlopes slopes_dev, int use_alibi, int h,
                                                  int T, int Nq, int dv, int block_size,
                                                  const unsigned char *__restrict__ active,  // [tb*tb] or null
                                                  int tb, int row_normalize, float *__restrict__ out) {
@@ -139,7 +144,7 @@ __global__ __launch_bounds__(256) void k_fsa_row(const float *__restrict__ q, co
   const float *Q = q + slice * (long)T * Nq;
   const float *V = v + b * (long)T * dv;
   const int rb = i / block_size;
-  const float slope = use_alibi ? slopes_dev[hh] : 0.0f;
+  const float slope = use_alibi ? slopes_dev.v[hh] : 0.0f;
   for (int n = tid; n < Nq; n += 256) s_q[n] = Q[(long)i * Nq + n];
   __syncthreads();
   bool any = false;
@@ -200,7 +205,7 @@ struct FsaArgs {
   // scores epilogue
   int block_size, tb, h, use_alibi, dense;
   const unsigned char *active;  // [tb*tb] when !dense
-  const float *slopes;          // [h] device
+  float slopes[64];             // per head, by value (no device copy, no host synchronisation)
   // output epilogue
   const float *norm;            // [slices][M] or null
   int beta;                     // EPI 2: C += acc instead of C = acc
@@ -523,27 +528,46 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
   const size_t act_bytes = sparse ? bdh_align_up((size_t)tb * tb, 256) : 0;
   const size_t sc_bytes = path == 1 ? bdh_align_up(sizeof(float) * (size_t)S * T * Tp, 256) : 0;
   const size_t nm_bytes = path == 1 ? bdh_align_up(sizeof(float) * (size_t)S * T, 256) : 0;
-  int rc = bdh_ws_reserve(ctx, q_bytes + act_bytes + 512 + sc_bytes + nm_bytes);
+  int rc = bdh_ws_reserve(ctx, q_bytes + sc_bytes + nm_bytes);
   if (rc != BDH_OK) return rc;
   char *ws = static_cast<char *>(ctx->ws);
   float *q = reinterpret_cast<float *>(ws);
-  unsigned char *active = sparse ? reinterpret_cast<unsigned char *>(ws + q_bytes) : nullptr;
-  float *slopes_dev = reinterpret_cast<float *>(ws + q_bytes + act_bytes);
-  float *scores = reinterpret_cast<float *>(ws + q_bytes + act_bytes + 512);
-  float *norm = reinterpret_cast<float *>(ws + q_bytes + act_bytes + 512 + sc_bytes);
+  float *scores = reinterpret_cast<float *>(ws + q_bytes);
+  float *norm = reinterpret_cast<float *>(ws + q_bytes + sc_bytes);
+  // The time-block mask of a sparse pattern lives in memory the context owns and is uploaded only when the
+  // pattern differs from the one already there (a model calls with the same pattern every time): no copy and
+  // no host synchronisation on the usual call.  The ALiBi slopes travel as a kernel argument.
+  unsigned char *active = nullptr;
   if (sparse) {
-    std::vector<unsigned char> m((size_t)tb * tb, 0);
-    for (int p = 0; p < n_pairs; ++p) {
-      const int r = block_pairs_host[2 * p], c = block_pairs_host[2 * p + 1];
-      if (r >= 0 && r < tb && c >= 0 && c < tb) m[(size_t)r * tb + c] = 1;  // iter_cols drops c >= total_blocks
+    std::vector<int> key;
+    key.reserve(2 * (size_t)n_pairs + 1);
+    key.push_back(tb);
+    key.insert(key.end(), block_pairs_host, block_pairs_host + 2 * (size_t)n_pairs);
+    if (!ctx->fsa_mask || ctx->fsa_mask_key != key) {
+      std::vector<unsigned char> m((size_t)tb * tb, 0);
+      for (int p = 0; p < n_pairs; ++p) {
+        const int r = block_pairs_host[2 * p], c = block_pairs_host[2 * p + 1];
+        if (r >= 0 && r < tb && c >= 0 && c < tb) m[(size_t)r * tb + c] = 1;  // iter_cols drops c >= total_blocks
+      }
+      BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));  // earlier calls may still read the old mask
+      if (ctx->fsa_mask_bytes < m.size()) {
+        if (ctx->fsa_mask) BDH_HIP_CHECK(ctx, hipFree(ctx->fsa_mask));
+        ctx->fsa_mask = nullptr;
+        ctx->fsa_mask_bytes = 0;
+        ctx->fsa_mask_key.clear();
+        if (hipMalloc(&ctx->fsa_mask, m.size()) != hipSuccess) {
+          (void)hipGetLastError();
+          return bdh_fail(ctx, BDH_E_NOMEM, "time-block mask of %zu bytes", m.size());
+        }
+        ctx->fsa_mask_bytes = m.size();
+      }
+      BDH_HIP_CHECK(ctx, hipMemcpy(ctx->fsa_mask, m.data(), m.size(), hipMemcpyHostToDevice));
+      ctx->fsa_mask_key = std::move(key);
     }
-    BDH_HIP_CHECK(ctx, hipMemcpyAsync(active, m.data(), m.size(), hipMemcpyHostToDevice, ctx->stream));
-    BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));  // m is a local buffer
+    active = static_cast<unsigned char *>(ctx->fsa_mask);
   }
-  if (alibi_slopes_host) {
-    BDH_HIP_CHECK(ctx, hipMemcpyAsync(slopes_dev, alibi_slopes_host, sizeof(float) * h, hipMemcpyHostToDevice, ctx->stream));
-    BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
-  }
+  FsaSlopes slopes_dev{};
+  if (alibi_slopes_host) memcpy(slopes_dev.v, alibi_slopes_host, sizeof(float) * h);
   hipLaunchKernelGGL(k_rotate_f32, dim3((unsigned)(S * T)), dim3(256), 0, ctx->stream, query, freqs, q, T, N, rotary);
   BDH_LAUNCH_CHECK(ctx, "k_rotate_f32");
   if (path == 1) {
@@ -552,7 +576,8 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     g.a_batch = g.b_batch = (long)T * Nq; g.c_batch = (long)T * Tp;
     g.lda = g.ldb = Nq; g.ldc = Tp; g.M = g.N = T; g.K = Nq; g.b_div = 1; g.n_slices = (int)S;
     g.block_size = block_size; g.tb = tb; g.h = h; g.use_alibi = alibi_slopes_host ? 1 : 0; g.dense = sparse ? 0 : 1;
-    g.active = active; g.slopes = slopes_dev; g.norm = nullptr;
+    g.active = active; g.norm = nullptr;
+    memcpy(g.slopes, slopes_dev.v, sizeof(g.slopes));
     // big tiles once there are enough of them to cover the chip; small ones for short sequences
     const bool big = (long)S * ((T + 255) / 256) * ((T + 255) / 256) >= 256;
     const unsigned groups = (unsigned)((S + 7) / 8);

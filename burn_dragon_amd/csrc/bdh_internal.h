@@ -7,6 +7,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 #include "../../include/bdh_mi355x.h"
 
@@ -28,6 +29,10 @@ struct bdh_ctx {
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on
   int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
+  // time-block mask of the last sparse fused_state_aligned pattern (device) and the pattern it was built from
+  void *fsa_mask = nullptr;
+  size_t fsa_mask_bytes = 0;
+  std::vector<int> fsa_mask_key;
   char err[512] = {0};
 };
 

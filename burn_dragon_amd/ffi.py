@@ -128,36 +128,58 @@ def ptr(t) -> Optional[int]:
 
 
 class Context:
-    """bdh_ctx bound to a device and a HIP stream (default: torch's current stream)."""
+    """bdh_ctx bound to a device and a HIP stream.  Without an explicit stream the context follows torch's
+    current stream: every access to `.lib` (each wrapper fetches it right before its call) re-binds the context
+    when the current stream has changed, so tensors torch allocates or fills on that stream and the library's
+    kernels stay ordered, also inside `with torch.cuda.stream(s)` and under graph capture.  A context created
+    with a stream, or given one through set_stream(..., pin=True), keeps it."""
 
     def __init__(self, device_id: int = 0, stream: Optional[int] = None):
-        self.lib = load_library()
+        self._lib = load_library()
+        self.device_id = device_id
+        self._follow = stream is None
         if stream is None:
             import torch
 
             stream = torch.cuda.current_stream(device_id).cuda_stream
         handle = c_void_p()
-        rc = self.lib.bdh_ctx_create(device_id, stream or None, ctypes.byref(handle))
+        rc = self._lib.bdh_ctx_create(device_id, stream or None, ctypes.byref(handle))
         if rc != OK:
-            raise BdhError(rc, self.lib.bdh_status_string(rc).decode() + " (bdh_ctx_create; is a HIP device present?)")
+            raise BdhError(rc, self._lib.bdh_status_string(rc).decode() + " (bdh_ctx_create; is a HIP device present?)")
         self.handle = handle
+        self._stream = stream or 0
+
+    @property
+    def lib(self):
+        if self._follow and getattr(self, "handle", None):
+            import torch
+
+            current = torch.cuda.current_stream(self.device_id).cuda_stream
+            if current != self._stream:
+                self._lib.bdh_ctx_set_stream(self.handle, current or None)
+                self._stream = current
+        return self._lib
 
     def check(self, rc: int):
         if rc != OK:
-            raise BdhError(rc, self.lib.bdh_last_error(self.handle).decode())
+            raise BdhError(rc, self._lib.bdh_last_error(self.handle).decode())
 
-    def set_stream(self, stream: int):
-        self.check(self.lib.bdh_ctx_set_stream(self.handle, stream or None))
+    def set_stream(self, stream: int, pin: bool = False):
+        """Binds the context to `stream`; with pin=True it stops following torch's current stream."""
+        self.check(self._lib.bdh_ctx_set_stream(self.handle, stream or None))
+        self._stream = stream or 0
+        if pin:
+            self._follow = False
 
     def set_option(self, name: str, value: int):
-        self.check(self.lib.bdh_ctx_set_option(self.handle, name.encode(), int(value)))
+        self.check(self._lib.bdh_ctx_set_option(self.handle, name.encode(), int(value)))
 
     def synchronize(self):
-        self.check(self.lib.bdh_ctx_synchronize(self.handle))
+        self.check(self._lib.bdh_ctx_synchronize(self.handle))
 
     def close(self):
         if getattr(self, "handle", None):
-            self.lib.bdh_ctx_destroy(self.handle)
+            self._lib.bdh_ctx_destroy(self.handle)
             self.handle = None
 
     def __del__(self):

@@ -203,3 +203,41 @@ def test_pope_step_at_the_config1_layer_shape(bda, corc):
     o_ref, r_ref = corc.recurrent_attention(corc.rotate(x, freqs, orc.POPE, 777), v, rho)
     assert rel_err(out.cpu().numpy(), o_ref) < 1e-3 and rel_err(rt.cpu().numpy(), r_ref) < 1e-3
     assert (rows.cpu().numpy() == 2 * N).all()
+
+
+def test_context_follows_torchs_current_stream(bda, corc):
+    """The wrappers launch on whatever stream torch considers current: work queued on a side stream before the
+    call (a large fill of the state) must be seen by the kernels, and the result must be ready for torch ops that
+    follow on that stream, with no device-wide synchronisation in between."""
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    rng = np.random.default_rng(5)
+    B, h, N, d = 8, 4, 2048, 256
+    x = np.maximum(rng.standard_normal((B, h, 1, N)) - 1.0, 0).astype(np.float32)
+    v = rng.standard_normal((B, 1, d)).astype(np.float32)
+    freqs = corc.build_freqs(N)
+    xt, vt, ft = (torch.from_numpy(a).to(DEV) for a in (x, v, freqs))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device=DEV)
+    ctx = ffi.default_context(0)
+    with torch.cuda.stream(side):
+        junk = torch.empty((1 << 28,), device=DEV)
+        for _ in range(4):  # a few milliseconds of fills queued ahead of the state's own fill
+            junk.fill_(1.0)
+        rho = torch.empty((B, h, N, d), device=DEV)
+        rho.fill_(0.25)  # queued on the side stream, certainly not finished when the call below returns to the host
+        out = recurrent_attention(xt, vt, rho, ft, 99, bda.RotaryEmbedding.ROPE)
+        total = out.sum()  # torch op on the same stream, right behind the kernels
+    assert ctx._stream == side.cuda_stream
+    side.synchronize()
+    q = corc.rotate(x, freqs, orc.ROPE, 99)
+    out_ref, rho_ref = corc.recurrent_attention(q, v, np.full((B, h, N, d), 0.25, np.float32))
+    assert rel_err(out.cpu().numpy(), out_ref) < 1e-3
+    assert rel_err(rho.cpu().numpy(), rho_ref) < 1e-3
+    assert abs(float(total) - float(out_ref.sum())) <= 1e-3 * np.abs(out_ref).sum()
+    # back on the default stream the context follows again
+    out2 = recurrent_attention(xt, vt, rho, ft, 100, bda.RotaryEmbedding.ROPE)
+    torch.cuda.synchronize()
+    assert ctx._stream == torch.cuda.current_stream(0).cuda_stream
+    assert np.isfinite(out2.cpu().numpy()).all()
