@@ -52,7 +52,7 @@ int bdh_fail(bdh_ctx *ctx, int status, const char *fmt, ...);
 // model_phase.hip: a decode step in two launches per layer (T = 1, f32 state, 128 <= d <= 512, N a multiple of 64)
 bool bdh_model_phase_fits(const bdh_model_config &c);
 size_t bdh_model_phase_scratch_floats(const bdh_model_config &c, int B);
-int bdh_launch_model_phases(bdh_model *m, const int64_t *tokens, int B, float *scratch, float *rho, int32_t *stamps,
+int bdh_launch_model_phases(bdh_model *m, const int64_t *tokens, int B, float *scratch, void *rho, int rho_dtype, int32_t *stamps,
                             int64_t position,
                             const int32_t *positions_dev, float **cur_final, float **dec_partial, int *G_out);
 int bdh_launch_phase_head(bdh_model *m, int B, const float *cur, const float *dec_partial, int G, float *logits,
@@ -62,7 +62,7 @@ int bdh_launch_decoder_finalize(bdh_ctx *ctx, const float *partial, int KBN, int
 
 // model_small.hip: the one-launch decode step of a small model (T = 1, f32 state)
 bool bdh_model_small_fits(const bdh_model_config &c);
-int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, float *rho, int32_t *stamps, int64_t position,
+int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, void *rho, int rho_dtype, int32_t *stamps, int64_t position,
                            const int32_t *positions_dev, float *logits, int64_t *next_tokens);
 
 // Grows ctx->ws to at least `bytes` (synchronises the stream before freeing the old one).
@@ -165,3 +165,25 @@ int bdh_launch_rho_energy(bdh_ctx *ctx, int B, int h, int N, int d, const void *
 int bdh_launch_gather_head_rows(bdh_ctx *ctx, const float *src, int h, long head_stride, long offset, int cols,
                                 float *dst);
 int bdh_launch_fill_zero_f32(bdh_ctx *ctx, float *p, long n);
+
+// Four adjacent elements of a state row, f32 or bf16 (raw 16-bit patterns; stores round to nearest even, NaN kept
+// quiet): the element access of the decode forms that keep the state in either type.
+__device__ __forceinline__ float4 bdh_rho_load4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 bdh_rho_load4(const unsigned short *p) {
+  const uint2 v = *reinterpret_cast<const uint2 *>(p);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                     __uint_as_float(v.y & 0xffff0000u));
+}
+__device__ __forceinline__ unsigned int bdh_bf16_rne(float f) {
+  unsigned int u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ void bdh_rho_store4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ void bdh_rho_store4(unsigned short *p, float4 v) {
+  uint2 o;
+  o.x = bdh_bf16_rne(v.x) | (bdh_bf16_rne(v.y) << 16);
+  o.y = bdh_bf16_rne(v.z) | (bdh_bf16_rne(v.w) << 16);
+  *reinterpret_cast<uint2 *>(p) = o;
+}

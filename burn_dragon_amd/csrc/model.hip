@@ -141,7 +141,7 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
   // per layer | kernel by kernel): tiny 77|77|112 at B=1, 84|100|145 at B=64; small 152|82|130 at B=1, 168|127|195 at
   // B=64, 323|442|478 at B=256; base 223|83|123 at B=1, 273|210|240 at B=64, 559|-|654 at B=256; large -|210|308 at
   // B=1, -|519|554 at B=16, -|1092|981 at B=33.
-  if (T == 1 && !x_tap && !viz && rho_dtype == BDH_F32 && ctx->opt_model_one_launch != 0) {
+  if (T == 1 && !x_tap && !viz && ctx->opt_model_one_launch != 0) {
     const size_t w_layer = sizeof(float) * (size_t)3 * h * N * d;
     const size_t w_bytes = w_layer * L;
     const bool small_fits = bdh_model_small_fits(c);
@@ -151,16 +151,15 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
                         (size_t)B * w_layer <= (size_t(256) << 20);
     const int b_min = w_bytes <= (size_t(8) << 20) ? 16 : 128;
     if (one_first || (!phases && small_fits && B >= b_min))
-      return bdh_launch_model_small(m, tokens, B, static_cast<float *>(rho), stamps, position, positions_dev, logits,
-                                    next_tokens);
+      return bdh_launch_model_small(m, tokens, B, rho, rho_dtype, stamps, position, positions_dev, logits, next_tokens);
     if (phases) {
       int rc2 = ensure_act(m, sizeof(float) * bdh_model_phase_scratch_floats(c, B));
       if (rc2 != BDH_OK) return rc2;
       float *scratch = static_cast<float *>(m->act);
       float *cur_final = nullptr, *dpart = nullptr;
       int G = 0;
-      rc2 = bdh_launch_model_phases(m, tokens, B, scratch, static_cast<float *>(rho), stamps, position, positions_dev,
-                                    &cur_final, &dpart, &G);
+      rc2 = bdh_launch_model_phases(m, tokens, B, scratch, rho, rho_dtype, stamps, position, positions_dev, &cur_final,
+                                    &dpart, &G);
       if (rc2 != BDH_OK) return rc2;
       if (V <= 1024)  // the last layer's second stage (:436-441) and the head (:446-449) in one launch
         return bdh_launch_phase_head(m, B, cur_final, dpart, G, logits, next_tokens);
@@ -233,6 +232,12 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
 }
 
 int bdh_model_forward_fast(bdh_model *m, const int64_t *tokens, int B, int T, int time_block_size, float *logits) {
+  return bdh_model_forward_fast_ex(m, tokens, B, T, time_block_size, nullptr, 0, 1, nullptr, 0, logits);
+}
+
+int bdh_model_forward_fast_ex(bdh_model *m, const int64_t *tokens, int B, int T, int time_block_size,
+                              const int32_t *time_pairs_host, int n_time_pairs, int latent_block_size,
+                              const uint8_t *latent_blocks_host, int n_latent_blocks, float *logits) {
   if (!m) return BDH_E_INVAL;
   bdh_ctx *ctx = m->ctx;
   if (B < 0 || T < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative batch or time");
@@ -253,17 +258,24 @@ int bdh_model_forward_fast(bdh_model *m, const int64_t *tokens, int B, int T, in
   rc = bdh_launch_embed_ln(ctx, tokens, (int64_t)M, d, V, m->w.embed, cur);  // :97-100
   if (rc != BDH_OK) return rc;
   const int block = time_block_size > 0 ? time_block_size : 1;  // plain branch: element-wise tril(-1)
+  const int lat_block = latent_block_size > 0 ? latent_block_size : 1;
+  if (time_pairs_host && time_block_size <= 0)
+    return bdh_fail(ctx, BDH_E_INVAL, "a time-block pattern belongs to the fused branch (time_block_size > 0)");
+  if (n_time_pairs < 0 || n_latent_blocks < 0 || (n_time_pairs > 0 && !time_pairs_host))
+    return bdh_fail(ctx, BDH_E_INVAL, "pattern counts do not match the pattern pointers");
   for (int l = 0; l < L; ++l) {  // :113
-    ReluLowrankParams px{B, 1, T, d, h, N, cur, m->w.encoder, nullptr, c.relu_threshold, 1, nullptr, 0, nullptr, x};
+    ReluLowrankParams px{B, 1, T, d, h, N, cur, m->w.encoder, nullptr, c.relu_threshold, lat_block, latent_blocks_host,
+                         n_latent_blocks, nullptr, x};
     rc = bdh_launch_relu_lowrank(ctx, px);  // :114-129
     if (rc != BDH_OK) return rc;
     // :131  Attention::forward: all tokens at once from position 0, row-normalised
     rc = bdh_fused_state_aligned(ctx, B, h, T, N, d, x, cur, m->freqs, c.rotary == BDH_ALIBI ? m->slopes : nullptr, block,
-                                 nullptr, 0, c.rotary, 1, attn);
+                                 time_pairs_host, n_time_pairs, c.rotary, 1, attn);
     if (rc != BDH_OK) return rc;
     rc = bdh_launch_layer_norm(ctx, (int64_t)M * h, d, attn, attn_ln);  // :132
     if (rc != BDH_OK) return rc;
-    ReluLowrankParams py{B, h, T, d, h, N, attn_ln, m->w.encoder_v, nullptr, c.relu_threshold, 1, nullptr, 0, x, xy};
+    ReluLowrankParams py{B, h, T, d, h, N, attn_ln, m->w.encoder_v, nullptr, c.relu_threshold, lat_block, latent_blocks_host,
+                         n_latent_blocks, x, xy};
     rc = bdh_launch_relu_lowrank(ctx, py);  // :134-151
     if (rc != BDH_OK) return rc;
     rc = bdh_launch_decoder_residual(ctx, B, T, h, N, d, xy, m->w.decoder, cur);  // :153-162

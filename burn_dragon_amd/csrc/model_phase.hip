@@ -29,7 +29,7 @@ struct PhaseArgs {
   float *attn_partial;        // [B][h][N/64][d]
   float *dec_partial_out;     // [G][B][d], G = h * N / 64
   const float *enc, *enc_v, *dec, *freqs;
-  float *rho;                 // this layer's state [B][h][Nq][d]
+  void *rho;                  // this layer's state [B][h][Nq][d], f32 or bf16
   int32_t *stamps;            // this layer's stamps [B][h][N] or null
   const int32_t *pos_dev;
   long pos;
@@ -97,7 +97,7 @@ __device__ __forceinline__ float chain_spans(const float *s_in, const float *wv,
 }
 
 // ---- phase A ---------------------------------------------------------------------------------------------------
-template <int NW>
+template <int NW, typename RhoT>
 __global__ __launch_bounds__(NW * 64) void k_layer_phase_a(PhaseArgs a) {
   constexpr int VPL = (NW + 3) / 4;  // float4 per lane per state row: columns (j*64 + lane)*4
   constexpr int kFlight = 64 / NW < 16 ? 64 / NW : 16;  // state rows in flight per wave: all of its share of a dense block
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(NW * 64) void k_layer_phase_a(PhaseArgs a) {
   // and takes every NW-th entry of it.
   const bool alibi = a.rotary == BDH_ALIBI, pope = a.rotary == BDH_POPE;
   const int Nq = pope ? 2 * N : N;
-  float *rho = a.rho + ((long)b * h + hh) * (long)Nq * d;
+  RhoT *rho = static_cast<RhoT *>(a.rho) + ((long)b * h + hh) * (long)Nq * d;
   int32_t *st = a.stamps ? a.stamps + ((long)b * h + hh) * N : nullptr;
   const bool lazy = alibi && st != nullptr;
   const float dec = alibi ? a.decay[hh] : 1.0f;
@@ -240,11 +240,11 @@ __global__ __launch_bounds__(NW * 64) void k_layer_phase_a(PhaseArgs a) {
       }
 #pragma unroll
       for (int u = 0; u < kFlight; ++u) {
-        const float *row = rho + (row_base + src[u]) * d;
+        const RhoT *row = rho + (row_base + src[u]) * d;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
           const int c = (j * 64 + lane) * 4;
-          rv[u][j] = *reinterpret_cast<const float4 *>(row + (c < d ? c : 0));
+          rv[u][j] = bdh_rho_load4(row + (c < d ? c : 0));
         }
       }
 #pragma unroll
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(NW * 64) void k_layer_phase_a(PhaseArgs a) {
         const float q_src = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(q_l), lu));
         const float scale = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(scale_l), lu));
         const float qn = ok[u] ? q_src : 0.0f;
-        float *row = rho + (row_base + src[u]) * d;
+        RhoT *row = rho + (row_base + src[u]) * d;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
           const int c = (j * 64 + lane) * 4;
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(NW * 64) void k_layer_phase_a(PhaseArgs a) {
           if (alibi) {  // src/model/bdh.rs:299-301
             e.x *= dec; e.y *= dec; e.z *= dec; e.w *= dec;
           }
-          if (ok[u] && c < d) *reinterpret_cast<float4 *>(row + c) = e;
+          if (ok[u] && c < d) bdh_rho_store4(row + c, e);
         }
       }
     }
@@ -483,8 +483,8 @@ size_t bdh_model_phase_scratch_floats(const bdh_model_config &c, int B) {
 
 // On return cur_final points at the buffer holding the last layer's input and dec_partial at its encoder partials
 // [G][B][d]: the caller runs the encoder's second stage and the head.
-int bdh_launch_model_phases(bdh_model *m, const int64_t *tokens, int B, float *scratch, float *rho, int32_t *stamps,
-                            int64_t position,
+int bdh_launch_model_phases(bdh_model *m, const int64_t *tokens, int B, float *scratch, void *rho, int rho_dtype,
+                            int32_t *stamps, int64_t position,
                             const int32_t *positions_dev, float **cur_final, float **dec_partial, int *G_out) {
   bdh_ctx *ctx = m->ctx;
   const bdh_model_config &c = m->cfg;
@@ -528,15 +528,23 @@ int bdh_launch_model_phases(bdh_model *m, const int64_t *tokens, int B, float *s
     a.cur_in = cur[in];
     a.cur_out = l == 0 ? cur[0] : cur[in ^ 1];
     a.dec_partial = l > 0 ? dpart : nullptr;
-    a.rho = rho + (size_t)l * B * h * Nq * d;
+    a.rho = static_cast<char *>(rho) + (size_t)l * B * h * Nq * d * (rho_dtype == BDH_BF16 ? 2 : 4);
     a.stamps = stamps ? stamps + (size_t)l * B * h * N : nullptr;
 #define BDH_PHASE(K_, NW_) hipLaunchKernelGGL((K_<NW_>), dim3((unsigned)grid), dim3(NW_ * 64), 0, ctx->stream, a)
-    if (nw <= 2) BDH_PHASE(k_layer_phase_a, 2); else if (nw <= 4) BDH_PHASE(k_layer_phase_a, 4); else BDH_PHASE(k_layer_phase_a, 8);
+#define BDH_PHASE_A(NW_)                                                                                           \
+  do {                                                                                                             \
+    if (rho_dtype == BDH_BF16)                                                                                     \
+      hipLaunchKernelGGL((k_layer_phase_a<NW_, unsigned short>), dim3((unsigned)grid), dim3(NW_ * 64), 0, ctx->stream, a); \
+    else                                                                                                           \
+      hipLaunchKernelGGL((k_layer_phase_a<NW_, float>), dim3((unsigned)grid), dim3(NW_ * 64), 0, ctx->stream, a);   \
+  } while (0)
+    if (nw <= 2) BDH_PHASE_A(2); else if (nw <= 4) BDH_PHASE_A(4); else BDH_PHASE_A(8);
     BDH_LAUNCH_CHECK(ctx, "k_layer_phase_a");
     if (l > 0) in ^= 1;  // phase A has applied the pending second stage: the layer's input is now cur[in ^ 1]
     if (nw <= 2) BDH_PHASE(k_layer_phase_b, 2); else if (nw <= 4) BDH_PHASE(k_layer_phase_b, 4); else BDH_PHASE(k_layer_phase_b, 8);
     BDH_LAUNCH_CHECK(ctx, "k_layer_phase_b");
 #undef BDH_PHASE
+#undef BDH_PHASE_A
   }
   *cur_final = cur[in];
   *dec_partial = dpart;

@@ -22,7 +22,7 @@ constexpr int kMaxCols = 2048;  // h * N
 struct SmallArgs {
   const int64_t *tokens;
   const float *embed, *enc, *enc_v, *dec, *lm_head, *freqs;
-  float *rho;
+  void *rho;  // f32 or bf16 elements
   int32_t *stamps;
   const int32_t *pos_dev;
   long pos;
@@ -30,7 +30,7 @@ struct SmallArgs {
   int64_t *next;
   int B, d, h, N, V, L, rotary;
   float thr;
-  size_t rho_layer_stride;    // floats
+  size_t rho_layer_stride;    // elements
   size_t stamps_layer_stride;  // entries
   float decay[16], log_decay[16];
 };
@@ -128,7 +128,7 @@ __device__ __forceinline__ float matvec_cols(const float *s_in, int K, const flo
 
 // LPR: lanes per state row, four adjacent columns each (d <= 4 * LPR); a wave instruction covers 64 / LPR rows and
 // 8 such groups of rows are in flight per wave
-template <int LPR>
+template <int LPR, typename RhoT>
 __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
   constexpr int RPI = 64 / LPR;  // rows per instruction
   constexpr int kFlight = 8;
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
     // recurrent attention with value = cur (src/model/bdh.rs:353-359, 232-306): readout with the old rows,
     // then the rank-1 update (and the ALiBi decay); only visited rows are touched
     {
-      float *rho = a.rho + (size_t)l * a.rho_layer_stride + (size_t)b * srows * d;
+      RhoT *rho = static_cast<RhoT *>(a.rho) + (size_t)l * a.rho_layer_stride + (size_t)b * srows * d;
       int32_t *st = a.stamps ? a.stamps + (size_t)l * a.stamps_layer_stride + (size_t)b * cols : nullptr;
       const bool lazy = alibi && st != nullptr;
       const float dec = alibi ? a.decay[hh_w] : 1.0f;
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
           // issued back to back
 #pragma unroll
           for (int u = 0; u < kFlight; ++u)
-            rv[u] = *reinterpret_cast<const float4 *>(rho + (size_t)(row0 + base + src[u]) * d + coff);
+            rv[u] = bdh_rho_load4(rho + (size_t)(row0 + base + src[u]) * d + coff);
 #pragma unroll
           for (int u = 0; u < kFlight; ++u) {
             const float q_src = __shfl(q_l, src[u], 64);
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(kThreads) void k_model_step_small(SmallArgs a) {
               r[j] = e;
             }
             if (ok[u] && has_c)
-              *reinterpret_cast<float4 *>(rho + (size_t)(row0 + base + src[u]) * d + coff) = make_float4(r[0], r[1], r[2], r[3]);
+              bdh_rho_store4(rho + (size_t)(row0 + base + src[u]) * d + coff, make_float4(r[0], r[1], r[2], r[3]));
           }
         }
         if (lazy && touch_l) st[r_l] = (int32_t)min(pos + 1, 0x7fffffffL);
@@ -374,7 +374,8 @@ bool bdh_model_small_fits(const bdh_model_config &c) {
   return true;
 }
 
-int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, float *rho, int32_t *stamps, int64_t position,
+int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, void *rho, int rho_dtype, int32_t *stamps,
+                           int64_t position,
                            const int32_t *positions_dev, float *logits, int64_t *next_tokens) {
   bdh_ctx *ctx = m->ctx;
   const bdh_model_config &c = m->cfg;
@@ -408,12 +409,20 @@ int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, float *rh
       a.decay[i] = expf(-m->slopes[i]);                 // src/model/attention.rs:181-186
       a.log_decay[i] = (float)log((double)a.decay[i]);  // of the rounded factor, as the lazy state step
     }
+#define BDH_SMALL(LPR)                                                                                              \
+  do {                                                                                                               \
+    if (rho_dtype == BDH_BF16)                                                                                       \
+      hipLaunchKernelGGL((k_model_step_small<LPR, unsigned short>), dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a); \
+    else                                                                                                             \
+      hipLaunchKernelGGL((k_model_step_small<LPR, float>), dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);     \
+  } while (0)
   if (a.d <= 64)
-    hipLaunchKernelGGL(k_model_step_small<16>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
+    BDH_SMALL(16);
   else if (a.d <= 128)
-    hipLaunchKernelGGL(k_model_step_small<32>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
+    BDH_SMALL(32);
   else
-    hipLaunchKernelGGL(k_model_step_small<64>, dim3((unsigned)B), dim3(kThreads), 0, ctx->stream, a);
+    BDH_SMALL(64);
+#undef BDH_SMALL
   BDH_LAUNCH_CHECK(ctx, "k_model_step_small");
   return BDH_OK;
 }

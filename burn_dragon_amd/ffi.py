@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import sys
 from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
 from typing import Optional
 
@@ -28,7 +29,7 @@ EXPORTS = [
     "bdh_model_state_bytes", "bdh_model_forward", "bdh_model_forward_ex", "bdh_advance_positions",
     "bdh_sample_top_k", "bdh_recurrent_attention_lazy_alibi", "bdh_alibi_materialize", "bdh_model_forward_lazy",
     "bdh_rho_energy", "bdh_model_forward_viz", "bdh_rotate",
-    "bdh_model_forward_fast", "bdh_state_step_noalloc", "bdh_probe_chunks",
+    "bdh_model_forward_fast", "bdh_model_forward_fast_ex", "bdh_state_step_noalloc", "bdh_probe_chunks",
 ]
 
 
@@ -106,6 +107,7 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_alibi_materialize.argtypes = [P, c_int, c_int, c_int, c_int, c_int64, P, P, P, c_int, P]
     lib.bdh_model_forward_lazy.argtypes = [P, P, c_int, c_int, P, c_int, P, c_int64, P, P, P, P]
     lib.bdh_model_forward_fast.argtypes = [P, P, c_int, c_int, c_int, P]
+    lib.bdh_model_forward_fast_ex.argtypes = [P, P, c_int, c_int, c_int, P, c_int, c_int, P, c_int, P]
     lib.bdh_rotate.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, c_int64, P, P]
     lib.bdh_rho_energy.argtypes = [P, c_int, c_int, c_int, c_int, P, c_int, P, c_int64, P, P, P]
     lib.bdh_model_forward_viz.argtypes = [P, P, c_int, c_int, P, c_int, P, c_int64, P, P, P, P, P]
@@ -151,7 +153,7 @@ class Context:
 
     @property
     def lib(self):
-        if self._follow and getattr(self, "handle", None):
+        if self._follow and getattr(self, "handle", None) and not sys.is_finalizing():
             import torch
 
             current = torch.cuda.current_stream(self.device_id).cuda_stream
@@ -179,7 +181,8 @@ class Context:
 
     def close(self):
         if getattr(self, "handle", None):
-            self._lib.bdh_ctx_destroy(self.handle)
+            if not sys.is_finalizing():  # at interpreter exit the HIP runtime may already be gone
+                self._lib.bdh_ctx_destroy(self.handle)
             self.handle = None
 
     def __del__(self):

@@ -7,6 +7,7 @@ forward_with_state is one call of bdh_model_forward.
 from __future__ import annotations
 
 import ctypes
+import sys
 from typing import Optional
 
 import numpy as np
@@ -84,8 +85,9 @@ class BDH:
 
     def __del__(self):
         try:
-            if getattr(self, "handle", None):
-                self.ctx.lib.bdh_model_destroy(self.handle)
+            # at interpreter exit the HIP runtime may already be gone: the process is about to release everything
+            if getattr(self, "handle", None) and not sys.is_finalizing():
+                self.ctx._lib.bdh_model_destroy(self.handle)  # not .lib: no stream lookup while tearing down
                 self.handle = None
         except Exception:
             pass
@@ -157,16 +159,24 @@ class BDH:
     def forward_fast(self, tokens: torch.Tensor) -> torch.Tensor:
         """src/model/bdh.rs:96-168: the stateless forward over all tokens at once (the form the reference
         trains with): Attention::forward in place of the recurrent state.  tokens [B,T] -> logits [B,T,V]."""
-        if self.kernel.enabled and (self.kernel.block_sparse.latent.is_sparse() or
-                                    self.kernel.block_sparse.time.is_sparse()):
-            raise NotImplementedError("forward_fast takes dense block patterns (build_model_config makes no others); "
-                                      "sparse patterns are available through kernel.relu_lowrank / linear_attention")
         tokens = tokens.to(self.device, torch.int64).contiguous()
         B, T = tokens.shape
         logits = torch.empty((B, T, self.vocab_size), device=self.device, dtype=torch.float32)
-        block = max(self.kernel.block_sparse.time.block_size, 1) if self.kernel.enabled else 0
-        self.ctx.check(self.ctx.lib.bdh_model_forward_fast(self.handle, tokens.data_ptr(), B, T, block,
-                                                           logits.data_ptr()))
+        sparse = self.kernel.block_sparse
+        if not self.kernel.enabled:  # plain branch: the patterns are not consulted (src/model/bdh.rs:114-151)
+            self.ctx.check(self.ctx.lib.bdh_model_forward_fast(self.handle, tokens.data_ptr(), B, T, 0, logits.data_ptr()))
+            return logits
+        block = max(sparse.time.block_size, 1)
+        pairs, n_pairs = None, 0
+        if sparse.time.is_sparse():
+            flat = np.array(sorted(sparse.time.active_pairs), dtype=np.int32).reshape(-1, 2)
+            pairs, n_pairs = np.ascontiguousarray(flat), flat.shape[0]
+            if n_pairs == 0:
+                pairs = np.zeros((1, 2), np.int32)  # a valid pointer: an empty pattern is still a sparse one
+        blocks = sparse.latent.block_bytes(self.latent) if sparse.latent.is_sparse() else None
+        self.ctx.check(self.ctx.lib.bdh_model_forward_fast_ex(
+            self.handle, tokens.data_ptr(), B, T, block, ffi.ptr(pairs), n_pairs, max(sparse.latent.block_size, 1),
+            blocks, 0 if blocks is None else len(blocks), logits.data_ptr()))
         return logits
 
     def generate(self, indices: torch.Tensor, max_new_tokens: int, temperature: float = 1.0,

@@ -331,6 +331,15 @@ int bdh_model_forward_ex(bdh_model *model, const int64_t *tokens, int B, int T, 
 int bdh_model_forward_fast(bdh_model *model, const int64_t *tokens, int B, int T, int time_block_size,
                            float *logits);
 
+/* bdh_model_forward_fast with the block patterns of FusedKernelConfig.block_sparse (src/model/bdh.rs:111,
+ * 114-129, 134-151 and src/model/attention.rs:142-152): the time-block pairs go to the attention of every
+ * layer as in bdh_fused_state_aligned (block_pairs_host [n_time_pairs][2] of (row, col), NULL = dense lower
+ * triangle; needs time_block_size > 0), the latent block mask to both projections of every layer as in
+ * bdh_relu_lowrank (one byte per block of latent_block_size neurons, NULL = dense). */
+int bdh_model_forward_fast_ex(bdh_model *model, const int64_t *tokens, int B, int T, int time_block_size,
+                              const int32_t *time_pairs_host, int n_time_pairs, int latent_block_size,
+                              const uint8_t *latent_blocks_host, int n_latent_blocks, float *logits);
+
 /* positions_dev[b] = saturating(positions_dev[b] + delta): the device-side form of
  * `state.position += T` (src/model/bdh.rs:445). */
 int bdh_advance_positions(bdh_ctx *ctx, int32_t *positions_dev, int B, int delta);

@@ -314,10 +314,13 @@ def forward_with_state(shape: BDHShape, w: BDHWeights, tokens, state: ModelState
     return np.matmul(cur.reshape(B * T, d), w.lm_head).reshape(B, T, shape.vocab_size)  # :446-449
 
 
-def forward_fast(shape: BDHShape, w: BDHWeights, tokens, fused: bool = False, time_block: int = 64):
+def forward_fast(shape: BDHShape, w: BDHWeights, tokens, fused: bool = False, time_block: int = 64,
+                 time_pairs=None, latent_block: int = 1, latent_active=None):
     """src/model/bdh.rs:96-168, numpy statement: the stateless forward over all tokens at once, a
     composition of relu_lowrank, Attention::forward (plain branch) or fused_state_aligned (fused branch),
-    layer_norm and two matmuls.  tokens [B,T] ints -> logits [B,T,V].  The parts are pinned (see the C
+    layer_norm and two matmuls.  tokens [B,T] ints -> logits [B,T,V].  The fused branch hands the latent
+    block pattern to both projections and the time-block pattern to the attention (:111, :114-151,
+    src/model/attention.rs:142-152); the plain branch consults neither.  The parts are pinned (see the C
     file's header); the reference itself checks only the shape of the result (tests/model_paths.rs:48,81),
     so the composition as a whole is "parity unpinned"."""
     dtype = w.encoder.dtype
@@ -330,13 +333,14 @@ def forward_fast(shape: BDHShape, w: BDHWeights, tokens, fused: bool = False, ti
     if shape.rotary == ALIBI:
         slopes = default_alibi_slopes(h, dtype) if shape.alibi_slopes is None else np.asarray(shape.alibi_slopes, dtype)
     for _ in range(shape.n_layer):
-        x = relu_lowrank(cur, w.encoder, None, shape.relu_threshold)  # :114-129
+        lat = dict(block_size=latent_block, active_blocks=latent_active) if fused else {}
+        x = relu_lowrank(cur, w.encoder, None, shape.relu_threshold, **lat)  # :114-129
         if fused:  # :131, src/model/attention.rs:142-152
-            attn = fused_state_aligned(x, cur[:, 0], freqs, slopes, time_block, shape.rotary)
+            attn = fused_state_aligned(x, cur[:, 0], freqs, slopes, time_block, shape.rotary, time_pairs)
         else:  # src/model/attention.rs:154-174
             attn = attention_forward(x, cur[:, 0], freqs, slopes, shape.rotary, True)
         attn = layer_norm(attn.astype(dtype))  # :132
-        y = relu_lowrank(attn, w.encoder_v, None, shape.relu_threshold)  # :134-151
+        y = relu_lowrank(attn, w.encoder_v, None, shape.relu_threshold, **lat)  # :134-151
         xy = x * y
         mixed = np.swapaxes(xy, 1, 2).reshape(B * T, h * N)  # :156-160
         mlp = layer_norm(np.matmul(mixed, w.decoder).reshape(B, 1, T, d))  # :162-164

@@ -119,6 +119,9 @@ extern "C" {
         next_tokens: *mut i64, x_tap: *mut f32) -> c_int;
     pub fn bdh_model_forward_fast(model: *mut bdh_model, tokens: *const i64, b: c_int, t: c_int,
         time_block_size: c_int, logits: *mut f32) -> c_int;
+    pub fn bdh_model_forward_fast_ex(model: *mut bdh_model, tokens: *const i64, b: c_int, t: c_int,
+        time_block_size: c_int, time_pairs_host: *const i32, n_time_pairs: c_int, latent_block_size: c_int,
+        latent_blocks_host: *const u8, n_latent_blocks: c_int, logits: *mut f32) -> c_int;
     pub fn bdh_advance_positions(ctx: *mut bdh_ctx, positions_dev: *mut i32, b: c_int,
         delta: c_int) -> c_int;
     pub fn bdh_recurrent_attention_lazy_alibi(ctx: *mut bdh_ctx, b: c_int, h: c_int, t: c_int, n: c_int,

@@ -252,6 +252,48 @@ def test_forward_fast_long_sequence_on_the_matrix_cores(bda):
         assert rel_err(got, want) < 1e-3
 
 
+@pytest.mark.parametrize("T", [12, 160])
+def test_forward_fast_with_sparse_block_patterns(bda, T):
+    """FusedKernelConfig.block_sparse with a sparse latent pattern (src/kernel/block_sparse.rs:25-36) and a sparse
+    time-block pattern (:84-95) through forward_fast (src/model/bdh.rs:111-151): the latent mask reaches both
+    projections, the pair list the attention, for the row kernel (T = 12) and the matrix-core form (T = 160).
+    A pattern naming every causal pair and every latent block gives the dense result
+    (tests/fused_kernel_tests.rs:108); with the fused kernels off the patterns are not consulted."""
+    from burn_dragon_amd.kernel import BlockPattern1d, BlockPattern2d, BlockSparseConfig
+
+    cfg = bda.BDHConfig(n_layer=2, n_embd=32, n_head=2, mlp_internal_dim_multiplier=8, vocab_size=64, dropout=0.0)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse("rope"))
+    cfg.fused_kernels.enabled = True
+    N = cfg.latent_per_head()  # 128
+    lat_block, time_block = 16, 4 if T < 64 else 32
+    tb = -(-T // time_block)
+    tokens = np.random.default_rng(5).integers(0, 64, (2, T))
+    latent_active = [0, 2, 3, 6]
+    pairs = {(r, c) for r in range(tb) for c in range(r + 1) if (r + c) % 3 != 1} | {(0, 0)}
+    cfg.fused_kernels.block_sparse = BlockSparseConfig(BlockPattern1d.from_blocks(lat_block, latent_active),
+                                                       BlockPattern2d.from_pairs(time_block, pairs))
+    shape, w, model = _model_pair(bda, cfg, seed=41)
+    got = model.forward_fast(torch.from_numpy(tokens)).cpu().numpy()
+    want = orc.forward_fast(shape, w, tokens, fused=True, time_block=time_block, time_pairs=pairs,
+                            latent_block=lat_block, latent_active=latent_active)
+    assert rel_err(got, want) < 1e-3
+    dense_ref = orc.forward_fast(shape, w, tokens, fused=True, time_block=time_block)
+    assert rel_err(dense_ref, want) > 1e-2  # the patterns matter at this size
+    # every causal pair and every latent block named explicitly: the dense result
+    cfg.fused_kernels.block_sparse = BlockSparseConfig(
+        BlockPattern1d.from_blocks(lat_block, range(N // lat_block)),
+        BlockPattern2d.from_pairs(time_block, {(r, c) for r in range(tb) for c in range(r + 1)}))
+    _, _, model_all = _model_pair(bda, cfg, seed=41)
+    assert rel_err(model_all.forward_fast(torch.from_numpy(tokens)).cpu().numpy(), dense_ref) < 1e-3
+    # the plain branch ignores the patterns
+    cfg.fused_kernels.block_sparse = BlockSparseConfig(BlockPattern1d.from_blocks(lat_block, latent_active),
+                                                       BlockPattern2d.from_pairs(time_block, pairs))
+    cfg.fused_kernels.enabled = False
+    shape_p, w_p, model_p = _model_pair(bda, cfg, seed=41)
+    assert rel_err(model_p.forward_fast(torch.from_numpy(tokens)).cpu().numpy(),
+                   orc.forward_fast(shape_p, w_p, tokens, fused=False)) < 1e-3
+
+
 def test_batched_decode_step_takes_the_split_k_encoder(bda, corc):
     """24+ sequences decoding together: the encoder E runs as a split-K product on the f32 matrix cores (the
     weights are streamed once); logits against the oracle and against the VALU kernel."""
@@ -487,6 +529,66 @@ def test_two_launch_layer_decode_step(bda, corc, rotary, lazy, d, h, mult, L, V)
     torch.cuda.synchronize()
     assert rel_err(s_fused.storage.cpu().numpy(), rho_ref) < 1e-3
     assert rel_err(s_fused.storage.cpu().numpy(), s_ref.storage.cpu().numpy()) < 1e-5
+    if lazy:
+        assert torch.equal(s_fused.stamps, s_ref.stamps)
+
+
+@pytest.mark.parametrize("rotary,lazy", [("rope", False), ("pope", False), ("alibi", False), ("alibi", True)])
+@pytest.mark.parametrize("form,d,h,mult,L,V", [("one-launch", 128, 4, 4, 3, 69), ("one-launch", 256, 8, 8, 2, 256),
+                                              ("two-launch-layer", 256, 4, 16, 2, 256),
+                                              ("two-launch-layer", 192, 3, 4, 3, 69)])
+def test_fused_decode_forms_with_bf16_state(bda, corc, form, rotary, lazy, d, h, mult, L, V):
+    """The one-launch step and the two-launch layer with the state stored in bf16 (f32 arithmetic, one rounding per
+    stored element per token, like the kernel-by-kernel bf16 step): logits against the f32 oracle within the 2e-2
+    allowed for a bf16 state, and against the kernel-by-kernel bf16 step, where only summation trees differ (the
+    inputs of a rounding can differ in their last bits, so a few stored elements may land one bf16 step apart)."""
+    from burn_dragon_amd import ffi
+
+    cfg = bda.BDHConfig(n_layer=L, n_embd=d, n_head=h, mlp_internal_dim_multiplier=mult, vocab_size=V, dropout=0.0)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.parse(rotary))
+    shape = _shape_from_cfg(cfg)
+    w = orc.init_weights(shape, seed=d + h)
+    weights = {"embed": w.embed, "encoder": w.encoder, "encoder_v": w.encoder_v, "decoder": w.decoder, "lm_head": w.lm_head}
+    fused = bda.BDH(cfg, DEV, weights=weights, alibi_lazy=lazy, rho_dtype=ffi.BF16)
+    ref = bda.BDH(cfg, DEV, weights=weights, alibi_lazy=lazy, rho_dtype=ffi.BF16)
+    B, T0, steps = 3, 5, 4
+    rng = np.random.default_rng(7 * d + h)
+    prompt = rng.integers(0, V, (B, T0))
+    rho_ref = np.zeros((L, B, h, fused.latent_q, d), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, prompt, rho_ref, 0, sparse_state=False)
+    s_fused, s_ref = fused.init_state(), ref.init_state()
+    ctx = bda.ffi.default_context(0)
+    fused.forward_with_state(torch.from_numpy(prompt), s_fused)
+    ref.forward_with_state(torch.from_numpy(prompt), s_ref)
+    assert s_fused.storage.dtype == torch.bfloat16
+    feed = logits_ref[:, -1].argmax(-1)
+    for step in range(steps):
+        tok = feed.reshape(B, 1)
+        logits_ref, pos, _, _ = corc.forward_with_state(shape, w, tok, rho_ref, pos, sparse_state=False)
+        try:
+            ctx.set_option("model.one_launch", 2 if form == "one-launch" else 1)
+            got, nxt = fused.forward_with_state(torch.from_numpy(tok), s_fused, want_next=True)
+            ctx.set_option("model.one_launch", 0)
+            kbk = ref.forward_with_state(torch.from_numpy(tok), s_ref)
+        finally:
+            ctx.set_option("model.one_launch", 1)
+        torch.cuda.synchronize()
+        got_np = got.cpu().numpy()
+        assert rel_err(got_np, logits_ref) < 2e-2, f"step {step} against the oracle"
+        assert rel_err(got_np, kbk.cpu().numpy()) < 2e-3, f"step {step} against the kernel-by-kernel step"
+        assert not np.array_equal(got_np, kbk.cpu().numpy()), "the fused form was not taken"
+        assert np.array_equal(nxt.cpu().numpy(), got_np[:, 0].argmax(-1))
+        feed = logits_ref[:, -1].argmax(-1)
+    fused.materialize_state(s_fused)
+    ref.materialize_state(s_ref)
+    torch.cuda.synchronize()
+    assert rel_err(s_fused.storage.float().cpu().numpy(), rho_ref) < 2e-2
+    # one bf16 step of the largest element is 2^-8 of it; an element that landed a step apart can drift by another
+    # step at a later token, so the bound is one step per decode step, and few elements may differ at all
+    err_forms = rel_err(s_fused.storage.float().cpu().numpy(), s_ref.storage.float().cpu().numpy())
+    assert err_forms < steps * 2.0 ** -8, err_forms
+    differing = (s_fused.storage != s_ref.storage).float().mean().item()
+    assert differing < 0.02, f"{differing:.4f} of the stored elements differ between the forms"
     if lazy:
         assert torch.equal(s_fused.stamps, s_ref.stamps)
 
