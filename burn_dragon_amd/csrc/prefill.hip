@@ -445,12 +445,14 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
 // ====================================================================================
 
 // The k loop of k_gemm_direct as a function: acc += A[0..255, k] * B[0..255, k] over K (a multiple of 64);
-// A_rows / B_rows point at the first row of the 256-row operand panels.  Ends with every wave past its last
-// LDS read.  SAME: B is A (a diagonal score tile), loaded once.
+// A_rows / B_rows point at the first row of the 256-row operand panels, whose 64 columns of k-tile t start
+// t * a_kstride (b_kstride) elements further on (64 for a plain row-major operand; a panel stored tile by tile,
+// [k / 64][row][64], has row stride 64 and the tile size as the k-tile stride).  Ends with every wave past its
+// last LDS read.  SAME: B is A (a diagonal score tile), loaded once.
 template <bool SAME>
 __device__ __forceinline__ void direct_mainloop(f32x16 (&acc)[4][2], const unsigned short *A_rows, long lda,
-                                                const unsigned short *B_rows, long ldb, int K,
-                                                unsigned short *s_dyn, int wave, int lane) {
+                                                long a_kstride, const unsigned short *B_rows, long ldb,
+                                                long b_kstride, int K, unsigned short *s_dyn, int wave, int lane) {
   constexpr int TILE = 256 * 64;
   constexpr int BUF = 2 * TILE;
   const int wm = wave >> 2, wn = wave & 3;
@@ -465,9 +467,11 @@ __device__ __forceinline__ void direct_mainloop(f32x16 (&acc)[4][2], const unsig
 #define BDH_ISSUE(buf, k0)                                                                                          \
   _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                                   \
     const int bi = c * 8 + wave;                                                                                    \
-    __builtin_amdgcn_global_load_lds((gptr_t)(pa[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + bi * 512), 16, 0, 0);     \
+    __builtin_amdgcn_global_load_lds((gptr_t)(pa[c] + ((k0) >> 6) * a_kstride),                                      \
+                                     (lptr_t)(s_dyn + (buf)*BUF + bi * 512), 16, 0, 0);                             \
     if (!SAME)                                                                                                      \
-      __builtin_amdgcn_global_load_lds((gptr_t)(pb[c] + (k0)), (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, 0); \
+      __builtin_amdgcn_global_load_lds((gptr_t)(pb[c] + ((k0) >> 6) * b_kstride),                                    \
+                                       (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, 0);                    \
   }
   BDH_ISSUE(0, 0)
   __builtin_amdgcn_s_waitcnt(0);
@@ -514,9 +518,9 @@ __device__ __forceinline__ void lds_barrier() {
 #define BDH_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
 struct ChunkOutArgs {
-  const unsigned short *Q;   // [S][Tc][N] rotated activations of this pass
+  const unsigned short *Q;   // [S][N/64][Tc][64] rotated activations of this pass, Tc = 256 nc
   long q_slice;
-  const unsigned short *P;   // [slot][S][256][N]: bf16(rho_c)^T, slot c = the state before chunk c
+  const unsigned short *P;   // [slot][S][N/64][256][64]: bf16(rho_c)^T, slot c = the state before chunk c
   long p_slot, p_slice;
   const unsigned short *Vt;  // [B][256][ldv]: V^T of this pass
   long vt_batch;
@@ -540,7 +544,10 @@ __global__ __launch_bounds__(512) void k_chunk_out(ChunkOutArgs g) {
   const int c = g.nc - 1 - r % g.nc;  // later chunks first: they all have a state term
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 2, wn = wave & 3;
-  const unsigned short *Qc = g.Q + (long)slice * g.q_slice + (long)c * 256 * g.N;
+  // Q [slice][N/64][Tc][64] and P [slot][slice][N/64][256][64]: operand panels stored k-tile by k-tile, so that a
+  // k-step of a panel is 32 KiB of consecutive bytes (and so that the state update writes whole strips)
+  const unsigned short *Qc = g.Q + (long)slice * g.q_slice + (long)c * 256 * 64;
+  const long q_kstride = (long)g.nc * 256 * 64, p_kstride = 256 * 64;
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -551,7 +558,7 @@ __global__ __launch_bounds__(512) void k_chunk_out(ChunkOutArgs g) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // 1. S = Q_c Q_c^T
-  direct_mainloop<true>(acc, Qc, g.N, Qc, g.N, g.N, s_dyn, wave, lane);
+  direct_mainloop<true>(acc, Qc, 64, q_kstride, Qc, 64, q_kstride, g.N, s_dyn, wave, lane);
 
   // 2. tril(-1), rounded to bf16, into LDS as the A operand of S V (the operand buffers are free now)
 #pragma unroll
@@ -604,10 +611,10 @@ __global__ __launch_bounds__(512) void k_chunk_out(ChunkOutArgs g) {
   // 4. out += Q_c bf16(rho_c)   (+ Q_0 times the rounding remainder of a carried state)
   if (c > 0 || g.has_state) {
     const unsigned short *Pc = g.P + (long)c * g.p_slot + (long)slice * g.p_slice;
-    direct_mainloop<false>(acc, Qc, g.N, Pc, g.N, g.N, s_dyn, wave, lane);
+    direct_mainloop<false>(acc, Qc, 64, q_kstride, Pc, 64, p_kstride, g.N, s_dyn, wave, lane);
     if (c == 0 && g.lo_slot >= 0) {
       const unsigned short *Pl = g.P + (long)g.lo_slot * g.p_slot + (long)slice * g.p_slice;
-      direct_mainloop<false>(acc, Qc, g.N, Pl, g.N, g.N, s_dyn, wave, lane);
+      direct_mainloop<false>(acc, Qc, 64, q_kstride, Pl, 64, p_kstride, g.N, s_dyn, wave, lane);
     }
   }
 
@@ -628,86 +635,133 @@ __global__ __launch_bounds__(512) void k_chunk_out(ChunkOutArgs g) {
 struct StateUpdArgs {
   const unsigned short *X;   // x bf16, token 0 of this pass; rows of N
   long x_slice;
-  unsigned short *Q;         // [S][Tc][N] out: bf16(rope(x))
+  unsigned short *Q;         // [S][N/64][Tc][64] out: bf16(rope(x))
   long q_slice;
-  const unsigned short *Vt;  // [B][256][ldv]
+  const unsigned short *Vf;  // [B][Tc/64][8][4][64][8]: V in B-fragment order (k_v_fragments), batch stride vt_batch
   long vt_batch;
   const float *freqs;        // [N]
   float *rho;                // [S][N][256] in/out
-  unsigned short *P;         // [slot][S][256][N]
+  unsigned short *P;         // [slot][S][N/64][256][64]
   long p_slot, p_slice;
   long pos0;                 // position of token 0 of this pass
-  int N, Tc, ldv, h, n_slices, nt;  // nt = N / 256 neuron tiles per slice
+  int N, Tc, h, n_slices;
   int has_state;             // the accumulators start from rho, and slot 0 is written
   int lo_slot;               // >= 0: bf16(rho_0 - float(bf16(rho_0))) goes to that slot
   const int *pairs_equal;    // device flag written by k_freq_pairs_equal
 };
 
-constexpr int UPD_A_TILE = 64 * KM_STRIDE;       // k-major activations tile: 64 tokens x (256+32) neurons
-constexpr int UPD_B_TILE = 256 * LDS_STRIDE;     // V^T tile: 256 value columns x (64+8) tokens
-constexpr int UPD_BUF = UPD_A_TILE + UPD_B_TILE;  // elements per stage (73728 bytes)
-constexpr int UPD_LDS = 2 * UPD_BUF * 2 + 256 * 2 * 4;  // two stages + the per-neuron 16-token rotation steps
-#ifndef BDH_UPD_SCHED
-#define BDH_UPD_SCHED 1
-#endif
-constexpr int DUMP_ROW = 256 + 8;                 // bf16 elements per staged row of a state dump
-static_assert(128 * DUMP_ROW <= UPD_BUF, "half a dump must fit the free stage");
+// V of a pass in the order the state update's B operand is consumed: Vf[b][step][dt][kk][lane][8] holds
+// V[b][token 64 step + 16 kk + 8 (lane >> 5) + e][value 32 dt + (lane & 31)], so that one fragment load of a
+// wavefront is 1 KiB of consecutive bytes.  in: [B][Tc][256] bf16 (batch stride in_batch), Tc a multiple of 64.
+__global__ __launch_bounds__(256) void k_v_fragments(const unsigned short *__restrict__ in, long in_batch,
+                                                     unsigned short *__restrict__ out, int Tc) {
+  __shared__ unsigned short s_v[64][256 + 2];
+  const int step = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const unsigned short *src = in + (long)b * in_batch + (long)step * 64 * 256;
+  for (int i = tid; i < 64 * 128; i += 256) {  // two bf16 per access
+    const int t = i >> 7, c2 = (i & 127) * 2;
+    const unsigned int v = *reinterpret_cast<const unsigned int *>(src + t * 256 + c2);
+    s_v[t][c2] = (unsigned short)(v & 0xffffu);
+    s_v[t][c2 + 1] = (unsigned short)(v >> 16);
+  }
+  __syncthreads();
+  unsigned short *dst = out + ((long)b * (Tc / 64) + step) * (64 * 256);
+  for (int piece = tid; piece < 8 * 4 * 64; piece += 256) {
+    const int lane = piece & 63, kk = (piece >> 6) & 3, dt = piece >> 8;
+    const int t0 = kk * 16 + (lane >> 5) * 8, c = dt * 32 + (lane & 31);
+    unsigned int w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = (unsigned int)s_v[t0 + 2 * e][c] | ((unsigned int)s_v[t0 + 2 * e + 1][c] << 16);
+    *reinterpret_cast<uint4 *>(dst + (long)piece * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
 
-template <bool EQ>  // EQ: the two elements of every lane pair share a frequency (what build_freqs makes)
-__device__ __forceinline__ void state_update_body(const StateUpdArgs &g, unsigned short *s_dyn) {
-  float *s_step = reinterpret_cast<float *>(s_dyn + 2 * UPD_BUF);  // [256][2]: cos, sin of 16 tokens' phase advance
+// ---- the state update as a streaming kernel ---------------------------------------------------------------------
+// The same work as state_update_body in workgroups of four wavefronts that own 64 neurons x 256 value columns of a
+// slice's state (wavefront w: value columns 64w..64w+63, accumulators in 64 registers).  The update moves ~3 GiB
+// through HBM at the headline shape and needs ~0.14 ms of matrix-core time: it is a memory stream, so it is
+// laid out for many independent workgroups per CU (three or four, against one of the 256-neuron tile) whose loads,
+// stores, rotations and matrix products overlap each other, instead of for operand reuse.  Per 64-token step a
+// workgroup reads a [64 tokens x 64 neurons] tile of x (128-byte row pieces), rotates it in registers, stores Q,
+// keeps the tile in LDS for the transposing reads of the A operand; the B operand (V^T, L2-resident) goes straight
+// from global memory into registers, one step ahead, in the registers the matrix instructions just consumed.
+// sine and cosine of a fraction of a turn in [0, 1): the hardware instructions take their argument in turns
+// (absolute error below 2e-6 on that interval), no range reduction and no branches
+__device__ __forceinline__ void turn_sincos(float turns, float &sn, float &cs) {
+  sn = __builtin_amdgcn_sinf(turns);
+  cs = __builtin_amdgcn_cosf(turns);
+}
+
+#ifndef BDH_ST_LOOK
+#define BDH_ST_LOOK 2
+#endif
+constexpr int ST_LOOK = BDH_ST_LOOK;  // k-steps of B fragments in flight (1, 2 or 4)
+constexpr int ST_TN = 64;
+constexpr int ST_ASTRIDE = ST_TN + 32;           // bf16 per token row of the LDS tile: 48 dwords, the four rows a
+                                                 // transposing read touches cover the 64 banks once
+constexpr int ST_A_TILE = 64 * ST_ASTRIDE;       // elements per stage
+constexpr int ST_DUMP_ROW = ST_TN + 8;           // bf16 per staged value row of a state copy (144 bytes)
+constexpr int ST_DUMP_WAVE = 32 * ST_DUMP_ROW;   // a wavefront stages 32 value rows at a time
+constexpr int ST_LDS = (2 * ST_A_TILE + 4 * ST_DUMP_WAVE) * 2;
+
+template <bool EQ>
+__device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigned short *s_dyn) {
+  const int nt = g.N / ST_TN;
   const int xcd = blockIdx.x & 7;
   const int r = blockIdx.x >> 3;
-  const int slice = xcd + 8 * (r / g.nt);
+  const int slice = xcd + 8 * (r / nt);
   if (slice >= g.n_slices) return;
-  const int m0 = (r % g.nt) * 256;  // first neuron of this workgroup
+  const int n0 = (r % nt) * ST_TN;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 2, wn = wave & 3;
 
-  const unsigned short *X = g.X + (long)slice * g.x_slice + m0;
-  unsigned short *Qo = g.Q + (long)slice * g.q_slice + m0;
-  const unsigned short *Vt = g.Vt + (long)(slice / g.h) * g.vt_batch;
-  float *rho = g.rho + ((long)slice * g.N + m0) * 256;
+  const unsigned short *X = g.X + (long)slice * g.x_slice + n0;
+  unsigned short *Qo = g.Q + (long)slice * g.q_slice + (long)(r % nt) * g.Tc * 64;  // this tile's [Tc][64] strip
+  const unsigned short *Vf = g.Vf + (long)(slice / g.h) * g.vt_batch;  // fragment order, as many elements as V^T
+  float *rho = g.rho + ((long)slice * g.N + n0) * 256;
+  unsigned short *s_stage = s_dyn + 2 * ST_A_TILE + wave * ST_DUMP_WAVE;  // this wavefront's own staging rows
 
-  // rotation state of this thread: neurons mc..mc+7 of the tile, tokens (tid >> 5) + 16 j, j = 0, 1, ...
-  // (cos, sin) of the even element of each of the four lane pairs, and of the odd one when the table gives
-  // the two elements of a pair different frequencies (build_freqs gives them the same: then the whole
-  // wavefront keeps four states instead of eight)
-  const int mc = (tid & 31) * 8, tk = tid >> 5;
-  float cse[4], sne[4], cso[EQ ? 1 : 4], sno[EQ ? 1 : 4];
+  // this thread rotates neurons mc..mc+7 of the tile at tokens tk + 32 j
+  const int mc = (tid & 7) * 8, tk = tid >> 3;
   constexpr bool eq = EQ;
-  if (tid < 256) {
-    // the phase advance of 16 tokens: 16 f is exact in binary32, the fraction is taken as the reference takes it
-    const float raw = 16.0f * g.freqs[m0 + tid];
-    float s16, c16;
-    sincosf((raw - floorf(raw)) * kTwoPi, &s16, &c16);
-    s_step[2 * tid] = c16;
-    s_step[2 * tid + 1] = s16;
+  float cse[4], sne[4], cso[EQ ? 1 : 4], sno[EQ ? 1 : 4];
+  float c32e[4], s32e[4], c32o[EQ ? 1 : 4], s32o[EQ ? 1 : 4];  // the phase advance of 32 tokens
+  {
+    const float4 f0 = *reinterpret_cast<const float4 *>(g.freqs + n0 + mc);
+    const float4 f1 = *reinterpret_cast<const float4 *>(g.freqs + n0 + mc + 4);
+    const float fre[4] = {f0.x, f0.z, f1.x, f1.z}, fro[4] = {f0.y, f0.w, f1.y, f1.w};
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const float raw = 32.0f * fre[p];  // exact in binary32; the fraction is taken as the reference takes it
+      turn_sincos(raw - floorf(raw), s32e[p], c32e[p]);
+      if constexpr (!eq) {
+        const float rawo = 32.0f * fro[p];
+        turn_sincos(rawo - floorf(rawo), s32o[p], c32o[p]);
+      }
+    }
   }
-  // exact phases (src/model/attention.rs:338-343) at the first token of a chunk; 16-token steps inside it
+  // exact phases (src/model/attention.rs:338-343) at the first tokens of a chunk; 32-token steps inside it
   auto seed = [&](int token) {
     const float pos = (float)(g.pos0 + token);
-    const float4 f0 = *reinterpret_cast<const float4 *>(g.freqs + m0 + mc);
-    const float4 f1 = *reinterpret_cast<const float4 *>(g.freqs + m0 + mc + 4);
+    const float4 f0 = *reinterpret_cast<const float4 *>(g.freqs + n0 + mc);
+    const float4 f1 = *reinterpret_cast<const float4 *>(g.freqs + n0 + mc + 4);
     const float fre[4] = {f0.x, f0.z, f1.x, f1.z}, fro[4] = {f0.y, f0.w, f1.y, f1.w};
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const float raw = pos * fre[p];
-      sincosf((raw - floorf(raw)) * kTwoPi, &sne[p], &cse[p]);
+      turn_sincos(raw - floorf(raw), sne[p], cse[p]);
       if constexpr (!eq) {
         const float rawo = pos * fro[p];
-        sincosf((rawo - floorf(rawo)) * kTwoPi, &sno[p], &cso[p]);
+        turn_sincos(rawo - floorf(rawo), sno[p], cso[p]);
       }
     }
   };
   auto advance = [&]() {
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-      const float4 st = *reinterpret_cast<const float4 *>(s_step + 2 * (mc + 2 * p));  // c16, s16 of 2p and 2p + 1
-      const float c0 = cse[p] * st.x - sne[p] * st.y, s0 = sne[p] * st.x + cse[p] * st.y;
+      const float c0 = cse[p] * c32e[p] - sne[p] * s32e[p], s0 = sne[p] * c32e[p] + cse[p] * s32e[p];
       cse[p] = c0; sne[p] = s0;
       if constexpr (!eq) {
-        const float c1 = cso[p] * st.z - sno[p] * st.w, s1 = sno[p] * st.z + cso[p] * st.w;
+        const float c1 = cso[p] * c32o[p] - sno[p] * s32o[p], s1 = sno[p] * c32o[p] + cso[p] * s32o[p];
         cso[p] = c1; sno[p] = s1;
       }
     }
@@ -729,196 +783,214 @@ __device__ __forceinline__ void state_update_body(const StateUpdArgs &g, unsigne
     return make_uint4(o[0], o[1], o[2], o[3]);
   };
 
-  f32x16 acc[4][2];
+  // every global access below is a wavefront-uniform base (scalar registers) plus this lane's unsigned 32-bit
+  // byte offset: no 64-bit address arithmetic per lane, no address registers kept alive across steps
+  auto at = [](const void *base, unsigned int byte_off) { return static_cast<const char *>(base) + byte_off; };
+  auto at_w = [](void *base, unsigned int byte_off) { return static_cast<char *>(base) + byte_off; };
+  // accumulators: rows = neurons 32 i + 8 (e >> 2) + 4 (lane >> 5) + (e & 3), column = value 64 wave + 32 j + (lane & 31)
+  f32x16 acc[2][2];
   if (g.has_state) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int col = wn * 64 + j * 32 + (lane & 31);
+        const int col = wave * 64 + j * 32 + (lane & 31);
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int row = wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-          acc[i][j][e] = rho[(long)row * 256 + col];
+          const int row = i * 32 + (e >> 2) * 8 + (e & 3);  // + 4 (lane >> 5), in the lane's offset
+          acc[i][j][e] = *reinterpret_cast<const float *>(at(rho + row * 256, (unsigned int)((lane >> 5) * 1024 + col) * 4u));
         }
       }
   } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
   }
 
-  uint4 ra[4];
-  // addresses = a wavefront-uniform row pointer + this lane's 32-bit offset (scalar base + vector offset form)
-  const int lane_off = tk * g.N + mc;
-  auto load_piece = [&](int step, int c) {  // activations of 16 tokens of a step into registers
-    const unsigned short *rowp = X + (long)(step * 64 + c * 16) * g.N;
-    ra[c] = *reinterpret_cast<const uint4 *>(rowp + lane_off);
+  // activations: two steps ahead of their use, in two register slots that alternate by step parity (under load a
+  // read from HBM takes longer than the matrix products of one step)
+  uint4 ra[2][2];
+  const unsigned int lane_off = (unsigned int)(tk * g.N + mc) * 2u, q_off = (unsigned int)(tk * 64 + mc) * 2u;
+  auto load_piece = [&](int step, auto slot_t, int c) {  // activations of 32 tokens of a step
+    constexpr int SLOT = decltype(slot_t)::value;
+    const unsigned short *rowp = X + (long)(step * 64 + c * 32) * g.N;
+    ra[SLOT][c] = *reinterpret_cast<const uint4 *>(at(rowp, lane_off));
   };
-  // The V^T tile of a step (256 value columns x 64 tokens, L2-resident) goes through registers, half a tile at a
-  // time.  (A direct global->LDS copy would save the registers, but the compiler then makes every LDS access that
-  // might alias its destination wait for ALL outstanding global accesses, the prefetched activations included.)
-  uint4 rb[2];
-  const int v_lane_off = (tid >> 3) * g.ldv + (tid & 7) * 8;
-  auto load_v = [&](int step, int half) {
+  // B fragments of a step: fb[kk][j] = V[tokens 16 kk + 8 (lane >> 5) .. + 8)[value 64 wave + 32 j + (lane & 31)],
+  // 1 KiB of consecutive bytes per wavefront and fragment in the fragment-order copy of V
+  // a ring of ST_LOOK k-steps: fragment kk + ST_LOOK is fetched into the slot the products of kk just read
+  bf16x8 fb[ST_LOOK][2];
+  const unsigned int vb_off = (unsigned int)(wave * 2 * 4 * 64 + lane) * 16u;
+  auto load_b = [&](int step, int kk) {
+    const unsigned short *vp = Vf + (long)step * (64 * 256) + kk * (64 * 8);
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      // chunk = (half*2 + c)*512 + tid: row = chunk >> 3 = (half*2 + c)*64 + (tid >> 3), k-chunk = tid & 7
-      const unsigned short *vp = Vt + (long)((half * 2 + c) * 64) * g.ldv + step * 64;
-      rb[c] = *reinterpret_cast<const uint4 *>(vp + v_lane_off);
-    }
+    for (int j = 0; j < 2; ++j) fb[kk % ST_LOOK][j] = *reinterpret_cast<const bf16x8 *>(at(vp + j * (4 * 64 * 8), vb_off));
   };
-  auto store_v = [&](int step, int half) {
-    unsigned short *sb = s_dyn + (step & 1) * UPD_BUF + UPD_A_TILE;
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const int chunk = (half * 2 + c) * 512 + tid;
-      const int row = chunk >> 3, kc = (chunk & 7) * 8;
-      *reinterpret_cast<uint4 *>(sb + row * LDS_STRIDE + kc) = rb[c];
-    }
-  };
-  // piece c of a staged step: rotate, write Q, put both operands into the stage's LDS buffers
-  auto stage_piece = [&](int step, int c) {
-    unsigned short *sa = s_dyn + (step & 1) * UPD_BUF;
-    const uint4 q = rotate(ra[c]);
+  auto stage_piece = [&](int step, auto slot_t, int c) {  // rotate, write Q, put the A operand into the stage's LDS tile
+    constexpr int SLOT = decltype(slot_t)::value;
+    unsigned short *sa = s_dyn + SLOT * ST_A_TILE;
+    const uint4 q = rotate(ra[SLOT][c]);
     advance();
-    const int kr = c * 16 + tk;
-    unsigned short *qrow = Qo + (long)(step * 64 + c * 16) * g.N;
-    *reinterpret_cast<uint4 *>(qrow + lane_off) = q;
-    *reinterpret_cast<uint4 *>(sa + kr * KM_STRIDE + (mc ^ (((kr >> 3) & 1) << 5))) = q;
+    const int kr = c * 32 + tk;
+    unsigned short *qrow = Qo + (step * 64 + c * 32) * 64;
+    *reinterpret_cast<uint4 *>(at_w(qrow, q_off)) = q;
+    *reinterpret_cast<uint4 *>(sa + kr * ST_ASTRIDE + (mc ^ (((kr >> 3) & 1) << 5))) = q;
   };
-  // bf16 of the accumulators, transposed to [value column][neuron], through the free stage buffer
-  auto dump = [&](unsigned short *stage, int slot, bool remainder) {
-    // per-lane bases laundered through the register file: every access below is base + constant, and the
-    // compiler cannot hoist 70 precomputed addresses out of the token loop (that spilled the accumulators)
-    unsigned short *wbase = stage + ((wn & 1) * 64 + (lane & 31)) * DUMP_ROW + wm * 128 + (lane >> 5) * 4;
-    unsigned short *rbase = stage + (tid >> 5) * DUMP_ROW + (tid & 31) * 8;
-    unsigned short *dst = g.P + (long)slot * g.p_slot + (long)slice * g.p_slice + m0 + (long)(tid >> 5) * g.N + (tid & 31) * 8;
-    asm volatile("" : "+v"(wbase), "+v"(rbase), "+v"(dst));
+  // bf16 of the accumulators, transposed to [value column][neuron]: each wavefront stages its own 64 value rows,
+  // 32 at a time, in LDS rows of its own (LDS operations of one wavefront execute in order: no barrier), and
+  // writes them as whole 128-byte row pieces
+  auto dump = [&](int slot, bool remainder) {
+    unsigned short *dst = g.P + (long)slot * g.p_slot + (long)slice * g.p_slice + (long)(r % nt) * (256 * 64);
+    const unsigned int dst_off = (unsigned int)((wave * 64 + (lane >> 3)) * 64 + (lane & 7) * 8) * 2u;
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      if ((wn >> 1) == half) {
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
+        for (int e4 = 0; e4 < 4; ++e4) {
+          unsigned int b[2];
 #pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-              unsigned short b[4];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const float v = acc[i][j][e4 * 4 + e];
-                const unsigned short hi = f32_to_bf16_bits(v);
-                b[e] = remainder ? f32_to_bf16_bits(v - bf16_bits_to_f32(hi)) : hi;
-              }
-              *reinterpret_cast<uint2 *>(wbase + j * 32 * DUMP_ROW + i * 32 + e4 * 8) =
-                  make_uint2((unsigned int)b[0] | ((unsigned int)b[1] << 16), (unsigned int)b[2] | ((unsigned int)b[3] << 16));
+          for (int e2 = 0; e2 < 2; ++e2) {  // round to nearest even by the conversion instruction, no branches
+            const f32x2 v = {acc[i][j][e4 * 4 + 2 * e2], acc[i][j][e4 * 4 + 2 * e2 + 1]};
+            unsigned int hi = __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
+            if (remainder) {
+              const f32x2 rest = {v[0] - __uint_as_float(hi << 16), v[1] - __uint_as_float(hi & 0xffff0000u)};
+              hi = __builtin_bit_cast(unsigned int, __builtin_convertvector(rest, bf16x2));
             }
+            b[e2] = hi;
           }
-      }
-      lds_barrier();
+          *reinterpret_cast<uint2 *>(s_stage + (lane & 31) * ST_DUMP_ROW + i * 32 + e4 * 8 + (lane >> 5) * 4) =
+              make_uint2(b[0], b[1]);
+        }
 #pragma unroll
-      for (int pass = 0; pass < 8; ++pass)
-        *reinterpret_cast<uint4 *>(dst + (long)(half * 128 + pass * 16) * g.N) =
-            *reinterpret_cast<const uint4 *>(rbase + pass * 16 * DUMP_ROW);
-      lds_barrier();
+      for (int pass = 0; pass < 4; ++pass)
+        *reinterpret_cast<uint4 *>(at_w(dst + (j * 32 + pass * 8) * 64, dst_off)) =
+            *reinterpret_cast<const uint4 *>(s_stage + (pass * 8 + (lane >> 3)) * ST_DUMP_ROW + (lane & 7) * 8);
     }
   };
 
-  const int nk = g.Tc / 64;
-  __syncthreads();  // s_step
+  // The token loop is laid out as straight-line code per 256-token chunk (four steps, no run-time branches
+  // inside): the compiler counts outstanding memory operations statically, and only in a branch-free body does
+  // it let the loads of the next step, the Q stores and the state copies stay in flight across the matrix
+  // products instead of draining them at every join.  Tc is a multiple of 256 here.
+  const int nc = g.Tc / 256;
+  // step kt = 4 c + S_: staging of step kt + 1 (MORE), fetch of the activations of step kt + 3 (MORE3) into the
+  // registers the staging just freed, then the matrix products of step kt from LDS tile S_ & 1.  (Placing the
+  // rotation inside the product regions, with the A fragments read one k-step ahead, measured 12 % slower: the
+  // Q stores and activation loads then sit between the B-fragment loads, and with one in-order memory counter
+  // every wait for a fragment becomes a wait for them.)
+  auto step = [&](int kt, auto s_t, auto more_t, auto more3_t) {
+    constexpr int S_ = decltype(s_t)::value;
+    constexpr bool MORE = decltype(more_t)::value, MORE3 = decltype(more3_t)::value;
+    using Next = std::integral_constant<int, (S_ + 1) & 1>;
+    const unsigned short *s_a = s_dyn + (S_ & 1) * ST_A_TILE;
+    if constexpr (MORE) {
 #pragma unroll
-  for (int c = 0; c < 4; ++c) load_piece(0, c);
-  load_v(0, 0);
-  seed(tk);
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    stage_piece(0, c);
-    if (nk > 1) load_piece(1, c);
-  }
-  store_v(0, 0);
-  load_v(0, 1);
-  store_v(0, 1);
-  lds_barrier();
-  // One step: the matrix products of step kt from one LDS stage and, between them and 16 tokens at a time,
-  // {rotate step kt+1's activations, store Q, fill the other stage, fetch step kt+2}; step kt+1's V^T tile
-  // follows in two halves.  MORE / MORE2 (is there a step kt+1 / kt+2) are compile-time so that the body is one
-  // straight block the scheduler can interleave; barriers order LDS only, global accesses stay in flight.
-  auto step = [&](int kt, auto more_t, auto more2_t) {
-    constexpr bool MORE = decltype(more_t)::value, MORE2 = decltype(more2_t)::value;
-    const unsigned short *s_a = s_dyn + (kt & 1) * UPD_BUF, *s_b = s_a + UPD_A_TILE;
-    if ((kt & 3) == 0 && (kt > 0 || g.has_state)) {
-      unsigned short *stage = s_dyn + ((kt + 1) & 1) * UPD_BUF;
-      dump(stage, kt >> 2, false);
-      if (kt == 0 && g.lo_slot >= 0) dump(stage, g.lo_slot, true);
-    }
-    if (MORE && (kt & 3) == 3) seed((kt + 1) * 64 + tk);  // the next step opens a chunk: exact phases
-    if (MORE) load_v(kt + 1, 0);
-#pragma unroll
-    for (int kk = 0; kk < BK; kk += 16) {
-      if (MORE) {
-        stage_piece(kt + 1, kk >> 4);
-        if (MORE2) load_piece(kt + 2, kk >> 4);
-        if (kk == 32) {
-          store_v(kt + 1, 0);
-          load_v(kt + 1, 1);
-        }
+      for (int c = 0; c < 2; ++c) {
+        stage_piece(kt + 1, Next{}, c);
+        if constexpr (MORE3) load_piece(kt + 3, Next{}, c);
       }
-      bf16x8 fa[4], fb[2];
-      const int kof = kk + (lane >> 5) * 8;
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+    for (int kk = 0; kk < 4; ++kk) {
+      bf16x8 fa[2];
+      const int kof = kk * 16 + (lane >> 5) * 8;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
         // transposing LDS read: see k_gemm
         const int j16 = lane & 15;
-        const int mcol = (wm * 128 + i * 32 + ((lane >> 4) & 1) * 16) ^ ((lane >> 5) << 5);
-        const unsigned short *src = s_a + (kof + (j16 >> 2)) * KM_STRIDE + mcol + (j16 & 3) * 4;
+        const int mcol = (i * 32 + ((lane >> 4) & 1) * 16) ^ ((lane >> 5) << 5);
+        const unsigned short *src = s_a + (kof + (j16 >> 2)) * ST_ASTRIDE + mcol + (j16 & 3) * 4;
         typedef short s16x4 __attribute__((ext_vector_type(4)));
         typedef short s16x8 __attribute__((ext_vector_type(8)));
         typedef __attribute__((address_space(3))) s16x4 *lds_s16x4_t;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(src));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(src + 4 * KM_STRIDE));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(src + 4 * ST_ASTRIDE));
         const s16x8 pk = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         fa[i] = __builtin_bit_cast(bf16x8, pk);
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        fb[j] = *reinterpret_cast<const bf16x8 *>(s_b + (wn * 64 + j * 32 + (lane & 31)) * LDS_STRIDE + kof);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-#if BDH_UPD_SCHED
-      if (MORE) {
-#pragma unroll
-        for (int q8 = 0; q8 < 8; ++q8) {  // the rotation arithmetic in the shadow of the matrix instructions
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 9, 0);
-        }
-      }
-#endif
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[kk % ST_LOOK][j], acc[i][j], 0, 0, 0);
+      // into the registers the products above just read: nothing may be scheduled across, or the compiler
+      // hoists these loads over the products and keeps more sets of fragments alive
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk + ST_LOOK < 4) load_b(kt, kk + ST_LOOK);
+      else if constexpr (MORE) load_b(kt + 1, kk + ST_LOOK - 4);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (MORE) store_v(kt + 1, 1);
     lds_barrier();
   };
-  int kt = 0;
-  for (; kt + 2 < nk; ++kt) step(kt, std::true_type{}, std::true_type{});
-  if (kt + 1 < nk) step(kt++, std::true_type{}, std::false_type{});
-  step(kt, std::false_type{}, std::false_type{});
+  auto chunk = [&](int c, auto dump_t, auto last_t) {
+    constexpr bool DUMP = decltype(dump_t)::value, LAST = decltype(last_t)::value;
+    using T = std::true_type;
+    using NotLast = std::integral_constant<bool, !LAST>;
+    const int kt = 4 * c;
+    if constexpr (DUMP) dump(c, false);
+    step(kt, std::integral_constant<int, 0>{}, T{}, T{});
+    step(kt + 1, std::integral_constant<int, 1>{}, T{}, NotLast{});
+    step(kt + 2, std::integral_constant<int, 2>{}, T{}, NotLast{});
+    if constexpr (!LAST) seed((kt + 4) * 64 + tk);  // the next step opens a chunk: exact phases
+    step(kt + 3, std::integral_constant<int, 3>{}, NotLast{}, NotLast{});
+  };
+
+  if (g.has_state) {
+    dump(0, false);
+    if (g.lo_slot >= 0) dump(g.lo_slot, true);
+  }
+  using Slot0 = std::integral_constant<int, 0>;
+  using Slot1 = std::integral_constant<int, 1>;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int c = 0; c < 2; ++c) load_piece(0, Slot0{}, c);
+  seed(tk);
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    stage_piece(0, Slot0{}, c);
+    load_piece(1, Slot1{}, c);
+  }
+#pragma unroll
+  for (int c = 0; c < 2; ++c) load_piece(2, Slot0{}, c);
+#pragma unroll
+  for (int kk = 0; kk < ST_LOOK; ++kk) load_b(0, kk);
+  lds_barrier();
+  if (nc == 1) {
+    chunk(0, std::false_type{}, std::true_type{});
+  } else {
+    chunk(0, std::false_type{}, std::false_type{});
+#pragma unroll 1
+    for (int c = 1; c + 1 < nc; ++c) chunk(c, std::true_type{}, std::false_type{});
+    chunk(nc - 1, std::true_type{}, std::true_type{});
+  }
+  // the addresses of the final stores equal those of the initial loads: hidden from the compiler here, or it
+  // keeps all of them in registers across the token loop
+  asm volatile("" : "+s"(rho));
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int col = wn * 64 + j * 32 + (lane & 31);
+      const int col = wave * 64 + j * 32 + (lane & 31);
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int row = wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        rho[(long)row * 256 + col] = acc[i][j][e];
+        const int row = i * 32 + (e >> 2) * 8 + (e & 3);  // + 4 (lane >> 5), in the lane's offset
+        *reinterpret_cast<float *>(at_w(rho + row * 256, (unsigned int)((lane >> 5) * 1024 + col) * 4u)) = acc[i][j][e];
       }
     }
+}
+
+#ifndef BDH_ST_WAVES
+#define BDH_ST_WAVES 2
+#endif
+template <bool EQ>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BDH_ST_WAVES, BDH_ST_WAVES))) void k_state_stream(StateUpdArgs g) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned short s_dyn[];
+  if ((g.pairs_equal[0] != 0) != EQ) return;
+  state_stream_body<EQ>(g, s_dyn);
 }
 
 // flag[0] = 1 when the two elements of every lane pair share a frequency (what build_freqs makes), else 0
@@ -930,15 +1002,6 @@ __global__ __launch_bounds__(256) void k_freq_pairs_equal(const float *__restric
   }
   ok = __syncthreads_and(ok);
   if (threadIdx.x == 0) flag[0] = ok;
-}
-
-// Both instantiations are launched; the one the frequency table does not call for returns at once (the choice
-// is made on the device, so no host synchronisation is needed, and each body gets its own register allocation).
-template <bool EQ>
-__global__ __launch_bounds__(512) void k_state_update(StateUpdArgs g) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned short s_dyn[];
-  if ((g.pairs_equal[0] != 0) != EQ) return;
-  state_update_body<EQ>(g, s_dyn);
 }
 
 template <bool AK, int EPI>
@@ -1078,45 +1141,49 @@ static int prefill_pass_chunks(bdh_ctx *ctx, int B, int h, int Tc, int N, const 
                                const uint16_t *v_bf16, long v_batch, const float *freqs, int64_t position,
                                int state_is_zero, int hilo, float *rho, float *out, long out_slice) {
   constexpr int d = 256;
-  const int S = B * h, nc = Tc / 256, nt = N / 256;
+  const int S = B * h, nc = Tc / 256;
   const int lo_slot = (!state_is_zero && hilo) ? nc : -1;
   const int slots = nc + (lo_slot >= 0 ? 1 : 0);
-  // workspace: Q bf16 [S,Tc,N] | P bf16 [slots,S,d,N] | V^T bf16 [B,d,Tc]
+  // workspace: Q bf16 [S,N/64,Tc,64] | P bf16 [slots,S,N/64,d,64] | V^T bf16 [B,d,Tc] | V in fragment order (same size)
   const size_t q_bytes = bdh_align_up((size_t)S * Tc * N * 2, 256);
   const size_t p_bytes = bdh_align_up((size_t)slots * S * d * N * 2, 256);
   const size_t vt_bytes = bdh_align_up((size_t)B * d * Tc * 2, 256);
-  int rc = bdh_ws_reserve(ctx, q_bytes + p_bytes + vt_bytes + 256);
+  int rc = bdh_ws_reserve(ctx, q_bytes + p_bytes + 2 * vt_bytes + 256);
   if (rc != BDH_OK) return rc;
   char *ws = static_cast<char *>(ctx->ws);
   unsigned short *Q = reinterpret_cast<unsigned short *>(ws);
   unsigned short *P = reinterpret_cast<unsigned short *>(ws + q_bytes);
   unsigned short *Vt = reinterpret_cast<unsigned short *>(ws + q_bytes + p_bytes);
-  int *flag = reinterpret_cast<int *>(ws + q_bytes + p_bytes + vt_bytes);
+  unsigned short *Vf = reinterpret_cast<unsigned short *>(ws + q_bytes + p_bytes + vt_bytes);
+  int *flag = reinterpret_cast<int *>(ws + q_bytes + p_bytes + 2 * vt_bytes);
   const int groups = (S + 7) / 8;
-  if ((long)groups * 8 * std::max(nt, nc) > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
+  if ((long)groups * 8 * std::max(N / ST_TN, nc) > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
 
   hipLaunchKernelGGL(k_transpose_to_bf16<unsigned short>, dim3(d / 64, Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16,
                      Vt, Tc, d, Tc, v_batch);
   BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<V>");
+  hipLaunchKernelGGL(k_v_fragments, dim3(Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16, v_batch, Vf, Tc);
+  BDH_LAUNCH_CHECK(ctx, "k_v_fragments");
   hipLaunchKernelGGL(k_freq_pairs_equal, dim3(1), dim3(256), 0, ctx->stream, freqs, N, flag);
   BDH_LAUNCH_CHECK(ctx, "k_freq_pairs_equal");
   {
     static std::atomic<uint64_t> configured_eq{0}, configured_ne{0};
-    BDH_HIP_CHECK(ctx, allow_lds(k_state_update<true>, UPD_LDS, configured_eq));
-    BDH_HIP_CHECK(ctx, allow_lds(k_state_update<false>, UPD_LDS, configured_ne));
+    BDH_HIP_CHECK(ctx, allow_lds(k_state_stream<true>, ST_LDS, configured_eq));
+    BDH_HIP_CHECK(ctx, allow_lds(k_state_stream<false>, ST_LDS, configured_ne));
     StateUpdArgs g{};
     g.X = x_bf16; g.x_slice = x_slice;
     g.Q = Q; g.q_slice = (long)Tc * N;
-    g.Vt = Vt; g.vt_batch = (long)d * Tc; g.ldv = Tc;
+    g.Vf = Vf; g.vt_batch = (long)d * Tc;
     g.freqs = freqs; g.rho = rho;
     g.P = P; g.p_slot = (long)S * d * N; g.p_slice = (long)d * N;
     g.pos0 = (long)position;
-    g.N = N; g.Tc = Tc; g.h = h; g.n_slices = S; g.nt = nt;
+    g.N = N; g.Tc = Tc; g.h = h; g.n_slices = S;
     g.has_state = state_is_zero ? 0 : 1; g.lo_slot = lo_slot;
     g.pairs_equal = flag;
-    hipLaunchKernelGGL(k_state_update<true>, dim3(8 * groups * nt), dim3(512), UPD_LDS, ctx->stream, g);
-    hipLaunchKernelGGL(k_state_update<false>, dim3(8 * groups * nt), dim3(512), UPD_LDS, ctx->stream, g);
-    BDH_LAUNCH_CHECK(ctx, "k_state_update");
+    const int nts = N / ST_TN;
+    hipLaunchKernelGGL(k_state_stream<true>, dim3(8 * groups * nts), dim3(256), ST_LDS, ctx->stream, g);
+    hipLaunchKernelGGL(k_state_stream<false>, dim3(8 * groups * nts), dim3(256), ST_LDS, ctx->stream, g);
+    BDH_LAUNCH_CHECK(ctx, "k_state_stream");
   }
   {
     static std::atomic<uint64_t> configured{0};
