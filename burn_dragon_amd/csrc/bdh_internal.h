@@ -142,8 +142,17 @@ int bdh_launch_embed_ln(bdh_ctx *ctx, const int64_t *tokens, int64_t rows, int d
                         const float *embed, float *out);
 // mlp = mixed . decoder with mixed[b*T+t, hh*N+n] = xy[b,hh,t,n]; cur = LN(cur + LN(mlp))
 // (src/model/bdh.rs:383,436-441)
+// The output head of the rows the decoder's second stage finishes, run in that same launch (the last layer of a
+// model): logits[m,:] = cur[m,:] . lm_head and, optionally, the greedy token of each sequence's last row.
+struct DecoderHead {
+  const float *lm_head;  // [d][V]
+  int T, V;
+  float *logits;         // [M][V]
+  int64_t *next_tokens;  // [B] or null
+};
 int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
-                                const float *xy, const float *decoder, float *cur);
+                                const float *xy, const float *decoder, float *cur,
+                                const DecoderHead *head = nullptr);
 // logits = cur . lm_head (+ argmax of the last token per sequence) (src/model/bdh.rs:446-449)
 // attention_parallel.hip: partial[hh][b*T+t][:] = xy[b,hh,t,:] . decoder[hh*N.., :] on the f32 matrix cores
 int bdh_launch_decoder_partials_f32(bdh_ctx *ctx, int B, int T, int h, int N, int d, const float *xy,

@@ -223,12 +223,12 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
         rc = bdh_launch_fill_zero_f32(ctx, vz + (size_t)3 * h * N, (long)h * N);
       if (rc != BDH_OK) return rc;
     }
-    // :383,436-441  cur = LN(cur + LN(mixed . decoder))
-    rc = bdh_launch_decoder_residual(ctx, B, T, h, N, d, xy, m->w.decoder, cur);
+    // :383,436-441  cur = LN(cur + LN(mixed . decoder)); the last layer's launch also runs the output head (:446-449)
+    const DecoderHead head{m->w.lm_head, T, V, logits, next_tokens};
+    rc = bdh_launch_decoder_residual(ctx, B, T, h, N, d, xy, m->w.decoder, cur, l == L - 1 ? &head : nullptr);
     if (rc != BDH_OK) return rc;
   }
-  // :446-449
-  return bdh_launch_lm_head(ctx, B, T, d, V, cur, m->w.lm_head, logits, next_tokens);
+  return BDH_OK;
 }
 
 int bdh_model_forward_fast(bdh_model *m, const int64_t *tokens, int B, int T, int time_block_size, float *logits) {

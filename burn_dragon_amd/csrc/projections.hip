@@ -562,116 +562,14 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
   }
 }
 
-// cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))   (src/model/bdh.rs:438-441)
-// 1024 threads = 16 groups of 64 lanes; a lane owns four adjacent columns (one 16-byte load per partial
-// row), a group adds a sixteenth of the k-block partials in index order with up to 16 loads in flight,
-// the groups are combined in order; after the one barrier the first wavefront applies the two LayerNorms
-// with wave shuffles only.
-__global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restrict__ partial, int KBN, int M,
-                                                           int d, float *__restrict__ cur) {
-  __shared__ float s_grp[16][1024];
-  const int m = blockIdx.x, lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
-  const int per = (KBN + 15) >> 4;
-  const int kb0 = min(KBN, grp * per), kb1 = min(KBN, kb0 + per);
-  // the residual row is fetched while the partials are summed: it was written by another
-  // workgroup of an earlier launch, so the load is a trip to memory
-  float res[16];
-  if (grp == 0) {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) res[j] = (j * 64 + lane < d) ? cur[(long)m * d + j * 64 + lane] : 0.0f;
-  }
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int c = (j * 64 + lane) * 4;  // d % 4 == 0
-    if (c < d) {
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      int kb = kb0;
-      for (; kb + 16 <= kb1; kb += 16) {
-        float4 t[16];
-#pragma unroll
-        for (int u = 0; u < 16; ++u) t[u] = *reinterpret_cast<const float4 *>(partial + ((long)(kb + u) * M + m) * d + c);
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-          v.x += t[u].x; v.y += t[u].y; v.z += t[u].z; v.w += t[u].w;
-        }
-      }
-      for (; kb < kb1; ++kb) {
-        const float4 t = *reinterpret_cast<const float4 *>(partial + ((long)kb * M + m) * d + c);
-        v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
-      }
-      *reinterpret_cast<float4 *>(&s_grp[grp][c]) = v;
-    }
-  }
-  __syncthreads();
-  if (threadIdx.x >= 64) return;  // no barrier follows: the first wave finishes the row alone
-  float vals[16];  // column c = j*64 + lane, d <= 1024
-  float s = 0.0f;
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    const int c = j * 64 + lane;
-    float v = 0.0f;
-    if (c < d) {
-      v = s_grp[0][c];
-#pragma unroll
-      for (int g = 1; g < 16; ++g) v += s_grp[g][c];
-      s += v;
-    }
-    vals[j] = v;
-  }
-  auto wave_sum = [](float v) {
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-  };
-  float mean = wave_sum(s) / (float)d;
-  float q = 0.0f;
-#pragma unroll
-  for (int j = 0; j < 16; ++j)
-    if (j * 64 + lane < d) {
-      const float t = vals[j] - mean;
-      q += t * t;
-    }
-  float den = sqrtf(wave_sum(q) / (float)d + kLnEps);
-  s = 0.0f;
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    const int c = j * 64 + lane;
-    if (c < d) {
-      const float mlp = (vals[j] - mean) / den;
-      vals[j] = res[j] + mlp;
-      s += vals[j];
-    }
-  }
-  mean = wave_sum(s) / (float)d;
-  q = 0.0f;
-#pragma unroll
-  for (int j = 0; j < 16; ++j)
-    if (j * 64 + lane < d) {
-      const float t = vals[j] - mean;
-      q += t * t;
-    }
-  den = sqrtf(wave_sum(q) / (float)d + kLnEps);
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    const int c = j * 64 + lane;
-    if (c < d) cur[(long)m * d + c] = (vals[j] - mean) / den;
-  }
-}
-
 // logits[m,:] = cur[m,:] . lm_head ; optional argmax of the last token of each sequence.
 // 1024 threads: 256 vocabulary columns x 4 groups over k; the four partial dot products of a
-// logit are added in group order.
-__global__ __launch_bounds__(1024) void k_lm_head(const float *__restrict__ cur, const float *__restrict__ W,
-                                                  int T, int d, int V, float *__restrict__ logits,
-                                                  int64_t *__restrict__ next_tokens) {
-  extern __shared__ float s_dyn[];  // [d] input row, then [4][256] partials
-  __shared__ float s_best[4];
-  __shared__ int s_arg[4];
-  float *s_cur = s_dyn;
-  float *s_acc = s_dyn + d;
-  const int m = blockIdx.x, tid = threadIdx.x & 255, grp = threadIdx.x >> 8;
+// logit are added in group order.  s_cur holds the input row (every thread sees it), s_acc has 1024 floats.
+__device__ __forceinline__ void lm_head_row(const float *s_cur, float *s_acc, float *s_best, int *s_arg, int m,
+                                            const float *__restrict__ W, int T, int d, int V,
+                                            float *__restrict__ logits, int64_t *__restrict__ next_tokens) {
+  const int tid = threadIdx.x & 255, grp = threadIdx.x >> 8;
   const int lane = tid & 63, wave = tid >> 6;
-  for (int k = threadIdx.x; k < d; k += 1024) s_cur[k] = cur[(long)m * d + k];
-  __syncthreads();
   const int per = (d + 3) >> 2;
   const int k0 = grp * per, k1 = min(d, k0 + per);
   float best = -INFINITY;
@@ -726,6 +624,128 @@ __global__ __launch_bounds__(1024) void k_lm_head(const float *__restrict__ cur,
       }
     next_tokens[b] = arg == 0x7fffffff ? 0 : arg;
   }
+}
+
+// cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:]))   (src/model/bdh.rs:438-441)
+// 1024 threads = 16 groups of 64 lanes; a lane owns four adjacent columns (one 16-byte load per partial
+// row), a group adds a sixteenth of the k-block partials in index order with up to 16 loads in flight,
+// the groups are combined in order; after the one barrier the first wavefront applies the two LayerNorms
+// with wave shuffles only.
+// HEAD: the output head of the same row follows in the same launch (the last layer of a model): the finished row
+// goes to LDS as well, and all 1024 threads run lm_head_row on it -- the arithmetic of k_lm_head, one launch less.
+template <bool HEAD>
+__global__ __launch_bounds__(1024) void k_decoder_finalize(const float *__restrict__ partial, int KBN, int M,
+                                                           int d, float *__restrict__ cur, DecoderHead head) {
+  __shared__ float s_grp[16][1024];
+  __shared__ float s_best[4];
+  __shared__ int s_arg[4];
+  const int m = blockIdx.x, lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int per = (KBN + 15) >> 4;
+  const int kb0 = min(KBN, grp * per), kb1 = min(KBN, kb0 + per);
+  // the residual row is fetched while the partials are summed: it was written by another
+  // workgroup of an earlier launch, so the load is a trip to memory
+  float res[16];
+  if (grp == 0) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) res[j] = (j * 64 + lane < d) ? cur[(long)m * d + j * 64 + lane] : 0.0f;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = (j * 64 + lane) * 4;  // d % 4 == 0
+    if (c < d) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      int kb = kb0;
+      for (; kb + 16 <= kb1; kb += 16) {
+        float4 t[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) t[u] = *reinterpret_cast<const float4 *>(partial + ((long)(kb + u) * M + m) * d + c);
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          v.x += t[u].x; v.y += t[u].y; v.z += t[u].z; v.w += t[u].w;
+        }
+      }
+      for (; kb < kb1; ++kb) {
+        const float4 t = *reinterpret_cast<const float4 *>(partial + ((long)kb * M + m) * d + c);
+        v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+      }
+      *reinterpret_cast<float4 *>(&s_grp[grp][c]) = v;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x >= 64) {  // the first wave finishes the row alone
+    if (!HEAD) return;      // (no barrier follows)
+  } else {
+  float vals[16];  // column c = j*64 + lane, d <= 1024
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int c = j * 64 + lane;
+    float v = 0.0f;
+    if (c < d) {
+      v = s_grp[0][c];
+#pragma unroll
+      for (int g = 1; g < 16; ++g) v += s_grp[g][c];
+      s += v;
+    }
+    vals[j] = v;
+  }
+  auto wave_sum = [](float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+  };
+  float mean = wave_sum(s) / (float)d;
+  float q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    if (j * 64 + lane < d) {
+      const float t = vals[j] - mean;
+      q += t * t;
+    }
+  float den = sqrtf(wave_sum(q) / (float)d + kLnEps);
+  s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int c = j * 64 + lane;
+    if (c < d) {
+      const float mlp = (vals[j] - mean) / den;
+      vals[j] = res[j] + mlp;
+      s += vals[j];
+    }
+  }
+  mean = wave_sum(s) / (float)d;
+  q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j)
+    if (j * 64 + lane < d) {
+      const float t = vals[j] - mean;
+      q += t * t;
+    }
+  den = sqrtf(wave_sum(q) / (float)d + kLnEps);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int c = j * 64 + lane;
+    if (c < d) {
+      const float y = (vals[j] - mean) / den;
+      cur[(long)m * d + c] = y;
+      if (HEAD) s_grp[2][c] = y;  // only this wave reads s_grp after the barrier above, and it has read all of it
+    }
+  }
+  }
+  if (!HEAD) return;
+  __syncthreads();  // the row is in s_grp[2]; rows 3.. are free for the partial dot products
+  lm_head_row(s_grp[2], s_grp[3], s_best, s_arg, m, head.lm_head, head.T, d, head.V, head.logits, head.next_tokens);
+}
+
+__global__ __launch_bounds__(1024) void k_lm_head(const float *__restrict__ cur, const float *__restrict__ W,
+                                                  int T, int d, int V, float *__restrict__ logits,
+                                                  int64_t *__restrict__ next_tokens) {
+  extern __shared__ float s_dyn[];  // [d] input row, then [4][256] partials
+  __shared__ float s_best[4];
+  __shared__ int s_arg[4];
+  const int m = blockIdx.x;
+  for (int k = threadIdx.x; k < d; k += 1024) s_dyn[k] = cur[(long)m * d + k];
+  __syncthreads();
+  lm_head_row(s_dyn, s_dyn + d, s_best, s_arg, m, W, T, d, V, logits, next_tokens);
 }
 
 __global__ void k_advance_positions(int32_t *pos, int B, int delta) {
@@ -864,8 +884,17 @@ int bdh_launch_embed_ln(bdh_ctx *ctx, const int64_t *tokens, int64_t rows, int d
   return BDH_OK;
 }
 
+static void launch_decoder_finalize(bdh_ctx *ctx, const float *partial, int KBN, int M, int d, float *cur,
+                                    const DecoderHead *head) {
+  if (head)
+    hipLaunchKernelGGL(k_decoder_finalize<true>, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur, *head);
+  else
+    hipLaunchKernelGGL(k_decoder_finalize<false>, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur,
+                       DecoderHead{});
+}
+
 int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d, const float *xy,
-                                const float *decoder, float *cur) {
+                                const float *decoder, float *cur, const DecoderHead *head) {
   const int M = B * T;
   const long K = (long)h * N;
   if (d > 1024 || (d & 3)) return bdh_fail(ctx, BDH_E_SHAPE, "decoder needs d %% 4 == 0 and d <= 1024, got %d", d);
@@ -878,7 +907,7 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
     float *partial = static_cast<float *>(ctx->ws);
     rc = bdh_launch_decoder_partials_f32(ctx, B, T, h, N, d, xy, decoder, partial);
     if (rc != BDH_OK) return rc;
-    hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, h, M, d, cur);
+    launch_decoder_finalize(ctx, partial, h, M, d, cur, head);
     BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
     return BDH_OK;
   }
@@ -895,7 +924,7 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
     float *partial = static_cast<float *>(ctx->ws);
     rc = bdh_launch_decoder_splitk_f32(ctx, M, K, d, KB, xy, decoder, partial);
     if (rc != BDH_OK) return rc;
-    hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur);
+    launch_decoder_finalize(ctx, partial, KBN, M, d, cur, head);
     BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
     return BDH_OK;
   }
@@ -934,14 +963,14 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   }
 #undef BDH_DEC
   BDH_LAUNCH_CHECK(ctx, "k_decoder_partial");
-  hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur);
+  launch_decoder_finalize(ctx, partial, KBN, M, d, cur, head);
   BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
   return BDH_OK;
 }
 
 int bdh_launch_decoder_finalize(bdh_ctx *ctx, const float *partial, int KBN, int M, int d, float *cur) {
   if (d > 1024 || (d & 3) != 0) return bdh_fail(ctx, BDH_E_SHAPE, "encoder second stage needs d %% 4 == 0 and d <= 1024");
-  hipLaunchKernelGGL(k_decoder_finalize, dim3(M), dim3(1024), 0, ctx->stream, partial, KBN, M, d, cur);
+  launch_decoder_finalize(ctx, partial, KBN, M, d, cur, nullptr);
   BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
   return BDH_OK;
 }
