@@ -155,6 +155,16 @@ def prefill_executed_flop(B, h, N, d, T):
     return B * h * per_slice
 
 
+def prefill_traffic_bytes(B, h, N, d, T):
+    """HBM bytes one call of the chunk-recurrent form moves from a fresh state: x read; Q (bf16) written by the
+    state update, read by the score product and again by the state product; a bf16 copy of the state per 256-token
+    chunk but the first, written and read; the f32 state written; out written."""
+    S, nc = B * h, T // 256
+    q = 2.0 * S * T * N
+    state_copy = 2.0 * S * N * d
+    return q + (q + 2 * q) + 2 * (nc - 1) * state_copy + 4.0 * S * N * d + 4.0 * S * T * d
+
+
 def bench_prefill(args):
     """BASELINE config 3 (see measure_prefill)."""
     B = 8 if args.batch == 32 else args.batch
@@ -176,10 +186,15 @@ def bench_prefill(args):
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "executed_tflops": (executed / (ms * 1e-3) / 1e12) if executed else None,
-                     "traffic": None,
-                     "kernel": "whole bdh_prefill_chunked call (k_state_update + k_chunk_out); algorithmic FLOP "
+                     "traffic": prefill_traffic_bytes(B, h, N, d, T) if chunked else None,
+                     "traffic_source": "buffer sizes of the chunk-recurrent form (x, Q written once and read twice, one "
+                                       "bf16 state copy per 256 tokens written and read, rho, out); counters in "
+                                       "profiles/prefill_config3_bf16_kernel_trace.md read 4 % more",
+                     "hbm_gbs": (prefill_traffic_bytes(B, h, N, d, T) / (ms * 1e-3) / 1e9) if chunked else None,
+                     "kernel": "whole bdh_prefill_chunked call (k_state_stream + k_chunk_out); algorithmic FLOP "
                                "= B*h*[T(T-1)N + T(T-1)d + 2TNd], the all-scores count of the workload; the "
-                               "chunk-recurrent form executes executed_flop_per_step of them"},
+                               "chunk-recurrent form executes executed_flop_per_step of them and is bound by its "
+                               "HBM traffic (hbm_gbs), not by the matrix cores"},
     }))
 
 
@@ -714,6 +729,9 @@ def main():
             "algorithmic_flop": p_flop, "tflops": p_flop / (p_ms * 1e-3) / 1e12,
             "frac": p_flop / (p_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
             "executed_flop": p_exec, "executed_tflops": p_exec / (p_ms * 1e-3) / 1e12,
+            # what bounds this form: its HBM traffic (buffer sizes; the counters of the profile read 4 % more)
+            "hbm_traffic_bytes": prefill_traffic_bytes(8, 4, 8192, 256, 2048),
+            "hbm_gbs": prefill_traffic_bytes(8, 4, 8192, 256, 2048) / (p_ms * 1e-3) / 1e9,
             "kernel_us_source": "profiles/prefill_config3_bf16_kernel_trace.md",
         }
     if not args.no_cpu_baseline:

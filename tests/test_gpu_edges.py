@@ -241,3 +241,41 @@ def test_context_follows_torchs_current_stream(bda, corc):
     torch.cuda.synchronize()
     assert ctx._stream == torch.cuda.current_stream(0).cuda_stream
     assert np.isfinite(out2.cpu().numpy()).all()
+
+
+def test_probe_chunks_moves_exactly_the_listed_chunks(bda):
+    """bdh_probe_chunks (the decode step's memory traffic without its arithmetic): mode 0 reads the listed chunks,
+    scales by 1 and writes them back -- the region is unchanged; mode 1 only reads; mode 2 writes zeros into the
+    listed chunks and nowhere else; chunks outside the region are skipped; argument errors are reported."""
+    from burn_dragon_amd import ffi
+
+    ctx = ffi.default_context(0)
+    lib = ctx.lib
+    rng = np.random.default_rng(9)
+    chunk_kib, n_region_chunks = 2, 4096  # an 8 MiB region
+    region = torch.from_numpy(rng.standard_normal(n_region_chunks * chunk_kib * 256).astype(np.float32)).to(DEV)
+    before = region.clone()
+    listed = rng.choice(n_region_chunks, 400, replace=False).astype(np.int32)
+    outside = np.array([n_region_chunks, n_region_chunks + 7, -1], np.int32)  # skipped
+    index = torch.from_numpy(np.concatenate([listed, outside])).to(DEV)
+    nbytes = region.numel() * 4
+    for mode in (0, 1):
+        ctx.check(lib.bdh_probe_chunks(ctx.handle, region.data_ptr(), nbytes, index.data_ptr(), index.numel(), chunk_kib,
+                                       mode, 64))
+        torch.cuda.synchronize()
+        assert torch.equal(region, before)
+    ctx.check(lib.bdh_probe_chunks(ctx.handle, region.data_ptr(), nbytes, index.data_ptr(), index.numel(), chunk_kib, 2, 64))
+    torch.cuda.synchronize()
+    got = region.view(n_region_chunks, -1)
+    mask = torch.zeros(n_region_chunks, dtype=torch.bool, device=DEV)
+    mask[torch.from_numpy(listed.astype(np.int64)).to(DEV)] = True
+    assert not got[mask].any()
+    assert torch.equal(got[~mask], before.view(n_region_chunks, -1)[~mask])
+    # nothing listed: a no-op; bad arguments: an error code and a message, no launch
+    assert lib.bdh_probe_chunks(ctx.handle, region.data_ptr(), nbytes, index.data_ptr(), 0, chunk_kib, 0, 64) == ffi.OK
+    for bad in (dict(mode=3), dict(chunk_kib=0), dict(workgroups=0), dict(n=-1)):
+        rc = lib.bdh_probe_chunks(ctx.handle, region.data_ptr(), nbytes, index.data_ptr(), bad.get("n", 4),
+                                  bad.get("chunk_kib", chunk_kib), bad.get("mode", 0), bad.get("workgroups", 64))
+        assert rc == ffi.E_INVAL, bad
+    assert lib.bdh_probe_chunks(ctx.handle, region.data_ptr() + 4, nbytes - 4, index.data_ptr(), 4, chunk_kib, 0,
+                                64) == ffi.E_ALIGN
