@@ -434,11 +434,11 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
 // It executes 45 % of the matrix work of the all-scores form at T = 2048 (one 256x256 score tile and
 // one 256x256 state product per chunk instead of (T/256+1)/2 score tiles), and its workspace is linear
 // in T.  Two kernels:
-//   k_state_update  one workgroup per (slice, 256 neurons): walks all tokens, keeps its 256x256 tile of
+//   k_state_stream  one workgroup per (slice, 64 neurons): walks all tokens, keeps its 64x256 tile of
 //                   rho in the accumulators (f32, started from the caller's state), rotates x on the way
 //                   in (RoPE; Q = bf16(rope(x)) is also written out for the second kernel) and, at every
-//                   chunk boundary, writes bf16(rho_c) transposed ([d][N], the k-contiguous B operand of
-//                   Q_c rho_c).
+//                   chunk boundary, writes bf16(rho_c) transposed (value-major, the k-contiguous B operand
+//                   of Q_c rho_c).  Q and the state copies are stored k-tile by k-tile, [N/64][rows][64].
 //   k_chunk_out     one workgroup per (slice, chunk): S = Q_c Q_c^T on the matrix cores (operands straight
 //                   from global memory into LDS), mask + round to bf16 into LDS, out = S V_c, then
 //                   out += Q_c bf16(rho_c) with the same accumulators, written once.
@@ -514,8 +514,6 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
-// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at "no wait")
-#define BDH_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
 struct ChunkOutArgs {
   const unsigned short *Q;   // [S][N/64][Tc][64] rotated activations of this pass, Tc = 256 nc
