@@ -218,6 +218,12 @@ struct FsaArgs {
   //   FSA_DECAY_STATE   EPI 2, A k-major: A[k,:] *= g^(K-k) on load and C = g^K * C + acc
   int decay_mode;
   float log_decay[64];
+  // EPI 3, relu_lowrank (src/kernel/relu_lowrank.rs:7-37): C = gate * mask * relu(acc + bias - thr), head = slice % mod
+  const float *rl_bias;            // [h][N] or null
+  float rl_thr;
+  const unsigned char *rl_mask;    // one byte per latent block (device) or null
+  int rl_block, rl_nblocks;
+  const float *rl_gate;            // laid out like C, or null
 };
 constexpr int FSA_DECAY_SCORES = 1, FSA_DECAY_ROWS = 2, FSA_DECAY_STATE = 4;
 
@@ -232,7 +238,10 @@ __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_
 }
 
 // EPI 0: scores (mask, ALiBi term, zero outside the pattern); EPI 1: out = acc / (norm + eps);
-// EPI 2: C = acc or C += acc.
+// EPI 2: C = acc or C += acc; EPI 3: the relu_lowrank epilogue.
+// SEQK: the eight matrix instructions of a 16-wide k stage take k = 0,1 | 2,3 | ... instead of 0,8 | 1,9 | ...; an
+// instruction adds its two k-steps one after the other as fused multiply-adds, so every output is then ONE
+// k-sequential fmaf chain -- the same bits as a scalar loop over k (A rows k-contiguous, B k-major only).
 // A k-major operand (its reduction index is the slow one in memory) is staged as it lies, [k][m] with a
 // row stride of tile + 4 floats: float4 stores, and fragment reads of one float per lane in which the
 // 32 lanes of a half-wave take consecutive addresses and the two halves (k and k + 8) fall on the two
@@ -240,8 +249,9 @@ __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_
 // Tile BM x BN, NWM x NWN waves, each wave (BM/NWM) x (BN/NWN).  The 128 x 128 tile needs 8 bytes per
 // clock and workgroup from the L2, which three resident workgroups per CU do not get; the
 // 256 x 256 tile halves that per FLOP and is the one that keeps the matrix cores busy.
-template <int EPI, bool A_KMAJOR, bool B_KMAJOR, int BM, int BN, int NWM, int NWN>
+template <int EPI, bool A_KMAJOR, bool B_KMAJOR, int BM, int BN, int NWM, int NWN, bool SEQK = false>
 __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
+  static_assert(!SEQK || (!A_KMAJOR && B_KMAJOR), "sequential k order is built for row-major A and k-major B");
   constexpr int NT = NWM * NWN * 64;
   constexpr int KLA = BM + 4, KLB = BN + 4;  // row strides of the k-major LDS layouts
   static_assert(FK * KLA <= BM * FLD && FK * KLB <= BN * FLD, "k-major tile must fit");
@@ -370,7 +380,12 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
         const int chunk = c * NT + tid;
         if (!A_KMAJOR) {
           const int row = chunk >> 2, kc = (chunk & 3) * 4;
-          *reinterpret_cast<float4 *>(s_a + row * FLD + kc) = pa[c];
+          if (SEQK) {  // k = kc, kc + 2 to places kc / 2, kc / 2 + 1; k = kc + 1, kc + 3 to places 8 + kc / 2, ...
+            *reinterpret_cast<float2 *>(s_a + row * FLD + (kc >> 1)) = make_float2(pa[c].x, pa[c].z);
+            *reinterpret_cast<float2 *>(s_a + row * FLD + 8 + (kc >> 1)) = make_float2(pa[c].y, pa[c].w);
+          } else {
+            *reinterpret_cast<float4 *>(s_a + row * FLD + kc) = pa[c];
+          }
         } else {
           const int kr = chunk / (BM / 4), mc = (chunk % (BM / 4)) * 4;
           *reinterpret_cast<float4 *>(s_a + kr * KLA + mc) = pa[c];
@@ -400,6 +415,8 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
           for (int q = 0; q < 8; ++q) fa[i][q] = p[q * KLA];
           continue;
         }
+        // (SEQK: the stage was stored with its even k in the first eight places of a row and its odd k in the
+        // last eight, so the same two reads give this half-wave k = 2 q + half)
         const float *p = s_a + (wm * (BM / NWM) + i * 32 + r) * FLD + kb;
         const float4 lo = *reinterpret_cast<const float4 *>(p), hi = *reinterpret_cast<const float4 *>(p + 4);
         fa[i][0] = lo.x; fa[i][1] = lo.y; fa[i][2] = lo.z; fa[i][3] = lo.w;
@@ -408,9 +425,9 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         if (B_KMAJOR) {
-          const float *p = s_b + kb * KLB + wn * (BN / NWN) + j * 32 + r;
+          const float *p = s_b + (SEQK ? (lane >> 5) : kb) * KLB + wn * (BN / NWN) + j * 32 + r;
 #pragma unroll
-          for (int q = 0; q < 8; ++q) fb[j][q] = p[q * KLB];
+          for (int q = 0; q < 8; ++q) fb[j][q] = p[(SEQK ? 2 * q : q) * KLB];
           continue;
         }
         const float *p = s_b + (wn * (BN / NWN) + j * 32 + r) * FLD + kb;
@@ -469,6 +486,20 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
           float v = acc[i][j][e];
           if (g.norm) v = v / (g.norm[(long)slice * g.M + row] + kRowNormEps);
           C[(long)row * g.ldc + col] = v;
+        } else if (EPI == 3) {
+          if (col >= g.N) continue;
+          const int hh = g.mod > 0 ? slice % g.mod : 0;
+          float pv = acc[i][j][e];
+          if (g.rl_bias) pv = pv + g.rl_bias[(long)hh * g.N + col];
+          if (g.rl_thr != 0.0f) pv = pv - g.rl_thr;
+          float y = pv > 0.0f ? pv : 0.0f;
+          if (g.rl_mask) {
+            const int blk = col / g.rl_block;
+            y = y * ((blk < g.rl_nblocks && g.rl_mask[blk]) ? 1.0f : 0.0f);
+          }
+          const long o = (long)row * g.ldc + col;
+          if (g.rl_gate) y = g.rl_gate[(C - g.C) + o] * y;
+          C[o] = y;
         } else {
           if (col >= g.N) continue;
           float *p = C + (long)row * g.ldc + col;
@@ -852,5 +883,48 @@ int bdh_launch_decoder_splitk_f32(bdh_ctx *ctx, int M, long K, int d, int KB, co
   hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128), 0,
                      ctx->stream, g);
   BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<decoder split-K>");
+  return BDH_OK;
+}
+
+// relu_lowrank for many rows per (sequence, head) on the f32 matrix cores: one product [T, d] x [d, N] per slice with
+// the k order of a scalar loop (SEQK), so the outputs are the bits of k_relu_lowrank.  mask_dev: one byte per latent
+// block in device memory, or null.
+int bdh_launch_relu_lowrank_gemm(bdh_ctx *ctx, const ReluLowrankParams &p, const unsigned char *mask_dev) {
+  FsaArgs g{};
+  g.A = p.in;
+  g.Bm = p.weight;
+  g.C = p.out;
+  g.mod = p.h;                                   // slice = b * h + head
+  g.a_batch = (long)p.h_in * p.T * p.d;
+  g.a_mod_stride = p.h_in == 1 ? 0 : (long)p.T * p.d;
+  g.b_batch = 0;
+  g.b_mod_stride = (long)p.d * p.N;
+  g.c_batch = (long)p.h * p.T * p.N;
+  g.c_mod_stride = (long)p.T * p.N;
+  g.lda = p.d;
+  g.ldb = p.N;
+  g.ldc = p.N;
+  g.M = p.T;
+  g.N = p.N;
+  g.K = p.d;
+  g.b_div = 1;
+  g.n_slices = p.B * p.h;
+  g.block_size = 1;
+  g.h = p.h;
+  g.rl_bias = p.bias;
+  g.rl_thr = p.threshold;
+  g.rl_mask = mask_dev;
+  g.rl_block = p.block_size > 0 ? p.block_size : 1;
+  g.rl_nblocks = p.n_blocks;
+  g.rl_gate = p.gate;
+  const int groups = (g.n_slices + 7) / 8;
+  // 128 x 128 tiles: K = d is short (a 256 x 256 tile spends as long in its prologue and 256 KiB epilogue as in its
+  // 32 k stages: 12.1 against 10.8 ms for [8192 x 512] x [512 x 131072])
+  g.mt = (p.T + 127) / 128;
+  g.nt = (p.N + 127) / 128;
+  if ((long)8 * groups * g.mt * g.nt > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
+  hipLaunchKernelGGL((k_fsa_gemm_f32<3, false, true, 128, 128, 2, 2, true>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                     ctx->stream, g);
+  BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<relu_lowrank>");
   return BDH_OK;
 }

@@ -131,6 +131,15 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     ctx->opt_lowrank_scalar = value;
     return BDH_OK;
   }
+  if (strcmp(name, "relu_lowrank.gemm_rows") == 0) {
+    ctx->opt_lowrank_gemm_rows = value;
+    return BDH_OK;
+  }
+  if (strcmp(name, "relu_lowrank.mfma_rows") == 0) {
+    if (value < 0) return bdh_fail(ctx, BDH_E_INVAL, "relu_lowrank.mfma_rows takes a row count >= 0 (0 = never)");
+    ctx->opt_lowrank_mfma_rows = value;
+    return BDH_OK;
+  }
   if (strcmp(name, "model.one_launch") == 0) {
     if (value < 0 || value > 2) return bdh_fail(ctx, BDH_E_INVAL, "model.one_launch takes 0, 1 or 2");
     ctx->opt_model_one_launch = value;

@@ -25,6 +25,8 @@ struct bdh_ctx {
   int opt_model_one_launch = 1;  // small model's decode step in one launch: 1 when it pays, 2 whenever it fits, 0 never
   int opt_lowrank_row = 1;     // 0: relu_lowrank with one input row and a small matrix uses the column-per-thread kernel
   int opt_model_phase_batch = 1 << 30;  // two launches per layer for a decode step of at most this many sequences (0: never)
+  int opt_lowrank_gemm_rows = 64;  // relu_lowrank with this many tokens per sequence or more runs as a matrix-core product (0: never)
+  int opt_lowrank_mfma_rows = 8;  // relu_lowrank takes the f32 matrix cores from this many rows on (0: never)
   int opt_lowrank_scalar = 1;  // 0: relu_lowrank with 8 to 63 rows stages its inputs in LDS instead of scalar loads
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on
@@ -132,6 +134,8 @@ struct ReluLowrankParams {
   float *out;
 };
 int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p);
+// the same on the f32 matrix cores for many rows per (sequence, head); csrc/attention_parallel.hip
+int bdh_launch_relu_lowrank_gemm(bdh_ctx *ctx, const ReluLowrankParams &p, const unsigned char *mask_dev);
 int bdh_launch_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);
 // the same for internal many-row use: statistics by wave reduction, not bit-identical to the index-order sums
 int bdh_launch_layer_norm_rows(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);

@@ -4,6 +4,9 @@
 // :346-350, :370-384, :436-449.
 #include "bdh_internal.h"
 
+#include <atomic>
+#include <type_traits>
+
 namespace {
 
 constexpr float kLnEps = 1e-5f;  // src/model/bdh.rs:17
@@ -766,7 +769,176 @@ void launch_relu(hipStream_t st, dim3 grid, size_t lds, const ReluLowrankParams 
                      p.h, p.N, p.bias, p.threshold, mask, p.block_size, p.n_blocks, p.gate, p.out, M);
 }
 
+// ------------------------------------------------------------------------------------
+// relu_lowrank on the f32 matrix cores, for 8 rows and more.  v_mfma_f32_32x32x2_f32 adds its two k-steps one
+// after the other, each as one fused multiply-add, so a chain of these instructions over k = 0, 1, 2, ... is the
+// same k-sequential fmaf chain per output as k_relu_lowrank computes, bit for bit (checked on the device against
+// the scalar chain, including denormal results): the active sets do not change, the weights are streamed once
+// for up to 32 * RT rows, and the arithmetic runs at the matrix rate.
+//   A operand (32 rows x 2 k): lane l holds in[row l % 32][k0 + l / 32], from an LDS copy of the input rows laid
+//   out [k][row]; B operand (2 k x 32 columns): lane l holds w[k0 + l / 32][column].  A lane loads four adjacent
+//   columns of a weight row at once (16 bytes, a wavefront reads two 512-byte row pieces per k-pair) and uses
+//   them in four matrix instructions: instruction j owns the columns n0 + 4 c + j, c = 0..31, so that the four
+//   results a lane holds for a row are again four adjacent columns (16-byte stores).
+// One workgroup = NW wavefronts x 128 columns; grid (column blocks, heads, row groups of 32 * RT).  Each wavefront
+// asks for its first UK k-pairs of weights before the input rows are staged, so the staging hides behind them.
+// ------------------------------------------------------------------------------------
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+template <int RT, int UK, int NW>  // RT row tiles of 32 rows per workgroup; UK k-pairs of weights in flight per wavefront
+__global__ __launch_bounds__(NW * 64) void k_relu_lowrank_mfma(const float *__restrict__ in, int h_in, int T, int d,
+                                                           const float *__restrict__ w, int h, int N,
+                                                           const float *__restrict__ bias, float thr,
+                                                           const unsigned char *__restrict__ block_active,
+                                                           int block_size, int n_blocks,
+                                                           const float *__restrict__ gate, float *__restrict__ out,
+                                                           int M) {
+  extern __shared__ float s_in[];  // [d][32 * RT + 1], zero for rows past M (the odd row stride keeps the
+                                   // transposing writes below and the two k-rows of a read off each other's banks)
+  constexpr int R = 32 * RT, RS = R + 1;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int hh = blockIdx.y;
+  // grid.x = column blocks (rounded up to 8) x row groups: the workgroups that share a block of weight columns
+  // follow each other on one XCD (blockIdx.x % 8 picks the XCD), so the block is fetched from memory once
+  const int row_groups = (M + R - 1) / R;
+  const int xj = blockIdx.x >> 3;
+  const int col_block = (xj / row_groups) * 8 + (blockIdx.x & 7);
+  const int m0 = (xj % row_groups) * R;
+  const int n0 = (col_block * NW + wave) * 128;  // first column of this wavefront
+  const bool wave_ok = n0 < N;
+  const int ncol = n0 + 4 * (lane & 31);          // this lane's four columns ncol .. ncol + 3 (N % 4 == 0)
+  const bool col_ok = ncol < N;
+  const float *wp = w + (long)hh * d * N + (long)(lane >> 5) * N + (col_ok ? ncol : (wave_ok ? n0 : 0));
+  float4 wv[UK];
+#pragma unroll
+  for (int u = 0; u < UK; ++u) wv[u] = *reinterpret_cast<const float4 *>(wp + (long)(2 * u) * N);
+  // the input rows of this group, transposed on the way in: four adjacent k per access (d % 4 == 0), sixteen
+  // accesses of a thread in flight at a time (one at a time, the staging is a chain of trips to the L2)
+  {
+    const int d4 = d >> 2;
+    const int total = R * d4;
+    for (int i0 = 0; i0 < total; i0 += NW * 64 * 16) {
+      float4 v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int i = i0 + u * NW * 64 + tid;
+        const int r = i / d4, k4 = i - r * d4;
+        const int m = m0 + r;
+        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < total && m < M) {
+          const int b = m / T, t = m - b * T;
+          v[u] = *reinterpret_cast<const float4 *>(in + (((long)b * h_in + (h_in == 1 ? 0 : hh)) * T + t) * d + 4 * k4);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int i = i0 + u * NW * 64 + tid;
+        const int r = i / d4, k4 = i - r * d4;
+        if (i < total) {
+          s_in[(4 * k4 + 0) * RS + r] = v[u].x;
+          s_in[(4 * k4 + 1) * RS + r] = v[u].y;
+          s_in[(4 * k4 + 2) * RS + r] = v[u].z;
+          s_in[(4 * k4 + 3) * RS + r] = v[u].w;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (!wave_ok) return;
+  const float *ap = s_in + (lane >> 5) * RS + (lane & 31);
+
+  f32x16_t acc[RT][4];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[rt][j][e] = 0.0f;
+
+  // k-pairs in groups of UK (d is a multiple of 2 * UK): the loop body has no branches, so the loads of the next
+  // group stay in flight across the matrix instructions of this one
+  const int groups = d / (2 * UK);
+  auto group = [&](int g, auto more_t) {
+    constexpr bool MORE = decltype(more_t)::value;
+#pragma unroll
+    for (int u = 0; u < UK; ++u) {
+      const int pr = g * UK + u;
+      const float4 b4 = wv[u];
+      if constexpr (MORE) wv[u] = *reinterpret_cast<const float4 *>(wp + (long)(2 * (pr + UK)) * N);
+      float a[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) a[rt] = ap[(2 * pr) * RS + rt * 32];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        acc[rt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rt], b4.x, acc[rt][0], 0, 0, 0);
+        acc[rt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rt], b4.y, acc[rt][1], 0, 0, 0);
+        acc[rt][2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rt], b4.z, acc[rt][2], 0, 0, 0);
+        acc[rt][3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[rt], b4.w, acc[rt][3], 0, 0, 0);
+      }
+      // keeps the load above where it is: left alone, the scheduler sinks all the loads of a group below its
+      // matrix instructions, and the next group then starts by waiting for every one of them
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  for (int g = 0; g + 1 < groups; ++g) group(g, std::true_type{});
+  group(groups - 1, std::false_type{});
+  if (!col_ok) return;
+
+  float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (bias) bv = *reinterpret_cast<const float4 *>(bias + (long)hh * N + ncol);
+  float mk[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+  if (block_active) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int blk = (ncol + j) / block_size;
+      mk[j] = (blk < n_blocks && block_active[blk]) ? 1.0f : 0.0f;
+    }
+  }
+  const float bvv[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int m = m0 + rt * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+      if (m < M) {
+        const int b = m / T, t = m - b * T;
+        const long o = (((long)b * h + hh) * T + t) * N + ncol;
+        float y[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float pv = acc[rt][j][e];
+          if (bias) pv = pv + bvv[j];
+          if (thr != 0.0f) pv = pv - thr;
+          float yy = pv > 0.0f ? pv : 0.0f;
+          if (block_active) yy = yy * mk[j];
+          y[j] = yy;
+        }
+        if (gate) {
+          const float4 g4 = *reinterpret_cast<const float4 *>(gate + o);
+          y[0] = g4.x * y[0]; y[1] = g4.y * y[1]; y[2] = g4.z * y[2]; y[3] = g4.w * y[3];
+        }
+        *reinterpret_cast<float4 *>(out + o) = make_float4(y[0], y[1], y[2], y[3]);
+      }
+    }
+}
+
 }  // namespace
+
+#ifndef BDH_RL_UK
+#define BDH_RL_UK 16
+#endif
+// lets a kernel take up to 144 KiB of dynamic LDS; once per device
+template <typename K>
+static hipError_t allow_big_lds(K kernel, std::atomic<uint64_t> &configured) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (configured.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+  if (e == hipSuccess) configured.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
   const long M = (long)p.B * p.T;
@@ -783,9 +955,43 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
     }
     mask_dev = static_cast<const unsigned char *>(ctx->ws);
   }
-  // many rows: the 64 x 256 tile (same values, an eighth of the weight traffic)
   const bool aligned16 = bdh_aligned(p.in, 16) && bdh_aligned(p.weight, 16) && bdh_aligned(p.out, 16) &&
                          bdh_aligned(p.bias, 16) && bdh_aligned(p.gate, 16);
+  // 8 to 64 rows (a batch of sequences decoding together): the f32 matrix cores, same values, the weights streamed
+  // once.  (Beyond 64 rows this kernel would stream them once per 64 rows; the 64 x 256 tile kernel below reuses them.)
+  if (M >= ctx->opt_lowrank_mfma_rows && ctx->opt_lowrank_mfma_rows > 0 && M <= 64 && (p.N & 3) == 0 &&
+      (p.d % (2 * BDH_RL_UK)) == 0 && p.d >= 2 * BDH_RL_UK && aligned16) {
+    const int rt = M > 32 ? 2 : 1;
+    const size_t lds = sizeof(float) * (size_t)p.d * (32 * rt + 1);
+    if (lds <= 144 * 1024) {
+      constexpr int UK = BDH_RL_UK;
+      const int nw = rt == 1 ? 2 : 4;  // 64 rows take 133 KiB of LDS at d = 512: one workgroup per CU, so four waves
+      const long row_groups = (M + 32 * rt - 1) / (32 * rt);
+      const long col_blocks8 = ((p.N + nw * 128 - 1) / (nw * 128) + 7) / 8 * 8;
+      if (col_blocks8 * row_groups > 0x7fffffffL || p.h > 65535)
+        return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (row groups %ld)", row_groups);
+      const dim3 grid((unsigned)(col_blocks8 * row_groups), p.h, 1);
+      static std::atomic<uint64_t> cfg1{0}, cfg2{0};
+      if (rt == 1) {
+        BDH_HIP_CHECK(ctx, allow_big_lds(k_relu_lowrank_mfma<1, UK, 2>, cfg1));
+        hipLaunchKernelGGL((k_relu_lowrank_mfma<1, UK, 2>), grid, dim3(128), lds, ctx->stream, p.in, p.h_in, p.T, p.d,
+                           p.weight, p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M);
+      } else {
+        BDH_HIP_CHECK(ctx, allow_big_lds(k_relu_lowrank_mfma<2, UK, 4>, cfg2));
+        hipLaunchKernelGGL((k_relu_lowrank_mfma<2, UK, 4>), grid, dim3(256), lds, ctx->stream, p.in, p.h_in, p.T, p.d,
+                           p.weight, p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M);
+      }
+      BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_mfma");
+      return BDH_OK;
+    }
+  }
+  // many tokens per sequence: one f32 matrix-core product per (sequence, head), same values
+  // (a negative option value -r takes it from r tokens on whatever the grid)
+  const int gemm_rows = ctx->opt_lowrank_gemm_rows;
+  const bool gemm_grid = (long)p.B * p.h * ((p.T + 127) / 128) * ((p.N + 127) / 128) >= (ctx->n_cu > 0 ? ctx->n_cu : 256);
+  if (p.d > 0 && p.N > 0 && (gemm_rows > 0 ? (p.T >= gemm_rows && gemm_grid) : (gemm_rows < 0 && p.T >= -gemm_rows)))
+    return bdh_launch_relu_lowrank_gemm(ctx, p, mask_dev);
+  // many rows: the 64 x 256 tile (same values, an eighth of the weight traffic)
   const long tile_wgs = (long)((p.N / 4 + 63) / 64) * p.h * ((M + 63) / 64);  // enough of them to cover the chip
   if (M >= 64 && ctx->opt_lowrank_tile != 0 && (p.N & 3) == 0 && (p.d & 3) == 0 && p.d > 0 && aligned16 &&
       (ctx->opt_lowrank_tile == 2 || tile_wgs >= (ctx->n_cu > 0 ? ctx->n_cu : 256))) {

@@ -76,6 +76,14 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       0 = always token by token, 1 = dense products for any T.
  *   "state_step.dense_kernel": 1 (default) PoPE and eagerly decayed ALiBi steps at d in {256,512} take
  *                       the dense streaming kernel, 0 = the generic kernel (same values).
+ *   "relu_lowrank.mfma_rows": 8 (default) calls with this many rows and at most 64 (N a multiple of 4, d a
+ *                       multiple of 32) run on the f32 matrix cores, the weights streamed once: a chain of
+ *                       v_mfma_f32_32x32x2_f32 over k is the same k-sequential fused-multiply-add chain per
+ *                       output, bit for bit; 0 = never.
+ *   "relu_lowrank.gemm_rows": 64 (default) calls with this many tokens per sequence or more (and enough tiles to
+ *                       cover the chip) run as one f32 matrix-core product per (sequence, head) with the k order
+ *                       of a scalar loop: the same bits again; 0 = never; a negative value -r takes it from
+ *                       r tokens on whatever the grid.
  *   "relu_lowrank.scalar": 1 (default) calls with 8 to 63 rows read their inputs through the scalar
  *                       cache, 0 = stage them in LDS (same values).
  *   "relu_lowrank.row": 1 (default) a call with one input row, 128 <= d <= 512 and at most 16 MiB of
@@ -90,7 +98,7 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       once) when its tiles cover half the chip; fewer sequences, and small models, take
  *                       the VALU kernel that skips inactive rows of E.  A negative value -r takes the
  *                       matrix-core form from r sequences on whatever the size.
- *   "model.one_launch": 1 (default) a decode step (T = 1, f32 state, no x_tap / viz) of a model that is
+ *   "model.one_launch": 1 (default) a decode step (T = 1, no x_tap / viz) of a model that is
  *                       small enough does not run kernel by kernel: a small model (d <= 256 and d % 4 == 0,
  *                       h * N <= 2048 and a multiple of 32, h in {1,2,4,8,16}, V <= 1024) can take ONE launch
  *                       for the whole step, a workgroup per sequence (always for up to 4 MiB of projection

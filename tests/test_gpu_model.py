@@ -82,11 +82,12 @@ def test_relu_lowrank_single_row_small_matrix_bit_exact(bda, corc, d, N, h, h_in
     assert 0.2 < (ref > 0).mean() < 0.8
 
 
-@pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (8, 1, 1), (17, 1, 4), (32, 1, 1), (1, 64, 4), (2, 100, 1),
-                                      (3, 43, 4)])
+@pytest.mark.parametrize("B,T,h_in", [(1, 1, 1), (3, 1, 1), (2, 5, 4), (8, 1, 1), (17, 1, 4), (32, 1, 1), (33, 1, 1), (1, 64, 4),
+                                      (4, 16, 1), (2, 100, 1), (3, 43, 4)])
 def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
     """One k-sequential FMA chain per output on both sides: values, and therefore the active
-    sets, are identical bit for bit whatever the launch tiling."""
+    sets, are identical bit for bit whatever the launch tiling -- also on the f32 matrix cores, which calls
+    of 8 to 64 rows take by default (a chain of v_mfma_f32_32x32x2_f32 over k is that same chain)."""
     from burn_dragon_amd.kernel import relu_lowrank
 
     h, d, N = 4, 256, 640
@@ -95,21 +96,86 @@ def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
     weight = (0.02 * rng.standard_normal((h, d, N))).astype(np.float32)
     gate = np.maximum(rng.standard_normal((B, h, T, N)), 0).astype(np.float32)
     ref = corc.relu_lowrank(inp, weight)
-    got = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
-                                     bda.BlockPattern1d.dense(64))
+    args = (torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0, bda.BlockPattern1d.dense(64))
+    got = relu_lowrank.fused_forward(*args)
     assert np.array_equal(got.cpu().numpy(), ref)
     assert 0.4 < (ref > 0).mean() < 0.6
     ctx = bda.ffi.default_context(0)
-    try:  # the LDS-staged kernels give the same bits as the scalar-input ones that 8 to 63 rows take by default
+    try:  # the scalar-input kernels (8 to 63 rows) and the LDS-staged ones give the same bits as the matrix cores
+        ctx.set_option("relu_lowrank.mfma_rows", 0)
+        scalar = relu_lowrank.fused_forward(*args)
         ctx.set_option("relu_lowrank.scalar", 0)
-        lds = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
-                                         bda.BlockPattern1d.dense(64))
+        lds = relu_lowrank.fused_forward(*args)
     finally:
         ctx.set_option("relu_lowrank.scalar", 1)
+        ctx.set_option("relu_lowrank.mfma_rows", 8)
+    assert np.array_equal(scalar.cpu().numpy(), ref)
     assert np.array_equal(lds.cpu().numpy(), ref)
-    gated = relu_lowrank.fused_forward(torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), None, 0.0,
-                                       bda.BlockPattern1d.dense(64), gate=torch.from_numpy(gate).to(DEV))
+    gated = relu_lowrank.fused_forward(*args, gate=torch.from_numpy(gate).to(DEV))
     assert np.array_equal(gated.cpu().numpy(), gate * ref)
+
+
+@pytest.mark.parametrize("M,d,N,h_in", [(40, 512, 1024, 1), (64, 512, 520, 2), (9, 64, 132, 1), (32, 128, 4096, 2)])
+def test_relu_lowrank_on_the_matrix_cores_with_every_option(bda, corc, M, d, N, h_in):
+    """The matrix-core projection (8 to 64 rows) with bias, threshold, block mask and gate, one and two row tiles,
+    ragged column counts and wide value ranges (products from 1e-30 to 1e+6, results down to denormals): bit-exact
+    against the oracle's fmaf chain and identical to the VALU kernels."""
+    from burn_dragon_amd.kernel import relu_lowrank
+
+    h = 2
+    rng = np.random.default_rng(M + d + N)
+    inp = (rng.standard_normal((M, h_in, 1, d)) * np.exp2(rng.integers(-40, 10, (M, h_in, 1, d)))).astype(np.float32)
+    weight = (rng.standard_normal((h, d, N)) * np.exp2(rng.integers(-60, 10, (h, d, N)))).astype(np.float32)
+    bias = (0.1 * rng.standard_normal((h, 1, N))).astype(np.float32)
+    gate = np.maximum(rng.standard_normal((M, h, 1, N)), 0).astype(np.float32)
+    blocks = [b for b in range(-(-N // 8)) if b % 3]
+    layout = bda.BlockPattern1d.from_blocks(8, blocks)
+    ref = corc.relu_lowrank(inp, weight, bias.reshape(h, N), 0.01, 8, blocks)
+    args = (torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), torch.from_numpy(bias).to(DEV), 0.01, layout)
+    got = relu_lowrank.fused_forward(*args).cpu().numpy()
+    gated = relu_lowrank.fused_forward(*args, gate=torch.from_numpy(gate).to(DEV)).cpu().numpy()
+    ctx = bda.ffi.default_context(0)
+    try:
+        ctx.set_option("relu_lowrank.mfma_rows", 0)
+        valu = relu_lowrank.fused_forward(*args).cpu().numpy()
+    finally:
+        ctx.set_option("relu_lowrank.mfma_rows", 8)
+    assert np.array_equal(got, ref)
+    assert np.array_equal(valu, ref)
+    assert np.array_equal(gated, gate * ref)
+    assert 0.05 < (ref > 0).mean() < 0.6
+
+
+@pytest.mark.parametrize("B,T,h_in,d,N", [(2, 100, 1, 256, 640), (1, 300, 3, 72, 203), (3, 64, 1, 512, 1024)])
+def test_relu_lowrank_as_a_matrix_core_product_per_sequence(bda, corc, B, T, h_in, d, N):
+    """Many tokens per sequence: one f32 matrix-core product per (sequence, head) whose k order is that of a scalar
+    loop, so the outputs are again the bits of the oracle's fmaf chain -- with bias, threshold, block mask and gate,
+    ragged tiles in rows, columns and k (K = 72 is not a multiple of the 16-wide stage), wide value ranges."""
+    from burn_dragon_amd.kernel import relu_lowrank
+
+    h = 3
+    rng = np.random.default_rng(B + T + N)
+    inp = (rng.standard_normal((B, h_in, T, d)) * np.exp2(rng.integers(-30, 8, (B, h_in, T, d)))).astype(np.float32)
+    weight = (rng.standard_normal((h, d, N)) * np.exp2(rng.integers(-50, 8, (h, d, N)))).astype(np.float32)
+    bias = (0.1 * rng.standard_normal((h, 1, N))).astype(np.float32)
+    gate = np.maximum(rng.standard_normal((B, h, T, N)), 0).astype(np.float32)
+    blocks = [b for b in range(-(-N // 8)) if b % 4]
+    layout = bda.BlockPattern1d.from_blocks(8, blocks)
+    ref = corc.relu_lowrank(inp, weight, bias.reshape(h, N), 0.01, 8, blocks)
+    args = (torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), torch.from_numpy(bias).to(DEV), 0.01, layout)
+    ctx = bda.ffi.default_context(0)
+    try:
+        ctx.set_option("relu_lowrank.gemm_rows", -64)  # whatever the grid
+        got = relu_lowrank.fused_forward(*args).cpu().numpy()
+        gated = relu_lowrank.fused_forward(*args, gate=torch.from_numpy(gate).to(DEV)).cpu().numpy()
+        ctx.set_option("relu_lowrank.gemm_rows", 0)
+        tile = relu_lowrank.fused_forward(*args).cpu().numpy()
+    finally:
+        ctx.set_option("relu_lowrank.gemm_rows", 64)
+    assert np.array_equal(tile, ref)
+    assert np.array_equal(got, ref)
+    assert np.array_equal(gated, gate * ref)
+    assert 0.05 < (ref > 0).mean() < 0.6
 
 
 def test_relu_lowrank_many_rows_with_bias_threshold_and_mask(bda, corc):
