@@ -136,7 +136,6 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     return BDH_OK;
   }
   if (strcmp(name, "relu_lowrank.mfma_rows") == 0) {
-    if (value < 0) return bdh_fail(ctx, BDH_E_INVAL, "relu_lowrank.mfma_rows takes a row count >= 0 (0 = never)");
     ctx->opt_lowrank_mfma_rows = value;
     return BDH_OK;
   }

@@ -804,6 +804,7 @@ __global__ __launch_bounds__(NW * 64) void k_relu_lowrank_mfma(const float *__re
   const int xj = blockIdx.x >> 3;
   const int col_block = (xj / row_groups) * 8 + (blockIdx.x & 7);
   const int m0 = (xj % row_groups) * R;
+  if (col_block * NW * 128 >= N) return;        // a workgroup of the rounding-up: nothing to do (uniform)
   const int n0 = (col_block * NW + wave) * 128;  // first column of this wavefront
   const bool wave_ok = n0 < N;
   const int ncol = n0 + 4 * (lane & 31);          // this lane's four columns ncol .. ncol + 3 (N % 4 == 0)
@@ -959,26 +960,35 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
                          bdh_aligned(p.bias, 16) && bdh_aligned(p.gate, 16);
   // 8 to 64 rows (a batch of sequences decoding together): the f32 matrix cores, same values, the weights streamed
   // once.  (Beyond 64 rows this kernel would stream them once per 64 rows; the 64 x 256 tile kernel below reuses them.)
-  if (M >= ctx->opt_lowrank_mfma_rows && ctx->opt_lowrank_mfma_rows > 0 && M <= 64 && (p.N & 3) == 0 &&
-      (p.d % (2 * BDH_RL_UK)) == 0 && p.d >= 2 * BDH_RL_UK && aligned16) {
-    const int rt = M > 32 ? 2 : 1;
-    const size_t lds = sizeof(float) * (size_t)p.d * (32 * rt + 1);
-    if (lds <= 144 * 1024) {
+  // (a negative option value -r takes it from r rows on whatever the width)
+  const int mf_rows = ctx->opt_lowrank_mfma_rows < 0 ? -ctx->opt_lowrank_mfma_rows : ctx->opt_lowrank_mfma_rows;
+  const bool mf_any_width = ctx->opt_lowrank_mfma_rows < 0;
+  if (mf_rows > 0 && M >= mf_rows && M <= 64 && (p.N & 3) == 0 && (p.d % (2 * BDH_RL_UK)) == 0 &&
+      p.d >= 2 * BDH_RL_UK && aligned16) {
+    // one 32-row tile per workgroup; 33 to 64 rows make two row groups that follow each other on one XCD.  (Two row
+    // tiles per workgroup would stream the weights once for 64 rows too, but need 133 KiB of LDS at d = 512, one
+    // workgroup per CU: a decode step of the reference's large model at B = 64 took 2.5 ms that way against 1.4.)
+    const size_t lds = sizeof(float) * (size_t)p.d * 33;
+    // a wavefront owns 128 columns: only for matrices wide enough to give every CU a wavefront or two (a model with
+    // 256 neurons per head would run on 16 workgroups; it keeps the kernels below)
+    const long row_groups = (M + 31) / 32;
+    const int n_cu_mf = ctx->n_cu > 0 ? ctx->n_cu : 256;
+    const long waves = (long)((p.N + 127) / 128) * p.h * row_groups;
+    if (lds <= 144 * 1024 && (waves >= n_cu_mf || mf_any_width)) {
       constexpr int UK = BDH_RL_UK;
-      const int nw = rt == 1 ? 2 : 4;  // 64 rows take 133 KiB of LDS at d = 512: one workgroup per CU, so four waves
-      const long row_groups = (M + 32 * rt - 1) / (32 * rt);
+      const int nw = waves >= 4L * n_cu_mf ? 2 : 1;
       const long col_blocks8 = ((p.N + nw * 128 - 1) / (nw * 128) + 7) / 8 * 8;
       if (col_blocks8 * row_groups > 0x7fffffffL || p.h > 65535)
         return bdh_fail(ctx, BDH_E_SHAPE, "grid too large (row groups %ld)", row_groups);
       const dim3 grid((unsigned)(col_blocks8 * row_groups), p.h, 1);
       static std::atomic<uint64_t> cfg1{0}, cfg2{0};
-      if (rt == 1) {
-        BDH_HIP_CHECK(ctx, allow_big_lds(k_relu_lowrank_mfma<1, UK, 2>, cfg1));
+      if (nw == 2) {
+        BDH_HIP_CHECK(ctx, allow_big_lds(k_relu_lowrank_mfma<1, UK, 2>, cfg2));
         hipLaunchKernelGGL((k_relu_lowrank_mfma<1, UK, 2>), grid, dim3(128), lds, ctx->stream, p.in, p.h_in, p.T, p.d,
                            p.weight, p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M);
       } else {
-        BDH_HIP_CHECK(ctx, allow_big_lds(k_relu_lowrank_mfma<2, UK, 4>, cfg2));
-        hipLaunchKernelGGL((k_relu_lowrank_mfma<2, UK, 4>), grid, dim3(256), lds, ctx->stream, p.in, p.h_in, p.T, p.d,
+        BDH_HIP_CHECK(ctx, allow_big_lds(k_relu_lowrank_mfma<1, UK, 1>, cfg1));
+        hipLaunchKernelGGL((k_relu_lowrank_mfma<1, UK, 1>), grid, dim3(64), lds, ctx->stream, p.in, p.h_in, p.T, p.d,
                            p.weight, p.h, p.N, p.bias, p.threshold, mask_dev, p.block_size, p.n_blocks, p.gate, p.out, (int)M);
       }
       BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_mfma");

@@ -77,9 +77,10 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *   "state_step.dense_kernel": 1 (default) PoPE and eagerly decayed ALiBi steps at d in {256,512} take
  *                       the dense streaming kernel, 0 = the generic kernel (same values).
  *   "relu_lowrank.mfma_rows": 8 (default) calls with this many rows and at most 64 (N a multiple of 4, d a
- *                       multiple of 32) run on the f32 matrix cores, the weights streamed once: a chain of
- *                       v_mfma_f32_32x32x2_f32 over k is the same k-sequential fused-multiply-add chain per
- *                       output, bit for bit; 0 = never.
+ *                       multiple of 32, enough columns for a wavefront per CU) run on the f32 matrix cores, the
+ *                       weights streamed once per 32 rows: a chain of v_mfma_f32_32x32x2_f32 over k is the same
+ *                       k-sequential fused-multiply-add chain per output, bit for bit; 0 = never; a negative
+ *                       value -r takes it from r rows on whatever the width.
  *   "relu_lowrank.gemm_rows": 64 (default) calls with this many tokens per sequence or more (and enough tiles to
  *                       cover the chip) run as one f32 matrix-core product per (sequence, head) with the k order
  *                       of a scalar loop: the same bits again; 0 = never; a negative value -r takes it from

@@ -101,7 +101,10 @@ def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
     assert np.array_equal(got.cpu().numpy(), ref)
     assert 0.4 < (ref > 0).mean() < 0.6
     ctx = bda.ffi.default_context(0)
-    try:  # the scalar-input kernels (8 to 63 rows) and the LDS-staged ones give the same bits as the matrix cores
+    try:  # the matrix cores (8 to 64 rows; by default only for wide matrices), the scalar-input kernels (8 to 63
+        # rows) and the LDS-staged ones all give the same bits
+        ctx.set_option("relu_lowrank.mfma_rows", -8)
+        mfma = relu_lowrank.fused_forward(*args)
         ctx.set_option("relu_lowrank.mfma_rows", 0)
         scalar = relu_lowrank.fused_forward(*args)
         ctx.set_option("relu_lowrank.scalar", 0)
@@ -109,13 +112,15 @@ def test_relu_lowrank_bit_exact_against_oracle(bda, corc, B, T, h_in):
     finally:
         ctx.set_option("relu_lowrank.scalar", 1)
         ctx.set_option("relu_lowrank.mfma_rows", 8)
+    assert np.array_equal(mfma.cpu().numpy(), ref)
     assert np.array_equal(scalar.cpu().numpy(), ref)
     assert np.array_equal(lds.cpu().numpy(), ref)
     gated = relu_lowrank.fused_forward(*args, gate=torch.from_numpy(gate).to(DEV))
     assert np.array_equal(gated.cpu().numpy(), gate * ref)
 
 
-@pytest.mark.parametrize("M,d,N,h_in", [(40, 512, 1024, 1), (64, 512, 520, 2), (9, 64, 132, 1), (32, 128, 4096, 2)])
+@pytest.mark.parametrize("M,d,N,h_in", [(40, 512, 1024, 1), (64, 512, 520, 2), (9, 64, 132, 1), (32, 128, 4096, 2),
+                                        (17, 64, 16384, 1)])
 def test_relu_lowrank_on_the_matrix_cores_with_every_option(bda, corc, M, d, N, h_in):
     """The matrix-core projection (8 to 64 rows) with bias, threshold, block mask and gate, one and two row tiles,
     ragged column counts and wide value ranges (products from 1e-30 to 1e+6, results down to denormals): bit-exact
@@ -132,10 +137,11 @@ def test_relu_lowrank_on_the_matrix_cores_with_every_option(bda, corc, M, d, N, 
     layout = bda.BlockPattern1d.from_blocks(8, blocks)
     ref = corc.relu_lowrank(inp, weight, bias.reshape(h, N), 0.01, 8, blocks)
     args = (torch.from_numpy(inp).to(DEV), torch.from_numpy(weight).to(DEV), torch.from_numpy(bias).to(DEV), 0.01, layout)
-    got = relu_lowrank.fused_forward(*args).cpu().numpy()
-    gated = relu_lowrank.fused_forward(*args, gate=torch.from_numpy(gate).to(DEV)).cpu().numpy()
     ctx = bda.ffi.default_context(0)
     try:
+        ctx.set_option("relu_lowrank.mfma_rows", -8)  # whatever the width
+        got = relu_lowrank.fused_forward(*args).cpu().numpy()
+        gated = relu_lowrank.fused_forward(*args, gate=torch.from_numpy(gate).to(DEV)).cpu().numpy()
         ctx.set_option("relu_lowrank.mfma_rows", 0)
         valu = relu_lowrank.fused_forward(*args).cpu().numpy()
     finally:
