@@ -998,7 +998,10 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
   // many tokens per sequence: one f32 matrix-core product per (sequence, head), same values
   // (a negative option value -r takes it from r tokens on whatever the grid)
   const int gemm_rows = ctx->opt_lowrank_gemm_rows;
-  const bool gemm_grid = (long)p.B * p.h * ((p.T + 127) / 128) * ((p.N + 127) / 128) >= (ctx->n_cu > 0 ? ctx->n_cu : 256);
+  // (the product kernel deals whole (sequence, head) slices to the 8 XCDs: with fewer than 16 of them half the chip
+  // idles -- config 1 at B = 1, four slices, took 24 ms for a 64-token prompt that way against 14)
+  const bool gemm_grid = (long)p.B * p.h >= 16 &&
+                         (long)p.B * p.h * ((p.T + 127) / 128) * ((p.N + 127) / 128) >= (ctx->n_cu > 0 ? ctx->n_cu : 256);
   if (p.d > 0 && p.N > 0 && (gemm_rows > 0 ? (p.T >= gemm_rows && gemm_grid) : (gemm_rows < 0 && p.T >= -gemm_rows)))
     return bdh_launch_relu_lowrank_gemm(ctx, p, mask_dev);
   // many rows: the 64 x 256 tile (same values, an eighth of the weight traffic)
