@@ -690,17 +690,34 @@ __device__ __forceinline__ void turn_sincos(float turns, float &sn, float &cs) {
   cs = __builtin_amdgcn_cosf(turns);
 }
 
-#ifndef BDH_ST_LOOK
-#define BDH_ST_LOOK 2
-#endif
-constexpr int ST_LOOK = BDH_ST_LOOK;  // k-steps of B fragments in flight (1, 2 or 4)
+constexpr int ST_LOOK = 4;  // k-steps of B fragments in flight (1, 2 or 4): a whole step
 constexpr int ST_TN = 64;
 constexpr int ST_ASTRIDE = ST_TN + 32;           // bf16 per token row of the LDS tile: 48 dwords, the four rows a
                                                  // transposing read touches cover the 64 banks once
 constexpr int ST_A_TILE = 64 * ST_ASTRIDE;       // elements per stage
 constexpr int ST_DUMP_ROW = ST_TN + 8;           // bf16 per staged value row of a state copy (144 bytes)
 constexpr int ST_DUMP_WAVE = 32 * ST_DUMP_ROW;   // a wavefront stages 32 value rows at a time
-constexpr int ST_LDS = (2 * ST_A_TILE + 4 * ST_DUMP_WAVE) * 2;
+constexpr int ST_LDS = (2 * ST_A_TILE + 4 * ST_DUMP_WAVE) * 2 + 64 * 4;  // + the tile's frequencies
+
+// Buffer addressing: a wavefront-uniform descriptor and byte offset in scalar registers plus one constant 32-bit
+// offset per lane, so the token loop keeps no per-lane 64-bit addresses alive and spends no vector arithmetic on
+// them.  Offsets stay below 2 GiB (checked by the host).
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ uint4 buffer_load16(__amdgpu_buffer_rsrc_t r, unsigned int lane_bytes, int uniform_bytes) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_bytes, uniform_bytes, 0);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+// Stores carry the whole offset in the lane's register.  With the uniform part in a scalar offset operand the
+// compiler assumes that a 16-byte store needs no idle cycles before the next write of its data registers; on this
+// chip it does (seen as corrupted state copies when a vector instruction followed the store directly), and with a
+// zero scalar offset the compiler inserts them.
+__device__ __forceinline__ void buffer_store16(uint4 q, __amdgpu_buffer_rsrc_t r, unsigned int lane_bytes, int uniform_bytes) {
+  const u32x4 v = {q.x, q.y, q.z, q.w};
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)(lane_bytes + (unsigned int)uniform_bytes), 0, 0);
+}
 
 template <bool EQ>
 __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigned short *s_dyn) {
@@ -738,10 +755,14 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
     }
   }
   // exact phases (src/model/attention.rs:338-343) at the first tokens of a chunk; 32-token steps inside it
-  auto seed = [&](int token) {
+  // (the tile's frequencies sit in LDS after the prologue: a global load here would make the token loop wait for
+  // every activation and value load in flight)
+  float *s_freq = reinterpret_cast<float *>(s_dyn + 2 * ST_A_TILE + 4 * ST_DUMP_WAVE);
+  auto seed = [&](int token, auto from_lds_t) {
     const float pos = (float)(g.pos0 + token);
-    const float4 f0 = *reinterpret_cast<const float4 *>(g.freqs + n0 + mc);
-    const float4 f1 = *reinterpret_cast<const float4 *>(g.freqs + n0 + mc + 4);
+    const float *fsrc = decltype(from_lds_t)::value ? s_freq + mc : g.freqs + n0 + mc;
+    const float4 f0 = *reinterpret_cast<const float4 *>(fsrc);
+    const float4 f1 = *reinterpret_cast<const float4 *>(fsrc + 4);
     const float fre[4] = {f0.x, f0.z, f1.x, f1.z}, fro[4] = {f0.y, f0.w, f1.y, f1.w};
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
@@ -812,10 +833,11 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
   // read from HBM takes longer than the matrix products of one step)
   uint4 ra[2][2];
   const unsigned int lane_off = (unsigned int)(tk * g.N + mc) * 2u, q_off = (unsigned int)(tk * 64 + mc) * 2u;
+  const __amdgpu_buffer_rsrc_t r_x = buffer_of(X), r_v = buffer_of(Vf), r_q = buffer_of(Qo);
+  const int row_bytes = g.N * 2;
   auto load_piece = [&](int step, auto slot_t, int c) {  // activations of 32 tokens of a step
     constexpr int SLOT = decltype(slot_t)::value;
-    const unsigned short *rowp = X + (long)(step * 64 + c * 32) * g.N;
-    ra[SLOT][c] = *reinterpret_cast<const uint4 *>(at(rowp, lane_off));
+    ra[SLOT][c] = buffer_load16(r_x, lane_off, (step * 64 + c * 32) * row_bytes);
   };
   // B fragments of a step: fb[kk][j] = V[tokens 16 kk + 8 (lane >> 5) .. + 8)[value 64 wave + 32 j + (lane & 31)],
   // 1 KiB of consecutive bytes per wavefront and fragment in the fragment-order copy of V
@@ -823,9 +845,10 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
   bf16x8 fb[ST_LOOK][2];
   const unsigned int vb_off = (unsigned int)(wave * 2 * 4 * 64 + lane) * 16u;
   auto load_b = [&](int step, int kk) {
-    const unsigned short *vp = Vf + (long)step * (64 * 256) + kk * (64 * 8);
+    const int so = (step * (64 * 256) + kk * (64 * 8)) * 2;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) fb[kk % ST_LOOK][j] = *reinterpret_cast<const bf16x8 *>(at(vp + j * (4 * 64 * 8), vb_off));
+    for (int j = 0; j < 2; ++j)
+      fb[kk % ST_LOOK][j] = __builtin_bit_cast(bf16x8, buffer_load16(r_v, vb_off, so + j * (4 * 64 * 8 * 2)));
   };
   auto stage_piece = [&](int step, auto slot_t, int c) {  // rotate, write Q, put the A operand into the stage's LDS tile
     constexpr int SLOT = decltype(slot_t)::value;
@@ -833,15 +856,14 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
     const uint4 q = rotate(ra[SLOT][c]);
     advance();
     const int kr = c * 32 + tk;
-    unsigned short *qrow = Qo + (step * 64 + c * 32) * 64;
-    *reinterpret_cast<uint4 *>(at_w(qrow, q_off)) = q;
+    buffer_store16(q, r_q, q_off, (step * 64 + c * 32) * 64 * 2);
     *reinterpret_cast<uint4 *>(sa + kr * ST_ASTRIDE + (mc ^ (((kr >> 3) & 1) << 5))) = q;
   };
   // bf16 of the accumulators, transposed to [value column][neuron]: each wavefront stages its own 64 value rows,
   // 32 at a time, in LDS rows of its own (LDS operations of one wavefront execute in order: no barrier), and
   // writes them as whole 128-byte row pieces
   auto dump = [&](int slot, bool remainder) {
-    unsigned short *dst = g.P + (long)slot * g.p_slot + (long)slice * g.p_slice + (long)(r % nt) * (256 * 64);
+    const __amdgpu_buffer_rsrc_t r_p = buffer_of(g.P + (long)slot * g.p_slot + (long)slice * g.p_slice + (long)(r % nt) * (256 * 64));
     const unsigned int dst_off = (unsigned int)((wave * 64 + (lane >> 3)) * 64 + (lane & 7) * 8) * 2u;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -865,8 +887,8 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
         }
 #pragma unroll
       for (int pass = 0; pass < 4; ++pass)
-        *reinterpret_cast<uint4 *>(at_w(dst + (j * 32 + pass * 8) * 64, dst_off)) =
-            *reinterpret_cast<const uint4 *>(s_stage + (pass * 8 + (lane >> 3)) * ST_DUMP_ROW + (lane & 7) * 8);
+        buffer_store16(*reinterpret_cast<const uint4 *>(s_stage + (pass * 8 + (lane >> 3)) * ST_DUMP_ROW + (lane & 7) * 8),
+                       r_p, dst_off, (j * 32 + pass * 8) * 64 * 2);
     }
   };
 
@@ -875,11 +897,14 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
   // it let the loads of the next step, the Q stores and the state copies stay in flight across the matrix
   // products instead of draining them at every join.  Tc is a multiple of 256 here.
   const int nc = g.Tc / 256;
-  // step kt = 4 c + S_: staging of step kt + 1 (MORE), fetch of the activations of step kt + 3 (MORE3) into the
-  // registers the staging just freed, then the matrix products of step kt from LDS tile S_ & 1.  (Placing the
-  // rotation inside the product regions, with the A fragments read one k-step ahead, measured 12 % slower: the
-  // Q stores and activation loads then sit between the B-fragment loads, and with one in-order memory counter
-  // every wait for a fragment becomes a wait for them.)
+  // step kt = 4 c + S_: staging of step kt + 1 (MORE), then the matrix products of step kt from LDS tile S_ & 1.
+  // Memory operations of a wavefront complete in issue order, so a wait for a value fragment is also a wait for
+  // every load and store issued before it.  Hence the order below: value fragments a whole step ahead (ST_LOOK = 4),
+  // and the activations of step kt + 3 (MORE3; from HBM, the slowest) requested only after the third k-step's
+  // fragment loads, into the registers the staging freed: the first wait that covers them is then a full step
+  // away.  (Requested at the start of the step they stalled the second half of the same step's products;
+  // fragments two k-steps ahead left every k-step waiting on the L2 latency.  Placing the rotation inside the
+  // product regions or reading the A fragments one k-step ahead gained nothing.)
   auto step = [&](int kt, auto s_t, auto more_t, auto more3_t) {
     constexpr int S_ = decltype(s_t)::value;
     constexpr bool MORE = decltype(more_t)::value, MORE3 = decltype(more3_t)::value;
@@ -887,10 +912,7 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
     const unsigned short *s_a = s_dyn + (S_ & 1) * ST_A_TILE;
     if constexpr (MORE) {
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        stage_piece(kt + 1, Next{}, c);
-        if constexpr (MORE3) load_piece(kt + 3, Next{}, c);
-      }
+      for (int c = 0; c < 2; ++c) stage_piece(kt + 1, Next{}, c);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -922,6 +944,13 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
       if (kk + ST_LOOK < 4) load_b(kt, kk + ST_LOOK);
       else if constexpr (MORE) load_b(kt + 1, kk + ST_LOOK - 4);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (MORE3) {
+        if (kk == 2) {
+#pragma unroll
+          for (int c = 0; c < 2; ++c) load_piece(kt + 3, Next{}, c);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
     }
     lds_barrier();
   };
@@ -934,7 +963,7 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
     step(kt, std::integral_constant<int, 0>{}, T{}, T{});
     step(kt + 1, std::integral_constant<int, 1>{}, T{}, NotLast{});
     step(kt + 2, std::integral_constant<int, 2>{}, T{}, NotLast{});
-    if constexpr (!LAST) seed((kt + 4) * 64 + tk);  // the next step opens a chunk: exact phases
+    if constexpr (!LAST) seed((kt + 4) * 64 + tk, std::true_type{});  // the next step opens a chunk: exact phases
     step(kt + 3, std::integral_constant<int, 3>{}, NotLast{}, NotLast{});
   };
 
@@ -946,7 +975,8 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
   using Slot1 = std::integral_constant<int, 1>;
 #pragma unroll
   for (int c = 0; c < 2; ++c) load_piece(0, Slot0{}, c);
-  seed(tk);
+  if (tid < 64) s_freq[tid] = g.freqs[n0 + tid];
+  seed(tk, std::false_type{});
 #pragma unroll
   for (int c = 0; c < 2; ++c) {
     stage_piece(0, Slot0{}, c);
@@ -1156,6 +1186,8 @@ static int prefill_pass_chunks(bdh_ctx *ctx, int B, int h, int Tc, int N, const 
   int *flag = reinterpret_cast<int *>(ws + q_bytes + p_bytes + 2 * vt_bytes);
   const int groups = (S + 7) / 8;
   if ((long)groups * 8 * std::max(N / ST_TN, nc) > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
+  // k_state_stream addresses a slice's activations by 32-bit byte offsets
+  if ((long)Tc * N * 2 > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "pass too long for 32-bit offsets (Tc=%d N=%d)", Tc, N);
 
   hipLaunchKernelGGL(k_transpose_to_bf16<unsigned short>, dim3(d / 64, Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16,
                      Vt, Tc, d, Tc, v_batch);
