@@ -217,6 +217,34 @@ def test_prefill_chunk_recurrent_form(bda, corc, T, N, chunk, rho0_scale, positi
     assert d_out < 2e-2 and d_rho < 5e-3, (d_out, d_rho)
 
 
+@pytest.mark.parametrize("T,N,rho0_scale,position,hilo", [(768, 256, 0.0, 0, False), (1024, 512, 0.05, 41, True)])
+def test_prefill_chunk_recurrent_form_with_unequal_pair_frequencies(bda, corc, T, N, rho0_scale, position, hilo):
+    """A frequency table whose two elements of a lane pair differ (not what build_freqs makes, but what the ABI
+    accepts): the state-update kernel then runs its second instantiation, with separate phases for the even and the
+    odd element (src/model/attention.rs:305-321 takes cos/sin per element).  Against the sequential oracle and the
+    all-scores form."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h, d = 1, 2, 256
+    x, v, rho0 = _prefill_case(5 * T + N, B, h, T, N, d, 0.2, rho0_scale)
+    freqs = corc.build_freqs(N).copy()
+    freqs[1::2] *= np.float32(1.25)
+    q = corc.rotate(x.float().numpy(), freqs, orc.ROPE, position)
+    out_ref, rho_ref = corc.recurrent_attention(q, v.float().numpy(), rho0.numpy(), sparse=True)
+    ft = torch.from_numpy(freqs).to(DEV)
+    rho = rho0.clone().to(DEV)
+    print(f"chunk-recurrent prefill, unequal pair frequencies T={T} N={N} hilo={hilo}", flush=True)
+    out = prefill_chunked(x.to(DEV), v.to(DEV), rho, ft, position, state_is_zero=(rho0_scale == 0.0), hilo=hilo)
+    torch.cuda.synchronize()
+    e_out, e_rho = rel_err(out.cpu().numpy(), out_ref), rel_err(rho.cpu().numpy(), rho_ref)
+    print(f"   out rel err {e_out:.2e}, state rel err {e_rho:.2e}")
+    assert e_out < 2e-2 and e_rho < 2e-2
+    rho_s = rho0.clone().to(DEV)
+    out_s = prefill_chunked(x.to(DEV), v.to(DEV), rho_s, ft, position, state_is_zero=(rho0_scale == 0.0), all_scores=True)
+    d_out, d_rho = rel_err(out.cpu().numpy(), out_s.cpu().numpy()), rel_err(rho.cpu().numpy(), rho_s.cpu().numpy())
+    assert d_out < 2e-2 and d_rho < 5e-3, (d_out, d_rho)
+
+
 def test_prefill_in_four_calls_equals_one_call(bda, corc):
     """One prompt fed as four successive calls (the state carried in the caller's f32 rho, entering each call's
     product as a bf16 pair) against the sequential oracle and against the single call: T = 4096 in chunks of 512."""
@@ -269,15 +297,20 @@ def test_prefill_chunked_then_decode_steps_continue_the_state(bda, corc):
     assert rel_err(rho.cpu().numpy(), rho_ref) < 2e-2
 
 
-def test_prefill_chunked_config3_shape_properties(bda, corc):
+@pytest.mark.parametrize("unequal_pairs", [False, True])
+def test_prefill_chunked_config3_shape_properties(bda, corc, unequal_pairs):
     """BASELINE config 3 per-slice shape (T=2048, N=8192, d=256, 5 % density) on a reduced batch
     (B=1, h=2) so the oracle finishes in seconds.  Checks against the sequential oracle and the
-    size-independent closed forms (first row zero, final state == Q^T V)."""
+    size-independent closed forms (first row zero, final state == Q^T V).  At this width two workgroups share a
+    compute unit, which the small shapes above never reach; the second case takes the kernel instantiation for
+    frequency tables whose pair elements differ."""
     from burn_dragon_amd.recurrent import prefill_chunked
 
     B, h, T, N, d = 1, 2, 2048, 8192, 256
     x, v, _ = _prefill_case(11, B, h, T, N, d, 0.05, 0.0)
-    freqs = corc.build_freqs(N)
+    freqs = corc.build_freqs(N).copy()
+    if unequal_pairs:
+        freqs[1::2] *= np.float32(1.25)
     rho = torch.zeros((B, h, N, d), device=DEV)
     out = prefill_chunked(x.to(DEV), v.to(DEV), rho, torch.from_numpy(freqs).to(DEV), 0, state_is_zero=True)
     torch.cuda.synchronize()
