@@ -635,7 +635,7 @@ struct StateUpdArgs {
   long x_slice;
   unsigned short *Q;         // [S][N/64][Tc][64] out: bf16(rope(x))
   long q_slice;
-  const unsigned short *Vf;  // [B][Tc/64][8][4][64][8]: V in B-fragment order (k_v_fragments), batch stride vt_batch
+  const unsigned short *Vf;  // [B][Tc/64][8][4][64][8]: V in B-fragment order (k_v_layouts), batch stride vt_batch
   long vt_batch;
   const float *freqs;        // [N]
   float *rho;                // [S][N][256] in/out
@@ -645,14 +645,18 @@ struct StateUpdArgs {
   int N, Tc, h, n_slices;
   int has_state;             // the accumulators start from rho, and slot 0 is written
   int lo_slot;               // >= 0: bf16(rho_0 - float(bf16(rho_0))) goes to that slot
-  const int *pairs_equal;    // device flag written by k_freq_pairs_equal
+  const int *pairs_equal;    // device flag written by k_v_layouts
 };
 
-// V of a pass in the order the state update's B operand is consumed: Vf[b][step][dt][kk][lane][8] holds
-// V[b][token 64 step + 16 kk + 8 (lane >> 5) + e][value 32 dt + (lane & 31)], so that one fragment load of a
-// wavefront is 1 KiB of consecutive bytes.  in: [B][Tc][256] bf16 (batch stride in_batch), Tc a multiple of 64.
-__global__ __launch_bounds__(256) void k_v_fragments(const unsigned short *__restrict__ in, long in_batch,
-                                                     unsigned short *__restrict__ out, int Tc) {
+// The layouts of V that a pass consumes, and the frequency table's flag, in one launch.
+// Vf[b][step][dt][kk][lane][8] holds V[b][token 64 step + 16 kk + 8 (lane >> 5) + e][value 32 dt + (lane & 31)]: the
+// order the state update's B operand is consumed in, one fragment load of a wavefront = 1 KiB of consecutive bytes.
+// Vt[b][value][token] is V^T, the B operand of the score-times-value product.  in: [B][Tc][256] bf16 (batch stride
+// in_batch), Tc a multiple of 64.  Workgroup (0, 0) also writes flag[0] = 1 when the two elements of every lane pair
+// share a frequency (what build_freqs makes), else 0.
+__global__ __launch_bounds__(256) void k_v_layouts(const unsigned short *__restrict__ in, long in_batch,
+                                                   unsigned short *__restrict__ vf, unsigned short *__restrict__ vt, int Tc,
+                                                   const float *__restrict__ freqs, int N, int *__restrict__ flag) {
   __shared__ unsigned short s_v[64][256 + 2];
   const int step = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const unsigned short *src = in + (long)b * in_batch + (long)step * 64 * 256;
@@ -663,7 +667,7 @@ __global__ __launch_bounds__(256) void k_v_fragments(const unsigned short *__res
     s_v[t][c2 + 1] = (unsigned short)(v >> 16);
   }
   __syncthreads();
-  unsigned short *dst = out + ((long)b * (Tc / 64) + step) * (64 * 256);
+  unsigned short *dst = vf + ((long)b * (Tc / 64) + step) * (64 * 256);
   for (int piece = tid; piece < 8 * 4 * 64; piece += 256) {
     const int lane = piece & 63, kk = (piece >> 6) & 3, dt = piece >> 8;
     const int t0 = kk * 16 + (lane >> 5) * 8, c = dt * 32 + (lane & 31);
@@ -672,17 +676,35 @@ __global__ __launch_bounds__(256) void k_v_fragments(const unsigned short *__res
     for (int e = 0; e < 4; ++e) w[e] = (unsigned int)s_v[t0 + 2 * e][c] | ((unsigned int)s_v[t0 + 2 * e + 1][c] << 16);
     *reinterpret_cast<uint4 *>(dst + (long)piece * 8) = make_uint4(w[0], w[1], w[2], w[3]);
   }
+  // V^T: value row c, tokens 64 step + 8 t8 .. + 8 (16 bytes); eight consecutive threads write one 128-byte row piece
+  unsigned short *dt_ = vt + (long)b * 256 * Tc + step * 64;
+  for (int piece = tid; piece < 256 * 8; piece += 256) {
+    const int c = piece >> 3, t8 = (piece & 7) * 8;
+    unsigned int w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = (unsigned int)s_v[t8 + 2 * e][c] | ((unsigned int)s_v[t8 + 2 * e + 1][c] << 16);
+    *reinterpret_cast<uint4 *>(dt_ + (long)c * Tc + t8) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    int ok = 1;
+    for (int p = tid; p < N / 2; p += 256) {
+      const float2 f = reinterpret_cast<const float2 *>(freqs)[p];
+      ok &= f.x == f.y;
+    }
+    ok = __syncthreads_and(ok);
+    if (tid == 0) flag[0] = ok;
+  }
 }
 
 // ---- the state update as a streaming kernel ---------------------------------------------------------------------
-// The same work as state_update_body in workgroups of four wavefronts that own 64 neurons x 256 value columns of a
-// slice's state (wavefront w: value columns 64w..64w+63, accumulators in 64 registers).  The update moves ~3 GiB
-// through HBM at the headline shape and needs ~0.14 ms of matrix-core time: it is a memory stream, so it is
-// laid out for many independent workgroups per CU (three or four, against one of the 256-neuron tile) whose loads,
-// stores, rotations and matrix products overlap each other, instead of for operand reuse.  Per 64-token step a
-// workgroup reads a [64 tokens x 64 neurons] tile of x (128-byte row pieces), rotates it in registers, stores Q,
-// keeps the tile in LDS for the transposing reads of the A operand; the B operand (V^T, L2-resident) goes straight
-// from global memory into registers, one step ahead, in the registers the matrix instructions just consumed.
+// Workgroups of four wavefronts own 64 neurons x 256 value columns of a slice's state (wavefront w: value columns
+// 64w..64w+63, accumulators in 64 registers), two workgroups per CU.  The update moves ~3.5 GiB through HBM at the
+// headline shape and needs ~0.11 ms of matrix-core time: it is a memory stream, laid out for many independent
+// workgroups whose loads, stores, rotations and matrix products overlap each other, not for operand reuse.  Per
+// 64-token step a workgroup reads a [64 tokens x 64 neurons] tile of x (128-byte row pieces), rotates it in
+// registers, stores Q, keeps the tile in LDS for the transposing reads of the A operand; the B operand (V in
+// fragment order, L2-resident) goes straight from global memory into the registers the matrix instructions just
+// consumed, a whole step ahead.
 // sine and cosine of a fraction of a turn in [0, 1): the hardware instructions take their argument in turns
 // (absolute error below 2e-6 on that interval), no range reduction and no branches
 __device__ __forceinline__ void turn_sincos(float turns, float &sn, float &cs) {
@@ -1014,22 +1036,11 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
 #ifndef BDH_ST_WAVES
 #define BDH_ST_WAVES 2
 #endif
-template <bool EQ>
+// one launch for both kinds of frequency table: the flag k_v_layouts wrote picks the body (uniform over the grid)
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BDH_ST_WAVES, BDH_ST_WAVES))) void k_state_stream(StateUpdArgs g) {
   extern __shared__ __attribute__((aligned(1024))) unsigned short s_dyn[];
-  if ((g.pairs_equal[0] != 0) != EQ) return;
-  state_stream_body<EQ>(g, s_dyn);
-}
-
-// flag[0] = 1 when the two elements of every lane pair share a frequency (what build_freqs makes), else 0
-__global__ __launch_bounds__(256) void k_freq_pairs_equal(const float *__restrict__ freqs, int N, int *__restrict__ flag) {
-  int ok = 1;
-  for (int p = threadIdx.x; p < N / 2; p += 256) {
-    const float2 f = reinterpret_cast<const float2 *>(freqs)[p];
-    ok &= f.x == f.y;
-  }
-  ok = __syncthreads_and(ok);
-  if (threadIdx.x == 0) flag[0] = ok;
+  if (g.pairs_equal[0] != 0) state_stream_body<true>(g, s_dyn);
+  else state_stream_body<false>(g, s_dyn);
 }
 
 template <bool AK, int EPI>
@@ -1189,17 +1200,11 @@ static int prefill_pass_chunks(bdh_ctx *ctx, int B, int h, int Tc, int N, const 
   // k_state_stream addresses a slice's activations by 32-bit byte offsets
   if ((long)Tc * N * 2 > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "pass too long for 32-bit offsets (Tc=%d N=%d)", Tc, N);
 
-  hipLaunchKernelGGL(k_transpose_to_bf16<unsigned short>, dim3(d / 64, Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16,
-                     Vt, Tc, d, Tc, v_batch);
-  BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<V>");
-  hipLaunchKernelGGL(k_v_fragments, dim3(Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16, v_batch, Vf, Tc);
-  BDH_LAUNCH_CHECK(ctx, "k_v_fragments");
-  hipLaunchKernelGGL(k_freq_pairs_equal, dim3(1), dim3(256), 0, ctx->stream, freqs, N, flag);
-  BDH_LAUNCH_CHECK(ctx, "k_freq_pairs_equal");
+  hipLaunchKernelGGL(k_v_layouts, dim3(Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16, v_batch, Vf, Vt, Tc, freqs, N, flag);
+  BDH_LAUNCH_CHECK(ctx, "k_v_layouts");
   {
-    static std::atomic<uint64_t> configured_eq{0}, configured_ne{0};
-    BDH_HIP_CHECK(ctx, allow_lds(k_state_stream<true>, ST_LDS, configured_eq));
-    BDH_HIP_CHECK(ctx, allow_lds(k_state_stream<false>, ST_LDS, configured_ne));
+    static std::atomic<uint64_t> configured_st{0};
+    BDH_HIP_CHECK(ctx, allow_lds(k_state_stream, ST_LDS, configured_st));
     StateUpdArgs g{};
     g.X = x_bf16; g.x_slice = x_slice;
     g.Q = Q; g.q_slice = (long)Tc * N;
@@ -1211,8 +1216,7 @@ static int prefill_pass_chunks(bdh_ctx *ctx, int B, int h, int Tc, int N, const 
     g.has_state = state_is_zero ? 0 : 1; g.lo_slot = lo_slot;
     g.pairs_equal = flag;
     const int nts = N / ST_TN;
-    hipLaunchKernelGGL(k_state_stream<true>, dim3(8 * groups * nts), dim3(256), ST_LDS, ctx->stream, g);
-    hipLaunchKernelGGL(k_state_stream<false>, dim3(8 * groups * nts), dim3(256), ST_LDS, ctx->stream, g);
+    hipLaunchKernelGGL(k_state_stream, dim3(8 * groups * nts), dim3(256), ST_LDS, ctx->stream, g);
     BDH_LAUNCH_CHECK(ctx, "k_state_stream");
   }
   {
