@@ -657,18 +657,19 @@ struct StateUpdArgs {
 __global__ __launch_bounds__(256) void k_v_layouts(const unsigned short *__restrict__ in, long in_batch,
                                                    unsigned short *__restrict__ vf, unsigned short *__restrict__ vt, int Tc,
                                                    const float *__restrict__ freqs, int N, int *__restrict__ flag) {
-  __shared__ unsigned short s_v[64][256 + 2];
-  const int step = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
-  const unsigned short *src = in + (long)b * in_batch + (long)step * 64 * 256;
-  for (int i = tid; i < 64 * 128; i += 256) {  // two bf16 per access
-    const int t = i >> 7, c2 = (i & 127) * 2;
+  // a workgroup takes 64 tokens x 64 value columns (quarter q of the 256)
+  __shared__ unsigned short s_v[64][64 + 2];
+  const int step = blockIdx.x, b = blockIdx.y, q = blockIdx.z, tid = threadIdx.x;
+  const unsigned short *src = in + (long)b * in_batch + (long)step * 64 * 256 + q * 64;
+  for (int i = tid; i < 64 * 32; i += 256) {  // two bf16 per access
+    const int t = i >> 5, c2 = (i & 31) * 2;
     const unsigned int v = *reinterpret_cast<const unsigned int *>(src + t * 256 + c2);
     s_v[t][c2] = (unsigned short)(v & 0xffffu);
     s_v[t][c2 + 1] = (unsigned short)(v >> 16);
   }
   __syncthreads();
-  unsigned short *dst = vf + ((long)b * (Tc / 64) + step) * (64 * 256);
-  for (int piece = tid; piece < 8 * 4 * 64; piece += 256) {
+  unsigned short *dst = vf + ((long)b * (Tc / 64) + step) * (64 * 256) + (long)q * (2 * 4 * 64 * 8);
+  for (int piece = tid; piece < 2 * 4 * 64; piece += 256) {
     const int lane = piece & 63, kk = (piece >> 6) & 3, dt = piece >> 8;
     const int t0 = kk * 16 + (lane >> 5) * 8, c = dt * 32 + (lane & 31);
     unsigned int w[4];
@@ -677,15 +678,15 @@ __global__ __launch_bounds__(256) void k_v_layouts(const unsigned short *__restr
     *reinterpret_cast<uint4 *>(dst + (long)piece * 8) = make_uint4(w[0], w[1], w[2], w[3]);
   }
   // V^T: value row c, tokens 64 step + 8 t8 .. + 8 (16 bytes); eight consecutive threads write one 128-byte row piece
-  unsigned short *dt_ = vt + (long)b * 256 * Tc + step * 64;
-  for (int piece = tid; piece < 256 * 8; piece += 256) {
+  unsigned short *dt_ = vt + ((long)b * 256 + q * 64) * Tc + step * 64;
+  for (int piece = tid; piece < 64 * 8; piece += 256) {
     const int c = piece >> 3, t8 = (piece & 7) * 8;
     unsigned int w[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) w[e] = (unsigned int)s_v[t8 + 2 * e][c] | ((unsigned int)s_v[t8 + 2 * e + 1][c] << 16);
     *reinterpret_cast<uint4 *>(dt_ + (long)c * Tc + t8) = make_uint4(w[0], w[1], w[2], w[3]);
   }
-  if (blockIdx.x == 0 && blockIdx.y == 0) {
+  if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
     int ok = 1;
     for (int p = tid; p < N / 2; p += 256) {
       const float2 f = reinterpret_cast<const float2 *>(freqs)[p];
@@ -1200,7 +1201,7 @@ static int prefill_pass_chunks(bdh_ctx *ctx, int B, int h, int Tc, int N, const 
   // k_state_stream addresses a slice's activations by 32-bit byte offsets
   if ((long)Tc * N * 2 > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "pass too long for 32-bit offsets (Tc=%d N=%d)", Tc, N);
 
-  hipLaunchKernelGGL(k_v_layouts, dim3(Tc / 64, B), dim3(256), 0, ctx->stream, v_bf16, v_batch, Vf, Vt, Tc, freqs, N, flag);
+  hipLaunchKernelGGL(k_v_layouts, dim3(Tc / 64, B, 4), dim3(256), 0, ctx->stream, v_bf16, v_batch, Vf, Vt, Tc, freqs, N, flag);
   BDH_LAUNCH_CHECK(ctx, "k_v_layouts");
   {
     static std::atomic<uint64_t> configured_st{0};
