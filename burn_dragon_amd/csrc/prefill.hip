@@ -977,12 +977,12 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
     }
     lds_barrier();
   };
-  auto chunk = [&](int c, auto dump_t, auto last_t) {
-    constexpr bool DUMP = decltype(dump_t)::value, LAST = decltype(last_t)::value;
+  auto chunk = [&](int c, auto last_t) {
+    constexpr bool LAST = decltype(last_t)::value;
     using T = std::true_type;
     using NotLast = std::integral_constant<bool, !LAST>;
     const int kt = 4 * c;
-    if constexpr (DUMP) dump(c, false);
+    if (c != 0) dump(c, false);  // (slot 0 is the carried-in state, written in the prologue)
     step(kt, std::integral_constant<int, 0>{}, T{}, T{});
     step(kt + 1, std::integral_constant<int, 1>{}, T{}, NotLast{});
     step(kt + 2, std::integral_constant<int, 2>{}, T{}, NotLast{});
@@ -1010,14 +1010,9 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
 #pragma unroll
   for (int kk = 0; kk < ST_LOOK; ++kk) load_b(0, kk);
   lds_barrier();
-  if (nc == 1) {
-    chunk(0, std::false_type{}, std::true_type{});
-  } else {
-    chunk(0, std::false_type{}, std::false_type{});
 #pragma unroll 1
-    for (int c = 1; c + 1 < nc; ++c) chunk(c, std::true_type{}, std::false_type{});
-    chunk(nc - 1, std::true_type{}, std::true_type{});
-  }
+  for (int c = 0; c + 1 < nc; ++c) chunk(c, std::false_type{});
+  chunk(nc - 1, std::true_type{});
   // the addresses of the final stores equal those of the initial loads: hidden from the compiler here, or it
   // keeps all of them in registers across the token loop
   asm volatile("" : "+s"(rho));
