@@ -825,8 +825,8 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
     return make_uint4(o[0], o[1], o[2], o[3]);
   };
 
-  // every global access below is a wavefront-uniform base (scalar registers) plus this lane's unsigned 32-bit
-  // byte offset: no 64-bit address arithmetic per lane, no address registers kept alive across steps
+  // the state's loads and stores (outside the token loop) are a wavefront-uniform base plus this lane's unsigned
+  // 32-bit byte offset; the accesses of the token loop go through buffer descriptors (buffer_of)
   auto at = [](const void *base, unsigned int byte_off) { return static_cast<const char *>(base) + byte_off; };
   auto at_w = [](void *base, unsigned int byte_off) { return static_cast<char *>(base) + byte_off; };
   // accumulators: rows = neurons 32 i + 8 (e >> 2) + 4 (lane >> 5) + (e & 3), column = value 64 wave + 32 j + (lane & 31)
@@ -852,8 +852,8 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
   }
 
-  // activations: two steps ahead of their use, in two register slots that alternate by step parity (under load a
-  // read from HBM takes longer than the matrix products of one step)
+  // activations: requested in the middle of step kt for the staging at the start of step kt + 2, in two register
+  // slots that alternate by step parity (under load a read from HBM takes longer than the matrix products of a step)
   uint4 ra[2][2];
   const unsigned int lane_off = (unsigned int)(tk * g.N + mc) * 2u, q_off = (unsigned int)(tk * 64 + mc) * 2u;
   const __amdgpu_buffer_rsrc_t r_x = buffer_of(X), r_v = buffer_of(Vf), r_q = buffer_of(Qo);
