@@ -996,19 +996,21 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
   }
   using Slot0 = std::integral_constant<int, 0>;
   using Slot1 = std::integral_constant<int, 1>;
+  // every load the first step needs goes out before anything waits: the activations of steps 0 and 1, the value
+  // fragments of step 0 (the first wait, for the activations of step 0, leaves the others in flight)
 #pragma unroll
   for (int c = 0; c < 2; ++c) load_piece(0, Slot0{}, c);
+#pragma unroll
+  for (int c = 0; c < 2; ++c) load_piece(1, Slot1{}, c);
+#pragma unroll
+  for (int kk = 0; kk < ST_LOOK; ++kk) load_b(0, kk);
+  __builtin_amdgcn_sched_barrier(0);
   if (tid < 64) s_freq[tid] = g.freqs[n0 + tid];
   seed(tk, std::false_type{});
 #pragma unroll
-  for (int c = 0; c < 2; ++c) {
-    stage_piece(0, Slot0{}, c);
-    load_piece(1, Slot1{}, c);
-  }
+  for (int c = 0; c < 2; ++c) stage_piece(0, Slot0{}, c);
 #pragma unroll
   for (int c = 0; c < 2; ++c) load_piece(2, Slot0{}, c);
-#pragma unroll
-  for (int kk = 0; kk < ST_LOOK; ++kk) load_b(0, kk);
   lds_barrier();
 #pragma unroll 1
   for (int c = 0; c + 1 < nc; ++c) chunk(c, std::false_type{});
