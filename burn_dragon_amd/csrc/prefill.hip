@@ -449,6 +449,9 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
 // t * a_kstride (b_kstride) elements further on (64 for a plain row-major operand; a panel stored tile by tile,
 // [k / 64][row][64], has row stride 64 and the tile size as the k-tile stride).  Ends with every wave past its
 // last LDS read.  SAME: B is A (a diagonal score tile), loaded once.
+// cache policy of the operand copies of direct_mainloop: streaming (in the chunk-recurrent form every tile is used
+// once: k_chunk_out 560 -> 545 us)
+constexpr int BDH_K2_LOAD_AUX = 2;
 template <bool SAME>
 __device__ __forceinline__ void direct_mainloop(f32x16 (&acc)[4][2], const unsigned short *A_rows, long lda,
                                                 long a_kstride, const unsigned short *B_rows, long ldb,
@@ -468,10 +471,10 @@ __device__ __forceinline__ void direct_mainloop(f32x16 (&acc)[4][2], const unsig
   _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                                   \
     const int bi = c * 8 + wave;                                                                                    \
     __builtin_amdgcn_global_load_lds((gptr_t)(pa[c] + ((k0) >> 6) * a_kstride),                                      \
-                                     (lptr_t)(s_dyn + (buf)*BUF + bi * 512), 16, 0, 0);                             \
+                                     (lptr_t)(s_dyn + (buf)*BUF + bi * 512), 16, 0, BDH_K2_LOAD_AUX);                             \
     if (!SAME)                                                                                                      \
       __builtin_amdgcn_global_load_lds((gptr_t)(pb[c] + ((k0) >> 6) * b_kstride),                                    \
-                                       (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, 0);                    \
+                                       (lptr_t)(s_dyn + (buf)*BUF + TILE + bi * 512), 16, 0, BDH_K2_LOAD_AUX);                    \
   }
   BDH_ISSUE(0, 0)
   __builtin_amdgcn_s_waitcnt(0);
@@ -729,8 +732,9 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7fffffff, 0x00020000);
 }
+template <int AUX = 0>
 __device__ __forceinline__ uint4 buffer_load16(__amdgpu_buffer_rsrc_t r, unsigned int lane_bytes, int uniform_bytes) {
-  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_bytes, uniform_bytes, 0);
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_bytes, uniform_bytes, AUX);
   return make_uint4(v[0], v[1], v[2], v[3]);
 }
 // Stores carry the whole offset in the lane's register.  With the uniform part in a scalar offset operand the
@@ -862,7 +866,8 @@ __device__ __forceinline__ void state_stream_body(const StateUpdArgs &g, unsigne
   const int row_bytes = g.N * 2;
   auto load_piece = [&](int step, auto slot_t, int c) {  // activations of 32 tokens of a step
     constexpr int SLOT = decltype(slot_t)::value;
-    ra[SLOT][c] = buffer_load16(r_x, lane_off, (step * 64 + c * 32) * row_bytes);
+    // streaming load: x is read once (k_state_stream 802 -> 784 us)
+    ra[SLOT][c] = buffer_load16<2>(r_x, lane_off, (step * 64 + c * 32) * row_bytes);
   };
   // B fragments of a step: fb[kk][j] = V[tokens 16 kk + 8 (lane >> 5) .. + 8)[value 64 wave + 32 j + (lane & 31)],
   // 1 KiB of consecutive bytes per wavefront and fragment in the fragment-order copy of V
