@@ -628,7 +628,7 @@ __global__ __launch_bounds__(512) void k_chunk_out(ChunkOutArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int row = wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        o[(long)row * 256 + col] = acc[i][j][e];
+        __builtin_nontemporal_store(acc[i][j][e], o + (long)row * 256 + col);  // streaming: 542 -> 528 us for the kernel
       }
     }
 }
