@@ -189,7 +189,7 @@ def bench_prefill(args):
                      "traffic": prefill_traffic_bytes(B, h, N, d, T) if chunked else None,
                      "traffic_source": "buffer sizes of the chunk-recurrent form (x, Q written once and read twice, one "
                                        "bf16 state copy per 256 tokens written and read, rho, out); counters in "
-                                       "profiles/prefill_config3_bf16_kernel_trace.md read 2 % more",
+                                       "profiles/prefill_config3_bf16_kernel_trace.md read the same within 1 %",
                      "hbm_gbs": (prefill_traffic_bytes(B, h, N, d, T) / (ms * 1e-3) / 1e9) if chunked else None,
                      "kernel": "whole bdh_prefill_chunked call (k_state_stream + k_chunk_out); algorithmic FLOP "
                                "= B*h*[T(T-1)N + T(T-1)d + 2TNd], the all-scores count of the workload; the "
@@ -729,7 +729,7 @@ def main():
             "algorithmic_flop": p_flop, "tflops": p_flop / (p_ms * 1e-3) / 1e12,
             "frac": p_flop / (p_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
             "executed_flop": p_exec, "executed_tflops": p_exec / (p_ms * 1e-3) / 1e12,
-            # what bounds this form: its HBM traffic (buffer sizes; the counters of the profile read 2 % more)
+            # what bounds this form: its HBM traffic (buffer sizes; the counters of the profile read the same within 1 %)
             "hbm_traffic_bytes": prefill_traffic_bytes(8, 4, 8192, 256, 2048),
             "hbm_gbs": prefill_traffic_bytes(8, 4, 8192, 256, 2048) / (p_ms * 1e-3) / 1e9,
             "kernel_us_source": "profiles/prefill_config3_bf16_kernel_trace.md",
