@@ -245,6 +245,33 @@ def test_prefill_chunk_recurrent_form_with_unequal_pair_frequencies(bda, corc, T
     assert d_out < 2e-2 and d_rho < 5e-3, (d_out, d_rho)
 
 
+@pytest.mark.parametrize("B,h,T,N,chunk,rho0_scale,hilo", [
+    (3, 3, 512, 768, 0, 0.0, False),      # 9 slices: a second, partly filled group of eight
+    (1, 1, 1280, 2048, 512, 0.05, True),  # one slice, 32 neuron tiles, passes of 512 + 256 tokens
+    (2, 5, 256, 256, 0, 0.05, False),     # 10 slices, a single chunk with a carried state
+    (9, 1, 768, 512, 256, 0.0, False),    # three one-chunk passes, fresh state
+    (1, 2, 2304, 1024, 0, 0.05, False)])  # a pass of 2 048 tokens and one of 256
+def test_prefill_chunk_recurrent_form_equals_all_scores_form(bda, B, h, T, N, chunk, rho0_scale, hilo):
+    """More slice counts, tile counts and pass structures of the chunk-recurrent kernels, against the all-scores form
+    of the same call (itself checked against the sequential oracle above): slices that do not fill the groups of
+    eight the grids are laid out in, one to 32 neuron tiles per slice, one to eight chunks per pass."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    d = 256
+    x, v, rho0 = _prefill_case(B * 1000 + T + N, B, h, T, N, d, 0.1, rho0_scale)
+    sys_freqs = orc.build_freqs(N)
+    ft = torch.from_numpy(np.asarray(sys_freqs, dtype=np.float32)).to(DEV)
+    zero = rho0_scale == 0.0
+    print(f"chunk-recurrent against all-scores: B={B} h={h} T={T} N={N} chunk={chunk} hilo={hilo}", flush=True)
+    rho_c, rho_s = rho0.clone().to(DEV), rho0.clone().to(DEV)
+    out_c = prefill_chunked(x.to(DEV), v.to(DEV), rho_c, ft, 17, state_is_zero=zero, chunk=chunk, hilo=hilo)
+    out_s = prefill_chunked(x.to(DEV), v.to(DEV), rho_s, ft, 17, state_is_zero=zero, chunk=chunk, all_scores=True)
+    torch.cuda.synchronize()
+    d_out, d_rho = rel_err(out_c.cpu().numpy(), out_s.cpu().numpy()), rel_err(rho_c.cpu().numpy(), rho_s.cpu().numpy())
+    print(f"   out {d_out:.2e} state {d_rho:.2e}")
+    assert d_out < 2e-2 and d_rho < 5e-3, (d_out, d_rho)
+
+
 def test_prefill_in_four_calls_equals_one_call(bda, corc):
     """One prompt fed as four successive calls (the state carried in the caller's f32 rho, entering each call's
     product as a bf16 pair) against the sequential oracle and against the single call: T = 4096 in chunks of 512."""
