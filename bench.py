@@ -146,6 +146,52 @@ def measure_prefill(B=8, h=4, N=8192, d=256, T=2048, density=0.05, steps=10, war
     return ms, flop
 
 
+def measure_prefill_queued(B=8, h=4, N=8192, d=256, T=2048, density=0.05, rounds=12, warmup=12):
+    """The same work as measure_prefill fed as a queue: two contexts on two streams, each given half-batch calls back
+    to back, so the write-bound first kernel of one call runs beside the read-bound second kernel of the other.  A
+    throughput figure for servers with independent prompts, not the latency of one call.  Returns ms per B sequences."""
+    import torch
+    from scipy.stats import norm
+
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.kernel.linear_attention import build_freqs
+    from burn_dragon_amd.positional import RotaryEmbedding
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(5)
+    mu = float(norm.ppf(density))
+    freqs = build_freqs(N, 65536.0, RotaryEmbedding.ROPE).reshape(-1).to(dev)
+    half = B // 2
+    sets = []
+    for _ in range(2):
+        x = torch.empty((half, h, T, N), device=dev, dtype=torch.bfloat16)
+        for b in range(half):
+            x[b] = torch.relu(torch.randn((h, T, N), device=dev, generator=g) + mu).to(torch.bfloat16)
+        sets.append((x, torch.randn((half, T, d), device=dev, generator=g).to(torch.bfloat16),
+                     torch.zeros((half, h, N, d), device=dev)))
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    ctxs = [ffi.Context(0, st.cuda_stream) for st in streams]
+    torch.cuda.synchronize()
+
+    def one_round():
+        for (x, v, rho), st, ctx in zip(sets, streams, ctxs):
+            with torch.cuda.stream(st):
+                prefill_chunked(x, v, rho, freqs, 0, state_is_zero=True, ctx=ctx)
+
+    for _ in range(warmup):
+        one_round()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(rounds):
+        one_round()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / rounds
+    for ctx in ctxs:
+        ctx.close()
+    return ms
+
+
 def prefill_executed_flop(B, h, N, d, T):
     """Matrix-core FLOP the chunk-recurrent form executes (d = 256, N % 256 == 0, T % 256 == 0): per 256-token chunk a
     full 256x256 score tile (K = N), scores x V (K = 256, half of it for the upper row block), the state term
@@ -721,6 +767,8 @@ def main():
         del rho, xs, vs
         torch.cuda.empty_cache()
         p_ms, p_flop = measure_prefill(steps=5, warmup=2)
+        torch.cuda.empty_cache()
+        q_ms = measure_prefill_queued()
         p_exec = prefill_executed_flop(8, 4, 8192, 256, 2048)
         result["prefill_config3"] = {
             "workload": "BASELINE config 3: bdh_prefill_chunked B=8 T=2048 h=4 N=8192 d=256, bf16 in / f32 accumulate, "
@@ -733,6 +781,9 @@ def main():
             "hbm_traffic_bytes": prefill_traffic_bytes(8, 4, 8192, 256, 2048),
             "hbm_gbs": prefill_traffic_bytes(8, 4, 8192, 256, 2048) / (p_ms * 1e-3) / 1e9,
             "kernel_us_source": "profiles/prefill_config3_bf16_kernel_trace.md",
+            # not the latency of a call: the same 8 sequences as two queues of half-batch calls on two streams
+            "queued_two_streams_ms_per_8_sequences": q_ms,
+            "queued_two_streams_frac": p_flop / (q_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(B, h, N, d, freqs_host.numpy())
