@@ -498,8 +498,10 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
             y = y * ((blk < g.rl_nblocks && g.rl_mask[blk]) ? 1.0f : 0.0f);
           }
           const long o = (long)row * g.ldc + col;
-          if (g.rl_gate) y = g.rl_gate[(C - g.C) + o] * y;
-          C[o] = y;
+          // the gate and the output are touched once per call: streaming accesses leave the L2 to the operand tiles
+          // ([8192 x 512] x [512 x 131072]: 9.98 -> 9.69 ms)
+          if (g.rl_gate) y = __builtin_nontemporal_load(g.rl_gate + (C - g.C) + o) * y;
+          __builtin_nontemporal_store(y, C + o);
         } else {
           if (col >= g.N) continue;
           float *p = C + (long)row * g.ldc + col;
