@@ -190,6 +190,33 @@ __global__ __launch_bounds__(256) void k_fsa_row(const float *__restrict__ q, co
 // f32 matrix-core path
 // ------------------------------------------------------------------------------------
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Eight floats as three bf16x8 operands h + m + l that add up to the floats exactly: each term holds the next eight
+// significant bits, cut off rather than rounded, so both remainders are exact.  A product of two such sums is taken
+// as the six matrix instructions l h, h l, m m, m h, h m, h h (smallest terms first); what is left out (m l, l m, l l)
+// is below 2^-23 of |a b|, the size of one f32 rounding.  An infinite input gives NaN (inf - inf in the remainder).
+__device__ __forceinline__ void fsa_split3(const float (&a)[8], bf16x8 &h, bf16x8 &m, bf16x8 &l) {
+  unsigned int uh[8], um[8], ul[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    uh[q] = __float_as_uint(a[q]) & 0xffff0000u;
+    const float r1 = a[q] - __uint_as_float(uh[q]);
+    um[q] = __float_as_uint(r1) & 0xffff0000u;
+    ul[q] = __float_as_uint(r1 - __uint_as_float(um[q]));
+  }
+  u32x4 ph, pm, pl;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {  // element 2q in the low half of a dword, 2q + 1 in the high half
+    ph[q] = __builtin_amdgcn_perm(uh[2 * q + 1], uh[2 * q], 0x07060302u);
+    pm[q] = __builtin_amdgcn_perm(um[2 * q + 1], um[2 * q], 0x07060302u);
+    pl[q] = __builtin_amdgcn_perm(ul[2 * q + 1], ul[2 * q], 0x07060302u);
+  }
+  h = __builtin_bit_cast(bf16x8, ph);
+  m = __builtin_bit_cast(bf16x8, pm);
+  l = __builtin_bit_cast(bf16x8, pl);
+}
 constexpr int FK = 16;    // k per LDS stage
 constexpr int FLD = 20;   // LDS row stride in floats (80 bytes: 16-byte aligned, spreads the banks)
 
@@ -246,11 +273,16 @@ __device__ __forceinline__ float4 fsa_ld4(const float *p, int n_valid, bool vec_
 // row stride of tile + 4 floats: float4 stores, and fragment reads of one float per lane in which the
 // 32 lanes of a half-wave take consecutive addresses and the two halves (k and k + 8) fall on the two
 // halves of the 64 banks.
+// SPLIT3: the products run on the bf16 matrix instructions (16 times the f32 rate) with every f32 operand split into
+// three bf16 terms in registers, six instructions per f32 one: f32-level accuracy (the result differs from the f32
+// instruction's by about one rounding of a product), not the bits of any particular summation order.  The fragment a
+// lane holds for eight f32 steps (k = half*8 .. +7 of its row) is the fragment of one 32 x 32 x 16 instruction.
 // Tile BM x BN, NWM x NWN waves, each wave (BM/NWM) x (BN/NWN).  The 128 x 128 tile needs 8 bytes per
 // clock and workgroup from the L2, which three resident workgroups per CU do not get; the
 // 256 x 256 tile halves that per FLOP and is the one that keeps the matrix cores busy.
-template <int EPI, bool A_KMAJOR, bool B_KMAJOR, int BM, int BN, int NWM, int NWN, bool SEQK = false>
+template <int EPI, bool A_KMAJOR, bool B_KMAJOR, int BM, int BN, int NWM, int NWN, bool SEQK = false, bool SPLIT3 = false>
 __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
+  static_assert(!(SEQK && SPLIT3), "the split product does not keep the bits of a scalar loop");
   static_assert(!SEQK || (!A_KMAJOR && B_KMAJOR), "sequential k order is built for row-major A and k-major B");
   constexpr int NT = NWM * NWN * 64;
   constexpr int KLA = BM + 4, KLB = BN + 4;  // row strides of the k-major LDS layouts
@@ -434,6 +466,26 @@ __global__ __launch_bounds__(NWM * NWN * 64) void k_fsa_gemm_f32(FsaArgs g) {
         const float4 lo = *reinterpret_cast<const float4 *>(p), hi = *reinterpret_cast<const float4 *>(p + 4);
         fb[j][0] = lo.x; fb[j][1] = lo.y; fb[j][2] = lo.z; fb[j][3] = lo.w;
         fb[j][4] = hi.x; fb[j][5] = hi.y; fb[j][6] = hi.z; fb[j][7] = hi.w;
+      }
+      if (SPLIT3) {
+        bf16x8 ah[MI], am[MI], al[MI], bh[NJ], bm[NJ], bl[NJ];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fsa_split3(fa[i], ah[i], am[i], al[i]);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) fsa_split3(fb[j], bh[j], bm[j], bl[j]);
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) {
+            f32x16 c = acc[i][j];
+            c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[i], bh[j], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[i], bl[j], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am[i], bm[j], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(am[i], bh[j], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[i], bm[j], c, 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[i], bh[j], c, 0, 0, 0);
+          }
+        return;
       }
 #pragma unroll
       for (int q = 0; q < 8; ++q)
@@ -622,11 +674,11 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     const unsigned groups = (unsigned)((S + 7) / 8);
     if (big) {
       g.mt = g.nt = (T + 255) / 256;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 256, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512), 0,
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 256, 256, 2, 4, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(512), 0,
                          ctx->stream, g);
     } else {
       g.mt = g.nt = (T + 127) / 128;
-      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+      hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 128, 128, 2, 2, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
                          ctx->stream, g);
     }
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<scores>");
@@ -643,7 +695,7 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
     o.norm = row_normalize ? norm : nullptr;
     o.mt = (T + 127) / 128;
     o.nt = (dv + 127) / 128;
-    hipLaunchKernelGGL((k_fsa_gemm_f32<1, false, true, 128, 128, 2, 2>), dim3(8 * groups * o.mt * o.nt), dim3(256), 0,
+    hipLaunchKernelGGL((k_fsa_gemm_f32<1, false, true, 128, 128, 2, 2, false, true>), dim3(8 * groups * o.mt * o.nt), dim3(256), 0,
                        ctx->stream, o);
     BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<out>");
     return BDH_OK;
@@ -745,11 +797,11 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
                            0, ctx->stream, g);
       } else if (big) {
         g.mt = g.nt = (tc + 255) / 256;
-        hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 256, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512),
+        hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 256, 256, 2, 4, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(512),
                            0, ctx->stream, g);
       } else {
         g.mt = g.nt = (tc + 127) / 128;
-        hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256),
+        hipLaunchKernelGGL((k_fsa_gemm_f32<0, false, false, 128, 128, 2, 2, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(256),
                            0, ctx->stream, g);
       }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<chunk scores>");
@@ -766,17 +818,9 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
         hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128), 0,
                            ctx->stream, g);
       } else {
-        // all 256 tokens of a call in one row tile where there are that many: the state (B operand) streams through
-        // once instead of twice (config-4 prompt shapes: 9.1 -> 7.9 ms per layer and 256-token call)
-        if (tc > 128) {
-          g.mt = (tc + 255) / 256; g.nt = nt_d;
-          hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 256, 128, 4, 2>), dim3(8 * groups * g.mt * g.nt), dim3(512), 0,
-                             ctx->stream, g);
-        } else {
-          g.mt = (tc + 127) / 128; g.nt = nt_d;
-          hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
-                             ctx->stream, g);
-        }
+        g.mt = (tc + 127) / 128; g.nt = nt_d;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                           ctx->stream, g);
       }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q rho>");
     }
@@ -792,7 +836,7 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
                            ctx->stream, g);
       } else {
         g.mt = (tc + 127) / 128; g.nt = nt_d;
-        hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
                            ctx->stream, g);
       }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<S V>");
@@ -810,17 +854,9 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
         hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 32, 64, 1, 2>), dim3(8 * groups * g.mt * g.nt), dim3(128), 0,
                            ctx->stream, g);
       } else {
-        // 128 x 256 tiles where the value dimension allows: A (the tokens' activations) is read half as often (config-4
-        // prompt shapes: 13.2 -> 12.1 ms per layer and 256-token call; 256 x 256 tiles 17.8 ms)
-        if (d % 256 == 0) {
-          g.mt = (Nq + 127) / 128; g.nt = d / 256;
-          hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 128, 256, 2, 4>), dim3(8 * groups * g.mt * g.nt), dim3(512), 0,
-                             ctx->stream, g);
-        } else {
-          g.mt = (Nq + 127) / 128; g.nt = nt_d;
-          hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
-                             ctx->stream, g);
-        }
+        g.mt = (Nq + 127) / 128; g.nt = nt_d;
+        hipLaunchKernelGGL((k_fsa_gemm_f32<2, true, true, 128, 128, 2, 2, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+                           ctx->stream, g);
       }
       BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<Q^T V>");
     }
@@ -857,7 +893,7 @@ int bdh_launch_decoder_partials_f32(bdh_ctx *ctx, int B, int T, int h, int N, in
   g.block_size = 1; g.h = h; g.dense = 0; g.beta = 0;
   g.mt = (T + 127) / 128; g.nt = (d + 127) / 128;
   if ((long)groups * 8 * g.mt * g.nt > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles");
-  hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
+  hipLaunchKernelGGL((k_fsa_gemm_f32<2, false, true, 128, 128, 2, 2, false, true>), dim3(8 * groups * g.mt * g.nt), dim3(256), 0,
                      ctx->stream, g);
   BDH_LAUNCH_CHECK(ctx, "k_fsa_gemm_f32<decoder>");
   return BDH_OK;

@@ -385,6 +385,36 @@ def test_dense_chunk_form_matches_sequential_oracle(gpu, corc, dense_chunks, rot
     assert rel_err(rho_new, rho_ref) < 2e-5, rel_err(rho_new, rho_ref)
 
 
+def test_dense_chunk_form_split_products_keep_f32_accuracy(gpu, corc, dense_chunks):
+    """The big-tile products of the dense form run on the bf16 matrix instructions with every f32 operand
+    split into three bf16 terms (six instructions per f32 one).  Against a float64 evaluation of the same
+    sums from the same rotated activations, the error must stay at the level of f32 rounding: a dropped
+    cross term (2^-16 of a product) would show up as several 1e-6 here.
+    64 slices of 256 tokens: every product takes the 128 x 128 / 256 x 256 tiles."""
+    _, recurrent_attention = gpu
+    B, h, T, N, d = 8, 8, 256, 256, 256
+    x, v, rho0 = make_inputs(4242, B, h, T, N, d, 0.5, rho_scale=0.05)
+    rng = np.random.default_rng(17)
+    x *= np.exp2(rng.integers(-6, 7, (1, h, 1, N))).astype(np.float32)   # operands of mixed magnitude
+    v *= np.exp2(rng.integers(-6, 7, (1, 1, d))).astype(np.float32)
+    freqs = corc.build_freqs(N)
+    position = 11
+    out, rho_new = _run_plain(recurrent_attention, x, v, rho0, freqs, position, orc.ROPE)
+    q = corc.rotate(x, freqs, orc.ROPE, position).astype(np.float64)
+    v64, r64 = v.astype(np.float64), rho0.astype(np.float64)
+    scores = np.tril(np.einsum("bhtn,bhsn->bhts", q, q), -1)
+    out_ref = np.einsum("bhts,bsd->bhtd", scores, v64) + np.einsum("bhtn,bhnd->bhtd", q, r64)
+    rho_ref = r64 + np.einsum("bhtn,btd->bhnd", q, v64)
+
+    def rms_err(a, b):
+        return float(np.sqrt(np.mean((a.astype(np.float64) - b) ** 2)) / np.sqrt(np.mean(b ** 2)))
+
+    # measured: 3.1e-7 and 2.5e-7 (the f32 matrix instructions: 2.7e-7 and 2.5e-7)
+    assert rms_err(out, out_ref) < 6e-7, rms_err(out, out_ref)
+    assert rms_err(rho_new, rho_ref) < 6e-7, rms_err(rho_new, rho_ref)
+    assert rel_err(out, out_ref) < 2e-6 and rel_err(rho_new, rho_ref) < 2e-6
+
+
 def test_dense_chunk_form_equals_step_kernels_and_handles_device_positions(gpu, corc):
     """The same call through the sparse step kernels and through the dense form; per-sequence device
     positions; T = 128 takes the dense form by default once the products have enough tiles to cover the
