@@ -193,25 +193,24 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// Eight floats as three bf16x8 operands h + m + l that add up to the floats exactly: each term holds the next eight
-// significant bits, cut off rather than rounded, so both remainders are exact.  A product of two such sums is taken
-// as the six matrix instructions l h, h l, m m, m h, h m, h h (smallest terms first); what is left out (m l, l m, l l)
-// is below 2^-23 of |a b|, the size of one f32 rounding.  An infinite input gives NaN (inf - inf in the remainder).
+// Eight floats as three bf16x8 operands h + m + l that add up to the floats exactly: each term is the remainder so far
+// rounded to bf16 (v_cvt_pk_bf16_f32, round to nearest even); a remainder is a difference of neighbours and therefore
+// exact, and the third one has at most eight significant bits.  A product of two such sums is taken as the six matrix
+// instructions l h, h l, m m, m h, h m, h h (smallest terms first); what is left out (m l, l m, l l) is below 2^-23 of
+// |a b|, the size of one f32 rounding.  An infinite input, or a finite one that rounds to an infinite bf16 (above
+// 3.389e38), gives NaN (inf - inf in the remainder).
 __device__ __forceinline__ void fsa_split3(const float (&a)[8], bf16x8 &h, bf16x8 &m, bf16x8 &l) {
-  unsigned int uh[8], um[8], ul[8];
-#pragma unroll
-  for (int q = 0; q < 8; ++q) {
-    uh[q] = __float_as_uint(a[q]) & 0xffff0000u;
-    const float r1 = a[q] - __uint_as_float(uh[q]);
-    um[q] = __float_as_uint(r1) & 0xffff0000u;
-    ul[q] = __float_as_uint(r1 - __uint_as_float(um[q]));
-  }
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
   u32x4 ph, pm, pl;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {  // element 2q in the low half of a dword, 2q + 1 in the high half
-    ph[q] = __builtin_amdgcn_perm(uh[2 * q + 1], uh[2 * q], 0x07060302u);
-    pm[q] = __builtin_amdgcn_perm(um[2 * q + 1], um[2 * q], 0x07060302u);
-    pl[q] = __builtin_amdgcn_perm(ul[2 * q + 1], ul[2 * q], 0x07060302u);
+    const f32x2 a2 = {a[2 * q], a[2 * q + 1]};
+    ph[q] = __builtin_bit_cast(unsigned int, __builtin_convertvector(a2, bf16x2));
+    const f32x2 r1 = {a2[0] - __uint_as_float(ph[q] << 16), a2[1] - __uint_as_float(ph[q] & 0xffff0000u)};
+    pm[q] = __builtin_bit_cast(unsigned int, __builtin_convertvector(r1, bf16x2));
+    const f32x2 r2 = {r1[0] - __uint_as_float(pm[q] << 16), r1[1] - __uint_as_float(pm[q] & 0xffff0000u)};
+    pl[q] = __builtin_bit_cast(unsigned int, __builtin_convertvector(r2, bf16x2));
   }
   h = __builtin_bit_cast(bf16x8, ph);
   m = __builtin_bit_cast(bf16x8, pm);

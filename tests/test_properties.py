@@ -116,3 +116,39 @@ def test_damaged_record_framing_fails_cleanly(data):
         record.weights_from_params(params)
     except record.RecordError:
         pass
+
+
+def _bf16_rne(a):
+    u = np.asarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def _split3_bf16(a):
+    """The three-term split the dense f32 products use on the GPU (csrc/attention_parallel.hip, fsa_split3):
+    each term is the remainder so far rounded to bf16 (= an f32 with a zero lower half), nearest even."""
+    a = np.asarray(a, np.float32)
+    h = _bf16_rne(a)
+    r1 = a - h
+    m = _bf16_rne(r1)
+    r2 = r1 - m
+    return h, m, _bf16_rne(r2), r1, r2
+
+
+@FAST
+@given(seed=st.integers(0, 2**31 - 1), spread=st.integers(0, 60))
+def test_three_bf16_terms_add_up_to_the_float_and_six_products_keep_f32_accuracy(seed, spread):
+    """h + m + l == a exactly (both remainders are exact in f32, the third term holds what is left), and
+    |a b - (hh + hm + mh + hl + lh + mm)| <= 2^-22 |a b|: the three dropped products."""
+    rng = np.random.default_rng(seed)
+    n = 4096
+    a = (rng.standard_normal(n) * np.exp2(rng.integers(-spread, spread + 1, n))).astype(np.float32)
+    b = (rng.standard_normal(n) * np.exp2(rng.integers(-spread, spread + 1, n))).astype(np.float32)
+    f = lambda t: t.astype(np.float64)
+    ha, ma, la, r1, r2 = _split3_bf16(a)
+    assert np.array_equal(f(r1), f(a) - f(ha)) and np.array_equal(f(r2), f(r1) - f(ma))  # exact remainders
+    assert np.array_equal(f(ha) + f(ma) + f(la), f(a))
+    hb, mb, lb, _, _ = _split3_bf16(b)
+    six = f(la) * f(hb) + f(ha) * f(lb) + f(ma) * f(mb) + f(ma) * f(hb) + f(ha) * f(mb) + f(ha) * f(hb)
+    exact = f(a) * f(b)
+    assert np.all(np.abs(exact - six) <= np.abs(exact) * 2.0**-22)
