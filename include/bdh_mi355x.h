@@ -69,7 +69,7 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *   "state_step.split": -1 (default) pick by grid size, 0 = 256 lane pairs per workgroup,
  *                       1 = 64 lane pairs per workgroup of 8 waves (small batches).
  *   "state_step.dense_chunks": -1 (default) a call of 128+ tokens without
- *                       bitmask / row-count outputs runs as dense products on the f32 matrix cores
+ *                       bitmask / row-count outputs runs as dense products on the matrix cores
  *                       (with only a few (sequence, head) slices an f32 RoPE state keeps the token loop;
  *                       from 8 tokens on for an f32 state that every token streams in full -- PoPE,
  *                       eager ALiBi -- or that is at most 64 MiB),
@@ -111,7 +111,8 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *   "model.phase_batch": the two-launch layer only for at most this many sequences (default: no limit
  *                       beyond the one above; 0 = never).
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
- *                       1 = the two products on the f32 matrix cores (T >= 128 by default). */
+ *                       1 = the two products on the matrix cores (T >= 128 by default; operands as three
+ *                       bf16 terms each, f32-level accuracy). */
 int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);
 
 /* ---- host-side tables (computed on the host in the reference as well) --------------- */
@@ -157,9 +158,11 @@ int bdh_rotate(bdh_ctx *ctx, int B, int h, int T, int N, int rotary, const float
  * RoPE requires even N (src/model/attention.rs:310).  T = 1 is the decode step.  A call of 128 or more
  * tokens that asks for neither bitmask nor row counts computes the same sums as dense
  * products (out = tril(-1)(Q Q^T) V + Q rho, rho += Q^T V, chunks of up to 512 tokens; for ALiBi with
- * the decay powers decay^(t-s), decay^t and decay^(T-s) applied to the three terms) on the f32 matrix
- * cores (a bf16 state is widened to f32 for the call and rounded once at its end); results agree with
- * the token loop to f32 reassociation (option "state_step.dense_chunks").
+ * the decay powers decay^(t-s), decay^t and decay^(T-s) applied to the three terms) on the matrix
+ * cores (a bf16 state is widened to f32 for the call and rounded once at its end).  Large products
+ * take every f32 operand as a sum of three bf16 terms, six bf16 matrix instructions per f32 one: what
+ * is left out is below 2^-23 of a product, so results agree with the token loop to f32 reassociation
+ * (option "state_step.dense_chunks").  Inputs are assumed finite.
  */
 int bdh_recurrent_attention(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary,
                             const float *x, const float *v, const float *freqs,
