@@ -467,6 +467,39 @@ def test_dense_chunk_form_alibi_matches_sequential_oracle(gpu, corc, dense_chunk
     assert rel_err(rt.cpu().numpy(), rho_ref) < 1e-4, rel_err(rt.cpu().numpy(), rho_ref)
 
 
+@pytest.mark.parametrize("rotary", [orc.ROPE, orc.POPE, orc.ALIBI])
+def test_dense_chunk_form_big_tiles_on_ragged_shapes(gpu, corc, dense_chunks, rotary):
+    """64 slices put every product on the 128 x 128 / 256 x 256 tiles (split-bf16 products); T, N and d are
+    no multiples of a tile, of the 16-wide k stage or of 8, so every edge tile takes the checked loads, and a
+    600-token call adds a second chunk with a carried state.  Against the oracle's token loop
+    (src/model/bdh.rs:286-303)."""
+    _, recurrent_attention = gpu
+    from burn_dragon_amd.positional import RotaryEmbedding
+
+    B, h, N, d = 8, 8, 138, 202
+    for T in (200, 600):
+        x, v, rho0 = make_inputs(77 + T, B, h, T, N, d, 0.3, rho_scale=0.05)
+        Nq = 2 * N if rotary == orc.POPE else N
+        rho0 = (0.05 * np.random.default_rng(9).standard_normal((B, h, Nq, d))).astype(np.float32)
+        if rotary == orc.ALIBI:
+            slopes = np.array([0.02 * (i + 1) for i in range(h)], np.float32)
+            dev = "cuda:0"
+            rt = torch.from_numpy(rho0).to(dev).contiguous()
+            out = recurrent_attention(torch.from_numpy(x).to(dev), torch.from_numpy(v).to(dev), rt,
+                                      torch.zeros(N, device=dev), 5, RotaryEmbedding.ALIBI, slopes)
+            torch.cuda.synchronize()
+            out, rho_new = out.cpu().numpy(), rt.cpu().numpy()
+            out_ref, rho_ref = corc.recurrent_attention(x, v, rho0.copy(), corc.alibi_decay(slopes))
+            tol = 1e-4
+        else:
+            freqs = corc.build_freqs(N, rotary=rotary)
+            out, rho_new = _run_plain(recurrent_attention, x, v, rho0, freqs, 5, rotary)
+            out_ref, rho_ref = corc.recurrent_attention(corc.rotate(x, freqs, rotary, 5), v, rho0.copy())
+            tol = 2e-5
+        assert rel_err(out, out_ref) < tol, (T, rel_err(out, out_ref))
+        assert rel_err(rho_new, rho_ref) < tol, (T, rel_err(rho_new, rho_ref))
+
+
 def test_dense_chunk_form_on_a_lazily_decayed_alibi_state(gpu, corc):
     """T = 150 on a state with pending decay: the call applies it, runs the dense form (default from T = 128)
     and leaves every stamp at clock + T; a following single-token lazy step continues correctly."""
