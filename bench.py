@@ -309,6 +309,97 @@ def measure_rmw_ceiling(region_bytes=1 << 30, chunk_kib=2, density=0.0975, lists
     return out, moved
 
 
+def measure_deferred(B=32, h=4, N=8192, d=256, density=0.05, rho_dtype="f32", capacity=128, steps=1000, warmup=128,
+                     ring=None, seed=2):
+    """The decode step with deferred updates (bdh_state_step_deferred) on the config-2 workload: every step reads its
+    active rows and logs its update; every `capacity` steps the step itself flushes the log into the state, and a
+    final bdh_state_flush ends the run -- ALL flushes are inside the timed region.  The ring holds at least
+    `capacity` distinct x sets, so the rows a flush rewrites are the union of that many independent steps.
+    Algorithmic bytes are those of the eager step (every touched row read once and written once per step)."""
+    import torch
+    from scipy.stats import norm
+
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.kernel.linear_attention import build_freqs
+    from burn_dragon_amd.positional import RotaryEmbedding
+    from burn_dragon_amd.recurrent import StateLog
+
+    dev = torch.device("cuda:0")
+    ctx = ffi.default_context(0)
+    lib = ctx.lib
+    ring = max(ring or 16, capacity)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    tdt = torch.float32 if rho_dtype == "f32" else torch.bfloat16
+    esz = 4 if rho_dtype == "f32" else 2
+    rho = (0.01 * torch.randn((B, h, N, d), device=dev, generator=g)).to(tdt).contiguous()
+    mu = float(norm.ppf(density))
+    xs = [torch.relu(torch.randn((B, h, N), device=dev, generator=g) + mu).contiguous() for _ in range(ring)]
+    vs = [torch.randn((B, d), device=dev, generator=g).contiguous() for _ in range(ring)]
+    freqs = build_freqs(N, 65536.0, RotaryEmbedding.ROPE).reshape(-1).to(dev)
+    out = torch.empty((B, h, d), device=dev)
+    rows = torch.zeros((B, h), device=dev, dtype=torch.int32)
+    positions = np.random.default_rng(3).integers(0, 4096, size=steps + warmup)
+    log = StateLog(B, h, N, d, tdt, capacity)
+    R = []
+    for i in range(ring):
+        ctx.check(lib.bdh_state_step_deferred(ctx.handle, log.handle, xs[i].data_ptr(), vs[i].data_ptr(), freqs.data_ptr(),
+                                              0, None, rho.data_ptr(), out.data_ptr(), None, rows.data_ptr()))
+        R.append(int(rows.sum().item()))
+    R_mean = float(np.mean(R))
+    bytes_per_step = 2.0 * R_mean * d * esz + 4.0 * B * h * N + 4.0 * B * d + 4.0 * B * h * d + 4.0 * N
+    fn, hnd, lh = lib.bdh_state_step_deferred, ctx.handle, log.handle
+    call_args = [(hnd, lh, xs[i % ring].data_ptr(), vs[i % ring].data_ptr(), freqs.data_ptr(), int(positions[i]), None,
+                  rho.data_ptr(), out.data_ptr(), None, None) for i in range(steps + warmup)]
+    for i in range(warmup):
+        ctx.check(fn(*call_args[i]))
+    log.flush(rho)  # the timed region starts on an empty log
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    rc_bad = 0
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(warmup, warmup + steps):
+        rc_bad |= fn(*call_args[i])
+    rc_bad |= lib.bdh_state_flush(hnd, lh, rho.data_ptr())
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ctx.check(rc_bad)
+    gpu_ms = start.elapsed_time(stop)
+    ms_per_step = max(gpu_ms, wall * 1e3) / steps
+    achieved = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+    flushes = (steps + capacity - 1) // capacity
+    res = {
+        "workload": f"bdh_state_step_deferred on config 2 (rho {rho_dtype} [{B},{h},{N},{d}], {density:.0%} active, {ring} input sets): "
+                    f"log capacity {capacity}, {steps} timed steps with all {flushes} flushes inside the timed region",
+        "log_capacity": capacity, "log_bytes": log.nbytes, "steps": steps, "flushes_timed": flushes,
+        "ms_per_step": ms_per_step, "tokens_per_s": B / (ms_per_step * 1e-3),
+        "gpu_event_ms_total": gpu_ms, "wall_ms_total": wall * 1e3,
+        "touched_rows_per_step": R_mean, "algorithmic_bytes_per_step": bytes_per_step,
+        "achieved_gbs": achieved, "frac": achieved / HBM_PEAK_GBS,
+        "kernels": "k_step_deferred + k_deferred_finalize per step, k_state_flush per flush; achieved = the eager step's "
+                   "algorithmic bytes / ms_per_step (the slower of the HIP-event and the host clock)",
+    }
+    log.close()
+    del rho, xs, vs
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_deferred(args):
+    """The deferred-update decode step alone (the default line carries the same figures as its `deferred` record)."""
+    r = measure_deferred(args.batch, args.heads, args.latent, args.embd, args.density, args.rho_dtype, args.log_capacity,
+                         args.steps, max(args.warmup, args.log_capacity), args.ring)
+    print(json.dumps({
+        "metric": "decode tokens/sec at batch B (single-layer state step, deferred updates) + achieved HBM GB/s",
+        "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.rho_dtype, "data": "synthetic", "config": r,
+        "roofline": {"bound": "hbm", "achieved": r["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": r["frac"], "traffic": None, "kernel": r["kernels"], "launch_us": r["ms_per_step"] * 1e3},
+    }))
+
+
 def bench_rmw_probe(args):
     """The bandwidth ceiling of the decode step's access pattern, measured on this box."""
     res, moved = measure_rmw_ceiling(modes=(0, 1, 2), iters=256 if args.steps == 1000 else args.steps)
@@ -617,9 +708,10 @@ def main():
     ap.add_argument("--rho-dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--ring", type=int, default=16, help="number of distinct (x, v) input sets")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--log-capacity", type=int, default=128, help="deferred: steps the update log holds between flushes")
     ap.add_argument("--prefill-chunk", type=int, default=0,
                     help="model workload: feed the prompt in calls of this many tokens (0 = one call)")
-    ap.add_argument("--workload", choices=["decode", "prefill", "model", "copy", "alibi", "parallel", "chunks", "rmw_probe"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "deferred", "prefill", "model", "copy", "alibi", "parallel", "chunks", "rmw_probe"], default="decode",
                     help="decode = BASELINE config 2 (the headline metric); prefill = config 3 (bf16 MFMA); "
                          "model = full-model greedy decode (config 1 by default, --model-config c4 for config 4); "
                          "alibi = ALiBi state step, lazily decayed state beside the eager dense decay; "
@@ -669,6 +761,8 @@ def main():
         return bench_chunks(args)
     if args.workload == "rmw_probe":
         return bench_rmw_probe(args)
+    if args.workload == "deferred":
+        return bench_deferred(args)
     B, h, N, d = args.batch, args.heads, args.latent, args.embd
     ctx = ffi.default_context(0)
     lib = ctx.lib
@@ -769,9 +863,11 @@ def main():
         },
     }
     if default_workload:
-        # BASELINE config 3 beside the headline: the chunked prefill, bf16 matrix cores (its own roofline)
+        # the same workload through the deferred-update step (flushes inside its timed region)
         del rho, xs, vs
         torch.cuda.empty_cache()
+        result["deferred"] = measure_deferred(steps=args.steps, warmup=max(args.warmup, 128))
+        # BASELINE config 3 beside the headline: the chunked prefill, bf16 matrix cores (its own roofline)
         p_ms, p_flop = measure_prefill(steps=5, warmup=2)
         torch.cuda.empty_cache()
         q_ms = measure_prefill_queued()

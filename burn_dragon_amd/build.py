@@ -13,7 +13,7 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libbdh_mi355x.so")
-SOURCES = ["bdh_api.hip", "state_step.hip", "projections.hip", "model.hip", "attention_parallel.hip", "prefill.hip",
+SOURCES = ["bdh_api.hip", "state_step.hip", "state_deferred.hip", "projections.hip", "model.hip", "attention_parallel.hip", "prefill.hip",
            "sampling.hip", "viz_taps.hip", "model_small.hip", "model_phase.hip", "probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -123,6 +123,13 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
 int bdh_launch_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, const float *slopes_host, int64_t clock,
                                  const int32_t *clocks_dev, void *rho, int rho_dtype, int32_t *stamps);
 
+// state_deferred.hip: the decode step with logged updates (RoPE, T = 1).  out_ln != nullptr: the readout is also
+// written LayerNorm-ed (src/model/bdh.rs:359).  The flush applies the pending steps to rho and empties the log.
+int bdh_launch_state_step_deferred(bdh_ctx *ctx, bdh_state_log *log, const float *x, const float *v, const float *freqs,
+                                   int64_t position, const int32_t *positions_dev, void *rho, float *out, float *out_ln,
+                                   uint64_t *bitmask, int32_t *rows_touched);
+int bdh_launch_state_flush(bdh_ctx *ctx, bdh_state_log *log, void *rho);
+
 struct ReluLowrankParams {
   int B, h_in, T, d, h, N;
   const float *in, *weight, *bias;

@@ -30,6 +30,8 @@ EXPORTS = [
     "bdh_sample_top_k", "bdh_recurrent_attention_lazy_alibi", "bdh_alibi_materialize", "bdh_model_forward_lazy",
     "bdh_rho_energy", "bdh_model_forward_viz", "bdh_rotate",
     "bdh_model_forward_fast", "bdh_model_forward_fast_ex", "bdh_state_step_noalloc", "bdh_probe_chunks",
+    "bdh_state_log_create", "bdh_state_log_destroy", "bdh_state_log_pending", "bdh_state_log_bytes",
+    "bdh_state_step_deferred", "bdh_state_flush",
 ]
 
 
@@ -88,6 +90,13 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_state_step.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, P, P, P, c_int, P, P, P]
     lib.bdh_state_step_noalloc.argtypes = lib.bdh_state_step.argtypes
     lib.bdh_probe_chunks.argtypes = [P, P, c_size_t, P, c_int, c_int, c_int, c_int]
+    lib.bdh_state_log_create.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, POINTER(P)]
+    lib.bdh_state_log_destroy.argtypes = [P, P]
+    lib.bdh_state_log_pending.argtypes = [P]
+    lib.bdh_state_log_bytes.restype = c_size_t
+    lib.bdh_state_log_bytes.argtypes = [P]
+    lib.bdh_state_step_deferred.argtypes = [P, P, P, P, P, c_int64, P, P, P, P, P]
+    lib.bdh_state_flush.argtypes = [P, P, P]
     lib.bdh_relu_lowrank.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_float, c_int, P, c_int,
                                      P, P]
     lib.bdh_layer_norm.argtypes = [P, c_int64, c_int, P, P]

@@ -141,3 +141,76 @@ def prefill_chunked(x_bf16: torch.Tensor, v_bf16: torch.Tensor, rho: torch.Tenso
                                           ffi.ptr(freqs), int(position), int(chunk), flags, ffi.ptr(rho),
                                           ffi.ptr(out)))
     return out
+
+
+class StateLog:
+    """The pending rank-1 updates of ONE state tensor rho [B,h,N,d] (bdh_state_log): the deferred decode step
+    reads its active state rows and logs its update; `flush` (called by the step itself when `capacity` steps are
+    pending) applies the logged updates in step order, after which rho holds the bits the eager step leaves.
+    Flush before anything else reads or writes rho."""
+
+    def __init__(self, B: int, h: int, N: int, d: int, rho_dtype: torch.dtype = torch.float32, capacity: int = 32,
+                 ctx: Optional[ffi.Context] = None, device_id: int = 0):
+        import ctypes
+
+        self.ctx = ctx or ffi.default_context(device_id)
+        self.shape = (B, h, N, d)
+        self.rho_dtype = rho_dtype
+        self.capacity = capacity
+        dt = {torch.float32: ffi.F32, torch.bfloat16: ffi.BF16}[rho_dtype]
+        handle = ctypes.c_void_p()
+        self.ctx.check(self.ctx.lib.bdh_state_log_create(self.ctx.handle, B, h, N, d, dt, capacity, ctypes.byref(handle)))
+        self.handle = handle
+
+    @property
+    def pending(self) -> int:
+        return int(self.ctx.lib.bdh_state_log_pending(self.handle))
+
+    @property
+    def nbytes(self) -> int:
+        return int(self.ctx.lib.bdh_state_log_bytes(self.handle))
+
+    def flush(self, rho: torch.Tensor) -> None:
+        self.ctx.check(self.ctx.lib.bdh_state_flush(self.ctx.handle, self.handle, ffi.ptr(rho)))
+
+    def close(self) -> None:
+        import sys
+
+        if getattr(self, "handle", None) and getattr(self.ctx, "handle", None):
+            if not sys.is_finalizing():
+                self.ctx.lib.bdh_state_log_destroy(self.ctx.handle, self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def state_step_deferred(log: StateLog, query: torch.Tensor, value: torch.Tensor, rho: torch.Tensor,
+                        freqs: torch.Tensor, position: int, positions: Optional[torch.Tensor] = None,
+                        want_bitmask: bool = False, want_rows: bool = False):
+    """BDH::recurrent_attention at T = 1 (src/model/bdh.rs:258-307, RoPE) with the update of :298 logged in `log`
+    instead of written to rho.  query [B,h,N] or [B,h,1,N] un-rotated, value [B,d]; returns out [B,h,d]
+    (+ bitmask [B,h,ceil(N/64)] int64 view, + rows_touched [B,h] int32 when asked)."""
+    ctx = log.ctx
+    B, h, N, d = log.shape
+    query = query.reshape(B, h, N)
+    value = value.reshape(B, d)
+    assert query.dtype == torch.float32 and query.is_contiguous()
+    assert value.dtype == torch.float32 and value.is_contiguous()
+    assert rho.is_contiguous() and tuple(rho.shape) == (B, h, N, d) and rho.dtype == log.rho_dtype
+    freqs = freqs.reshape(-1)
+    out = torch.empty((B, h, d), device=query.device, dtype=torch.float32)
+    bm = torch.zeros((B, h, (N + 63) // 64), device=query.device, dtype=torch.int64) if want_bitmask else None
+    rows = torch.zeros((B, h), device=query.device, dtype=torch.int32) if want_rows else None
+    ctx.check(ctx.lib.bdh_state_step_deferred(ctx.handle, log.handle, ffi.ptr(query), ffi.ptr(value), ffi.ptr(freqs),
+                                              int(position), ffi.ptr(positions), ffi.ptr(rho), ffi.ptr(out), ffi.ptr(bm),
+                                              ffi.ptr(rows)))
+    res = [out]
+    if want_bitmask:
+        res.append(bm)
+    if want_rows:
+        res.append(rows)
+    return res[0] if len(res) == 1 else tuple(res)

@@ -194,6 +194,44 @@ int bdh_state_step_noalloc(bdh_ctx *ctx, int B, int h, int N, int d, int rotary,
                            int rho_dtype, float *out, uint64_t *active_bitmask,
                            int32_t *rows_touched);
 
+/* ---- the decode step with deferred state updates ---------------------------------- */
+/*
+ * BDH::recurrent_attention at T = 1 (src/model/bdh.rs:258-307 with the rotation of :265; RoPE only) like
+ * bdh_state_step, but the rank-1 update of :298 is LOGGED instead of written: a step reads its active state
+ * rows once and writes none of them.  What differs from the reference's step:
+ *   - readout: out_t = sum_n rho_base[n,:] q_t[n] + sum_s (q_t . q_s) v_s over the logged steps s, the sums of
+ *     src/model/bdh.rs:293-295 reassociated (agrees with bdh_state_step to f32 rounding, ~1e-6 relative);
+ *   - state: `rho` lags behind by the logged steps until a flush applies them.  bdh_state_flush (and every
+ *     capacity-th call of bdh_state_step_deferred by itself, before it logs) walks the state rows the logged
+ *     steps touched and applies their updates in step order, row + (q_s[n] * v_s) with the product rounded
+ *     before the add: afterwards rho holds, bit for bit, what the same calls of bdh_state_step would have left
+ *     (a bf16 state is rounded after every logged step, as the eager step stores it).
+ * The caller flushes before anything else reads or writes rho (another entry point, an export, a copy), the way
+ * bdh_alibi_materialize precedes such uses of a lazily decayed state.  A log serves ONE state tensor at a time:
+ * while steps are pending, a call with another rho pointer fails with BDH_E_INVAL.
+ *   bdh_state_log_create  B, h, N, d, rho_dtype as in bdh_state_step (d in {256, 512}, even N); capacity =
+ *                         steps the log holds, 1..128 with capacity * d <= 32768 (the flush keeps the logged
+ *                         value rows in LDS).  Device memory of the log: about B*h*(N/512)*(capacity*2 + 4.5) KiB
+ *                         (config 2 at capacity 128: 521 MiB).  The larger the capacity, the less often the
+ *                         state is rewritten: at config 2 a flush rewrites nearly every row from 32 steps on.
+ *   bdh_state_log_pending steps logged and not yet applied.
+ *   bdh_state_step_deferred  x [B,h,N], v [B,d], freqs [N], position / positions_dev, out [B,h,d],
+ *                         active_bitmask and rows_touched exactly as bdh_state_step (rows_touched counts the
+ *                         rows of the active pairs, which this call only reads).
+ * The number of pending steps is host-side state of the log, so one step is not a fixed launch sequence: a HIP
+ * graph can hold `capacity` steps followed by a flush, not a single step.
+ */
+typedef struct bdh_state_log bdh_state_log; /* opaque: pending rank-1 updates of one state tensor */
+int bdh_state_log_create(bdh_ctx *ctx, int B, int h, int N, int d, int rho_dtype, int capacity,
+                         bdh_state_log **out);
+int bdh_state_log_destroy(bdh_ctx *ctx, bdh_state_log *log);
+int bdh_state_log_pending(const bdh_state_log *log);
+size_t bdh_state_log_bytes(const bdh_state_log *log);
+int bdh_state_step_deferred(bdh_ctx *ctx, bdh_state_log *log, const float *x, const float *v,
+                            const float *freqs, int64_t position, const int32_t *positions_dev, void *rho,
+                            float *out, uint64_t *active_bitmask, int32_t *rows_touched);
+int bdh_state_flush(bdh_ctx *ctx, bdh_state_log *log, void *rho);
+
 /* ---- a3 / a7: ReLU low-rank projection ------------------------------------------- */
 /*
  * Replaces kernel::relu_lowrank::fused_forward (src/kernel/relu_lowrank.rs:7-37) and the

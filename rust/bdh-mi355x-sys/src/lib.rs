@@ -25,6 +25,12 @@ pub struct bdh_model {
     _private: [u8; 0],
 }
 
+/// opaque: pending rank-1 updates of one state tensor (the deferred decode step)
+#[repr(C)]
+pub struct bdh_state_log {
+    _private: [u8; 0],
+}
+
 pub const BDH_OK: c_int = 0;
 pub const BDH_E_INVAL: c_int = -1;
 pub const BDH_E_SHAPE: c_int = -2;
@@ -96,6 +102,15 @@ extern "C" {
         x: *const f32, v: *const f32, freqs: *const f32, position: i64, positions_dev: *const i32,
         alibi_slopes_host: *const f32, rho: *mut c_void, rho_dtype: c_int, out: *mut f32,
         active_bitmask: *mut u64, rows_touched: *mut i32) -> c_int;
+    pub fn bdh_state_log_create(ctx: *mut bdh_ctx, b: c_int, h: c_int, n: c_int, d: c_int, rho_dtype: c_int,
+        capacity: c_int, out: *mut *mut bdh_state_log) -> c_int;
+    pub fn bdh_state_log_destroy(ctx: *mut bdh_ctx, log: *mut bdh_state_log) -> c_int;
+    pub fn bdh_state_log_pending(log: *const bdh_state_log) -> c_int;
+    pub fn bdh_state_log_bytes(log: *const bdh_state_log) -> usize;
+    pub fn bdh_state_step_deferred(ctx: *mut bdh_ctx, log: *mut bdh_state_log, x: *const f32, v: *const f32,
+        freqs: *const f32, position: i64, positions_dev: *const i32, rho: *mut c_void, out: *mut f32,
+        active_bitmask: *mut u64, rows_touched: *mut i32) -> c_int;
+    pub fn bdh_state_flush(ctx: *mut bdh_ctx, log: *mut bdh_state_log, rho: *mut c_void) -> c_int;
     pub fn bdh_relu_lowrank(ctx: *mut bdh_ctx, b: c_int, h_in: c_int, t: c_int, d: c_int, h: c_int, n: c_int,
         input: *const f32, weight: *const f32, bias: *const f32, threshold: f32, block_size: c_int,
         active_blocks_host: *const u8, n_blocks: c_int, gate: *const f32, out: *mut f32) -> c_int;
