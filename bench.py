@@ -649,7 +649,9 @@ def bench_model(args):
             B = args.batch
             steps = 64 if args.steps == 1000 else args.steps
         cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
-        model = bda.BDH(cfg, dev, seed=7, rho_dtype=rho_dtype)
+        model = bda.BDH(cfg, dev, seed=7, rho_dtype=rho_dtype, defer_updates=args.defer)
+        if args.defer:
+            weights_note += f", state updates deferred (log of {args.defer} steps; flushes inside the timed region)"
         prompt = torch.randint(0, 256, (B, args.prompt), generator=torch.Generator().manual_seed(1))
     state = model.init_state()
     chunk = args.prefill_chunk or args.prompt
@@ -674,6 +676,7 @@ def bench_model(args):
     else:
         for _ in range(steps):
             _, nxt = model.forward_with_state(nxt.reshape(B, 1), state, want_next=True)
+    model.materialize_state(state)  # a deferred state is flushed inside the timed region
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -724,6 +727,8 @@ def main():
     ap.add_argument("--alibi-lazy", action="store_true", help="model, shipped sizes: keep the ALiBi state lazily decayed")
     ap.add_argument("--prompt", type=int, default=64, help="model: prompt tokens per sequence")
     ap.add_argument("--graph", action="store_true", help="model: replay one captured HIP graph per token")
+    ap.add_argument("--defer", type=int, default=0, metavar="K",
+                    help="model (c1, c4): decode with deferred state updates, a log of K steps per layer")
     ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="library launch-shape option set on the context before the run (repeatable)")

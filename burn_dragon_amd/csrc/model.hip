@@ -26,7 +26,41 @@ int ensure_act(bdh_model *m, size_t bytes) {
   return BDH_OK;
 }
 
+// Where a call finds the recurrent state of layer l: one allocation [L,B,h,Nq,d] (the layers `layer_bytes` apart) or
+// one pointer per layer, as the reference's ModelState holds it (a Vec of independent per-layer tensors,
+// src/model/state.rs:5-15, each taken and put back by its layer, src/model/bdh.rs:274,304).
+struct StateRefs {
+  void *rho_base = nullptr;
+  void *const *rho_layers = nullptr;
+  int32_t *stamps_base = nullptr;
+  int32_t *const *stamps_layers = nullptr;
+  size_t layer_bytes = 0, stamps_layer = 0;
+  void *rho(int l) const { return rho_layers ? rho_layers[l] : static_cast<char *>(rho_base) + (size_t)l * layer_bytes; }
+  int32_t *stamps(int l) const {
+    return stamps_layers ? stamps_layers[l] : (stamps_base ? stamps_base + (size_t)l * stamps_layer : nullptr);
+  }
+  bool contiguous(int L) const {
+    if (!rho_layers) return true;
+    for (int l = 1; l < L; ++l)
+      if (rho_layers[l] != static_cast<char *>(rho_layers[0]) + (size_t)l * layer_bytes) return false;
+    if (stamps_layers)
+      for (int l = 1; l < L; ++l)
+        if (stamps_layers[l] != stamps_layers[0] + (size_t)l * stamps_layer) return false;
+    return true;
+  }
+};
+
+int model_forward_impl(bdh_model *m, const int64_t *tokens, int B, int T, StateRefs st, int rho_dtype, int64_t position,
+                       const int32_t *positions_dev, float *logits, int64_t *next_tokens, float *x_tap, float *viz,
+                       bdh_model_logs *logs);
+
 }  // namespace
+
+// the update logs of a model's layers (bdh_model_forward_deferred): one bdh_state_log per layer
+struct bdh_model_logs {
+  std::vector<bdh_state_log *> layer;
+  int B = 0, rho_dtype = BDH_F32, capacity = 0;
+};
 
 extern "C" {
 
@@ -117,20 +151,60 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
                           int32_t *stamps, int64_t position, const int32_t *positions_dev, float *logits,
                           int64_t *next_tokens, float *x_tap, float *viz) {
   if (!m) return BDH_E_INVAL;
+  if (B > 0 && T > 0 && !rho) return bdh_fail(m->ctx, BDH_E_INVAL, "null data pointer");
+  StateRefs st;
+  st.rho_base = rho;
+  st.stamps_base = stamps;
+  return model_forward_impl(m, tokens, B, T, st, rho_dtype, position, positions_dev, logits, next_tokens, x_tap, viz,
+                            nullptr);
+}
+
+int bdh_model_forward_layers(bdh_model *m, const int64_t *tokens, int B, int T, void *const *rho_layers_host,
+                             int rho_dtype, int32_t *const *stamps_layers_host, int64_t position,
+                             const int32_t *positions_dev, float *logits, int64_t *next_tokens, float *x_tap) {
+  if (!m) return BDH_E_INVAL;
+  if (B > 0 && T > 0) {
+    if (!rho_layers_host) return bdh_fail(m->ctx, BDH_E_INVAL, "null data pointer");
+    for (int l = 0; l < m->cfg.n_layer; ++l)
+      if (!rho_layers_host[l] || (stamps_layers_host && !stamps_layers_host[l]))
+        return bdh_fail(m->ctx, BDH_E_INVAL, "null state pointer of layer %d", l);
+  }
+  StateRefs st;
+  st.rho_layers = rho_layers_host;
+  st.stamps_layers = stamps_layers_host;
+  return model_forward_impl(m, tokens, B, T, st, rho_dtype, position, positions_dev, logits, next_tokens, x_tap,
+                            nullptr, nullptr);
+}
+
+}  // extern "C"
+
+namespace {
+
+int model_forward_impl(bdh_model *m, const int64_t *tokens, int B, int T, StateRefs st, int rho_dtype, int64_t position,
+                       const int32_t *positions_dev, float *logits, int64_t *next_tokens, float *x_tap, float *viz,
+                       bdh_model_logs *logs) {
   bdh_ctx *ctx = m->ctx;
-  if (stamps && m->cfg.rotary != BDH_ALIBI)
+  const bool has_stamps = st.stamps_base || st.stamps_layers;
+  if (has_stamps && m->cfg.rotary != BDH_ALIBI)
     return bdh_fail(ctx, BDH_E_INVAL, "decay stamps only apply to an ALiBi model");
-  if (stamps && position + T > 0x7fffffffLL) return bdh_fail(ctx, BDH_E_INVAL, "position beyond the stamp range");
+  if (has_stamps && position + T > 0x7fffffffLL) return bdh_fail(ctx, BDH_E_INVAL, "position beyond the stamp range");
   if (B < 0 || T < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative batch or time");
   if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
   if (rho_dtype != BDH_F32 && rho_dtype != BDH_BF16) return bdh_fail(ctx, BDH_E_INVAL, "bad rho_dtype");
   if (B == 0 || T == 0) return BDH_OK;
-  if (!tokens || !rho || !logits) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
-  if (!bdh_aligned(rho, 16)) return bdh_fail(ctx, BDH_E_ALIGN, "rho needs 16-byte alignment");
+  if (!tokens || !logits) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
   const bdh_model_config &c = m->cfg;
   const int d = c.n_embd, h = c.n_head, N = c.latent, V = c.vocab, L = c.n_layer;
   const size_t Nq = c.rotary == BDH_POPE ? 2 * (size_t)N : (size_t)N;
   const size_t M = (size_t)B * T;
+  st.layer_bytes = (size_t)B * h * Nq * d * (rho_dtype == BDH_BF16 ? 2 : 4);
+  st.stamps_layer = (size_t)B * h * N;
+  for (int l = 0; l < L; ++l)
+    if (!bdh_aligned(st.rho(l), 16)) return bdh_fail(ctx, BDH_E_ALIGN, "rho needs 16-byte alignment");
+  // the fused decode forms below walk one allocation: layers given one by one take them only when they are adjacent
+  const bool contiguous = st.contiguous(L);
+  void *rho = st.rho(0);
+  int32_t *stamps = st.stamps(0);
 
   // A decode step (one token per sequence, f32 state, no by-products) need not run kernel by kernel:
   //  * a small model (d <= 256, h*N <= 2048) can run the whole step in ONE launch, a workgroup per sequence; one CU then
@@ -141,7 +215,7 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
   // per layer | kernel by kernel): tiny 77|77|112 at B=1, 84|100|145 at B=64; small 152|82|130 at B=1, 168|127|195 at
   // B=64, 323|442|478 at B=256; base 223|83|123 at B=1, 273|210|240 at B=64, 559|-|654 at B=256; large -|210|308 at
   // B=1, -|519|554 at B=16, -|1092|981 at B=33.
-  if (T == 1 && !x_tap && !viz && ctx->opt_model_one_launch != 0) {
+  if (T == 1 && !x_tap && !viz && !logs && contiguous && ctx->opt_model_one_launch != 0) {
     const size_t w_layer = sizeof(float) * (size_t)3 * h * N * d;
     const size_t w_bytes = w_layer * L;
     const bool small_fits = bdh_model_small_fits(c);
@@ -183,7 +257,6 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
 
   rc = bdh_launch_embed_ln(ctx, tokens, (int64_t)M, d, V, m->w.embed, cur);  // :319-322
   if (rc != BDH_OK) return rc;
-  const size_t rho_layer_bytes = (size_t)B * h * Nq * d * (rho_dtype == BDH_BF16 ? 2 : 4);
   for (int l = 0; l < L; ++l) {  // :336 — the same weights in every layer
     float *x_l = x_tap ? x_tap + (size_t)l * M * h * N : x;
     // :337-351  x = relu(cur . encoder - thr)
@@ -191,11 +264,14 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
     rc = bdh_launch_relu_lowrank(ctx, px);
     if (rc != BDH_OK) return rc;
     // :353-359  recurrent attention (value = cur) and LayerNorm of its output
-    StateStepParams ps{B, h, T, N, d, c.rotary, rho_dtype, x_l, cur, m->freqs, position, positions_dev,
-                       c.rotary == BDH_ALIBI ? m->slopes : nullptr,
-                       static_cast<char *>(rho) + (size_t)l * rho_layer_bytes, attn, nullptr, nullptr,
-                       stamps ? stamps + (size_t)l * B * h * N : nullptr};
-    rc = bdh_launch_state_steps_ln(ctx, ps, attn_ln);
+    if (logs) {  // the update of :298 goes to the layer's log, the state is only read
+      rc = bdh_launch_state_step_deferred(ctx, logs->layer[l], x_l, cur, m->freqs, position, positions_dev, st.rho(l), attn,
+                                          attn_ln, nullptr, nullptr);
+    } else {
+      StateStepParams ps{B, h, T, N, d, c.rotary, rho_dtype, x_l, cur, m->freqs, position, positions_dev,
+                         c.rotary == BDH_ALIBI ? m->slopes : nullptr, st.rho(l), attn, nullptr, nullptr, st.stamps(l)};
+      rc = bdh_launch_state_steps_ln(ctx, ps, attn_ln);
+    }
     if (rc != BDH_OK) return rc;
     // :361-381  xy = x * relu(LN(attn) . encoder_v - thr)
     ReluLowrankParams py{B, h, T, d, h, N, attn_ln, m->w.encoder_v, nullptr, c.relu_threshold, 1, nullptr, 0, x_l, xy};
@@ -216,8 +292,7 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
       rc = bdh_launch_gather_head_rows(ctx, xy, h, hs, off, N, vz + (size_t)2 * h * N);
       if (rc != BDH_OK) return rc;
       if (Nq == (size_t)N)
-        rc = bdh_launch_rho_energy(ctx, B, h, N, d, static_cast<char *>(rho) + (size_t)l * rho_layer_bytes, rho_dtype,
-                                   stamps ? stamps + (size_t)l * B * h * N : nullptr, m->slopes, position + T,
+        rc = bdh_launch_rho_energy(ctx, B, h, N, d, st.rho(l), rho_dtype, st.stamps(l), m->slopes, position + T,
                                    positions_dev, T, vz + (size_t)3 * h * N);
       else  // PoPE: the state has 2N rows, the reference stores a zero map (:413-424)
         rc = bdh_launch_fill_zero_f32(ctx, vz + (size_t)3 * h * N, (long)h * N);
@@ -226,6 +301,78 @@ int bdh_model_forward_viz(bdh_model *m, const int64_t *tokens, int B, int T, voi
     // :383,436-441  cur = LN(cur + LN(mixed . decoder)); the last layer's launch also runs the output head (:446-449)
     const DecoderHead head{m->w.lm_head, T, V, logits, next_tokens};
     rc = bdh_launch_decoder_residual(ctx, B, T, h, N, d, xy, m->w.decoder, cur, l == L - 1 ? &head : nullptr);
+    if (rc != BDH_OK) return rc;
+  }
+  return BDH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int bdh_model_logs_create(bdh_model *m, int B, int rho_dtype, int capacity, bdh_model_logs **out) {
+  if (!m) return BDH_E_INVAL;
+  bdh_ctx *ctx = m->ctx;
+  if (!out) return bdh_fail(ctx, BDH_E_INVAL, "null argument");
+  *out = nullptr;
+  const bdh_model_config &c = m->cfg;
+  if (c.rotary != BDH_ROPE) return bdh_fail(ctx, BDH_E_UNSUPPORTED, "deferred state updates are built for RoPE models");
+  bdh_model_logs *logs = new (std::nothrow) bdh_model_logs();
+  if (!logs) return bdh_fail(ctx, BDH_E_NOMEM, "host allocation failed");
+  logs->B = B;
+  logs->rho_dtype = rho_dtype;
+  logs->capacity = capacity;
+  for (int l = 0; l < c.n_layer; ++l) {
+    bdh_state_log *one = nullptr;
+    const int rc = bdh_state_log_create(ctx, B, c.n_head, c.latent, c.n_embd, rho_dtype, capacity, &one);
+    if (rc != BDH_OK) {
+      for (bdh_state_log *p : logs->layer) bdh_state_log_destroy(ctx, p);
+      delete logs;
+      return rc;
+    }
+    logs->layer.push_back(one);
+  }
+  *out = logs;
+  return BDH_OK;
+}
+
+int bdh_model_logs_destroy(bdh_model *m, bdh_model_logs *logs) {
+  if (!logs) return BDH_OK;
+  for (bdh_state_log *p : logs->layer) bdh_state_log_destroy(m ? m->ctx : nullptr, p);
+  delete logs;
+  return BDH_OK;
+}
+
+int bdh_model_logs_pending(const bdh_model_logs *logs) {
+  return (logs && !logs->layer.empty()) ? bdh_state_log_pending(logs->layer[0]) : BDH_E_INVAL;
+}
+
+int bdh_model_forward_deferred(bdh_model *m, bdh_model_logs *logs, const int64_t *tokens, int B, void *rho, int rho_dtype,
+                               int64_t position, const int32_t *positions_dev, float *logits, int64_t *next_tokens) {
+  if (!m) return BDH_E_INVAL;
+  bdh_ctx *ctx = m->ctx;
+  if (!logs) return bdh_fail(ctx, BDH_E_INVAL, "null model logs");
+  if ((int)logs->layer.size() != m->cfg.n_layer || B != logs->B || rho_dtype != logs->rho_dtype)
+    return bdh_fail(ctx, BDH_E_INVAL, "the logs were created for %zu layers, batch %d, state type %d", logs->layer.size(),
+                    logs->B, logs->rho_dtype);
+  if (!rho) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  StateRefs st;
+  st.rho_base = rho;
+  return model_forward_impl(m, tokens, B, 1, st, rho_dtype, position, positions_dev, logits, next_tokens, nullptr,
+                            nullptr, logs);
+}
+
+int bdh_model_flush(bdh_model *m, bdh_model_logs *logs, void *rho) {
+  if (!m) return BDH_E_INVAL;
+  bdh_ctx *ctx = m->ctx;
+  if (!logs) return bdh_fail(ctx, BDH_E_INVAL, "null model logs");
+  if ((int)logs->layer.size() != m->cfg.n_layer) return bdh_fail(ctx, BDH_E_INVAL, "the logs belong to another model");
+  if (bdh_model_logs_pending(logs) == 0) return BDH_OK;
+  if (!rho) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  const bdh_model_config &c = m->cfg;
+  const size_t layer_bytes = (size_t)logs->B * c.n_head * c.latent * c.n_embd * (logs->rho_dtype == BDH_BF16 ? 2 : 4);
+  for (int l = 0; l < c.n_layer; ++l) {
+    const int rc = bdh_state_flush(ctx, logs->layer[l], static_cast<char *>(rho) + (size_t)l * layer_bytes);
     if (rc != BDH_OK) return rc;
   }
   return BDH_OK;

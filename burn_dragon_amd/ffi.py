@@ -31,7 +31,9 @@ EXPORTS = [
     "bdh_rho_energy", "bdh_model_forward_viz", "bdh_rotate",
     "bdh_model_forward_fast", "bdh_model_forward_fast_ex", "bdh_state_step_noalloc", "bdh_probe_chunks",
     "bdh_state_log_create", "bdh_state_log_destroy", "bdh_state_log_pending", "bdh_state_log_bytes",
-    "bdh_state_step_deferred", "bdh_state_flush",
+    "bdh_state_step_deferred", "bdh_state_flush", "bdh_model_forward_layers",
+    "bdh_model_logs_create", "bdh_model_logs_destroy", "bdh_model_logs_pending", "bdh_model_forward_deferred",
+    "bdh_model_flush",
 ]
 
 
@@ -97,6 +99,12 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_state_log_bytes.argtypes = [P]
     lib.bdh_state_step_deferred.argtypes = [P, P, P, P, P, c_int64, P, P, P, P, P]
     lib.bdh_state_flush.argtypes = [P, P, P]
+    lib.bdh_model_forward_layers.argtypes = [P, P, c_int, c_int, P, c_int, P, c_int64, P, P, P, P]
+    lib.bdh_model_logs_create.argtypes = [P, c_int, c_int, c_int, POINTER(P)]
+    lib.bdh_model_logs_destroy.argtypes = [P, P]
+    lib.bdh_model_logs_pending.argtypes = [P]
+    lib.bdh_model_forward_deferred.argtypes = [P, P, P, c_int, P, c_int, c_int64, P, P, P]
+    lib.bdh_model_flush.argtypes = [P, P, P]
     lib.bdh_relu_lowrank.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_float, c_int, P, c_int,
                                      P, P]
     lib.bdh_layer_norm.argtypes = [P, c_int64, c_int, P, P]

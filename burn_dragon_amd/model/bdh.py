@@ -23,13 +23,17 @@ UINT63_MAX = (1 << 63) - 1
 
 class BDH:
     def __init__(self, config: BDHConfig, device="cuda:0", seed: Optional[int] = None, weights: Optional[dict] = None,
-                 rho_dtype: int = ffi.F32, alibi_lazy: bool = False):
+                 rho_dtype: int = ffi.F32, alibi_lazy: bool = False, defer_updates: int = 0):
         """BDH::new (src/model/bdh.rs:37-84).  `weights` (numpy/torch, the reference's shapes) or a
         seed for Normal(0, 0.02) projections and a Normal(0, 1) embedding.  alibi_lazy (ALiBi models
         only): keep the state lazily decayed, so a step touches only the rows of the active neurons
         instead of multiplying the whole state by exp(-slope) (src/model/bdh.rs:299-301);
-        materialize_state() turns it back into the reference's state."""
+        materialize_state() turns it back into the reference's state.  defer_updates = K > 0 (RoPE models with
+        n_embd in {256, 512}): single-token calls log their state updates (src/model/bdh.rs:298) instead of
+        writing them and the state is rewritten once per K tokens; any other call, and materialize_state(),
+        applies what is pending first, after which the state holds the bits of the eager steps."""
         self.config = config
+        self.defer_updates = int(defer_updates)
         self.alibi_lazy = bool(alibi_lazy)
         self.device = torch.device(device)
         self.n_layer, self.n_embd, self.n_head = config.n_layer, config.n_embd, config.n_head
@@ -69,6 +73,8 @@ class BDH:
         if self.alibi_lazy and rot != RotaryEmbedding.ALIBI:
             raise ValueError("alibi_lazy needs rotary_embedding = alibi")
         self._slopes = slopes
+        if self.defer_updates and (rot != RotaryEmbedding.ROPE or d not in (256, 512)):
+            raise ValueError("defer_updates needs a RoPE model with n_embd in {256, 512}")
 
     @classmethod
     def from_checkpoint_dir(cls, directory: str, device="cuda:0", rho_dtype: int = ffi.F32, alibi_lazy: bool = False):
@@ -105,15 +111,25 @@ class BDH:
             for i, layer in enumerate(state.layers):
                 layer.rho = state.storage[i]
             state.stamps = None
+            state.logs = None  # updates logged against the old storage go with it
         if self.alibi_lazy and state.stamps is None:
             # a state that arrives without stamps is up to date as of its position
             state.stamps = torch.full(shape[:-1], min(state.position, 0x7FFFFFFF), device=self.device,
                                       dtype=torch.int32)
         return state.storage
 
+    def flush_state(self, state: ModelState) -> None:
+        """Applies the logged updates of a model built with defer_updates: afterwards state.storage holds what
+        the eager steps would have left.  No-op when nothing is pending."""
+        logs = getattr(state, "logs", None)
+        if logs is not None and state.storage is not None and logs.pending:
+            self.ctx.check(self.ctx.lib.bdh_model_flush(self.handle, logs.handle, state.storage.data_ptr()))
+
     def materialize_state(self, state: ModelState) -> None:
-        """Applies the pending decay of a lazily decayed ALiBi state: afterwards state.storage is the
-        state the reference holds after state.position tokens.  No-op for an eager state."""
+        """Applies the pending decay of a lazily decayed ALiBi state, or the logged updates of a deferred one:
+        afterwards state.storage is the state the reference holds after state.position tokens.  No-op for an
+        eager state."""
+        self.flush_state(state)
         if state.storage is None or state.stamps is None:
             return
         from ..recurrent import alibi_materialize
@@ -132,6 +148,15 @@ class BDH:
         rho = self._ensure_state(state, B)
         logits = torch.empty((B, T, self.vocab_size), device=self.device, dtype=torch.float32)
         nxt = torch.empty((B,), device=self.device, dtype=torch.int64) if want_next else None
+        if self.defer_updates and T == 1 and x_tap is None and not viz:
+            if state.logs is None or state.logs.batch != B:
+                state.logs = ModelLogs(self, B, self.defer_updates)
+            self.ctx.check(self.ctx.lib.bdh_model_forward_deferred(self.handle, state.logs.handle, tokens.data_ptr(), B,
+                                                                   rho.data_ptr(), self.rho_dtype, state.position, None,
+                                                                   logits.data_ptr(), ffi.ptr(nxt)))
+            state.position = min(state.position + T, UINT63_MAX)
+            return (logits, nxt) if want_next else logits
+        self.flush_state(state)  # a call that writes the state itself: the logged updates go first
         maps = None
         if viz and T > 0:
             maps = torch.empty((self.n_layer, 4, self.n_head, self.latent), device=self.device, dtype=torch.float32)
@@ -204,6 +229,29 @@ class BDH:
         return torch.cat(out, dim=1)
 
 
+class ModelLogs:
+    """bdh_model_logs: the update logs of a model's layers for a batch of `batch` sequences."""
+
+    def __init__(self, model: BDH, batch: int, capacity: int):
+        self.model, self.batch, self.capacity = model, batch, capacity
+        handle = ctypes.c_void_p()
+        model.ctx.check(model.ctx.lib.bdh_model_logs_create(model.handle, batch, model.rho_dtype, capacity,
+                                                            ctypes.byref(handle)))
+        self.handle = handle
+
+    @property
+    def pending(self) -> int:
+        return int(self.model.ctx._lib.bdh_model_logs_pending(self.handle))
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None) and getattr(self.model, "handle", None) and not sys.is_finalizing():
+                self.model.ctx._lib.bdh_model_logs_destroy(self.model.handle, self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
 class DecodeGraph:
     """One captured decode step.  `tokens` [B] int64 are the tokens to feed first (e.g. the argmax of the
     prefill); after each replay() the buffer holds the newly generated tokens and `logits` [B,1,V] the
@@ -211,6 +259,7 @@ class DecodeGraph:
 
     def __init__(self, model: BDH, state: ModelState, tokens: torch.Tensor):
         assert state.storage is not None, "run the prefill before capturing the decode step"
+        model.flush_state(state)  # the captured step writes the state itself (the pending count of a log lives on the host)
         self.model, self.state = model, state
         B = state.storage.shape[1]
         dev = model.device

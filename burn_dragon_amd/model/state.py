@@ -38,6 +38,8 @@ class ModelState:
     # ALiBi with lazy decay only: [L,B,h,N] int32, the token count at which each state row was last brought
     # up to date (see BDH(alibi_lazy=True)); None for an eagerly decayed state
     stamps: Optional[torch.Tensor] = None
+    # a model built with defer_updates only: the update logs of its layers (BDH.flush_state applies them)
+    logs: Optional[object] = None
 
     @classmethod
     def new(cls, num_layers: int) -> "ModelState":
@@ -48,6 +50,7 @@ class ModelState:
             layer.rho = None
         self.storage = None
         self.stamps = None
+        self.logs = None
         self.position = 0
 
     def len(self) -> int:

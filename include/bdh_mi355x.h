@@ -423,6 +423,16 @@ int bdh_model_forward_lazy(bdh_model *model, const int64_t *tokens, int B, int T
                            const int32_t *positions_dev, float *logits, int64_t *next_tokens,
                            float *x_tap);
 
+/* bdh_model_forward_lazy with the state given layer by layer, the way the reference holds it: ModelState is a
+ * Vec<LayerState> of independent Option<Tensor<B,4>> (src/model/state.rs:5-15), each taken out and put back by its
+ * layer (src/model/bdh.rs:274,304).  rho_layers_host: HOST array of n_layer DEVICE pointers, layer l's state
+ * [B,h,Nq,d]; stamps_layers_host: the same for the decay stamps [B,h,N] of a lazily decayed ALiBi state, or NULL.
+ * Results are those of the one-allocation entry points bit for bit.  (Layers that happen to lie adjacent in memory
+ * also take the fused decode forms of option "model.one_launch"; separate allocations run kernel by kernel.) */
+int bdh_model_forward_layers(bdh_model *model, const int64_t *tokens, int B, int T, void *const *rho_layers_host,
+                             int rho_dtype, int32_t *const *stamps_layers_host, int64_t position,
+                             const int32_t *positions_dev, float *logits, int64_t *next_tokens, float *x_tap);
+
 /* The energy map of a state: out[h,N] = (sum over b of (sum over c of |rho[b,h,n,c]|) / d) / B, the
  * `rho_last` of LayerVizState (src/model/bdh.rs:411-419, built under the reference's "viz" feature).
  * rho [B,h,N,d] f32 or bf16.  stamps [B,h,N] (optional, ALiBi only) marks a lazily decayed state, read
@@ -442,6 +452,22 @@ int bdh_model_forward_viz(bdh_model *model, const int64_t *tokens, int B, int T,
                           int rho_dtype, int32_t *stamps, int64_t position,
                           const int32_t *positions_dev, float *logits, int64_t *next_tokens,
                           float *x_tap, float *viz);
+
+/* A decode step (T = 1) of bdh_model_forward_ex with the state updates of every layer deferred
+ * (bdh_state_step_deferred in place of the step of src/model/bdh.rs:288-302): RoPE models with n_embd in {256, 512}.
+ * `logs` holds one update log per layer for a batch of B sequences (capacity as in bdh_state_log_create; every
+ * layer logs one step per call, so all layers fill and flush together, the call that finds the logs full flushing
+ * them first).  Until bdh_model_flush, rho [L,B,h,N,d] lags behind by the pending steps; flush before any other
+ * entry point (a prompt call, bdh_model_forward*, bdh_rho_energy, an export) touches rho.  Logits agree with
+ * bdh_model_forward_ex to f32 rounding of the reassociated readout; the flushed state holds its bits. */
+typedef struct bdh_model_logs bdh_model_logs; /* opaque: one bdh_state_log per layer */
+int bdh_model_logs_create(bdh_model *model, int B, int rho_dtype, int capacity, bdh_model_logs **out);
+int bdh_model_logs_destroy(bdh_model *model, bdh_model_logs *logs);
+int bdh_model_logs_pending(const bdh_model_logs *logs);
+int bdh_model_forward_deferred(bdh_model *model, bdh_model_logs *logs, const int64_t *tokens, int B, void *rho,
+                               int rho_dtype, int64_t position, const int32_t *positions_dev, float *logits,
+                               int64_t *next_tokens);
+int bdh_model_flush(bdh_model *model, bdh_model_logs *logs, void *rho);
 
 /* Draws the next token of every sequence on the device.  Replaces the temperature division of
  * sample_next_token (src/generation.rs:117) and sample_from_logits_values (src/generation.rs:26-72),

@@ -31,6 +31,12 @@ pub struct bdh_state_log {
     _private: [u8; 0],
 }
 
+/// opaque: one bdh_state_log per layer of a model (the deferred decode step of a whole model)
+#[repr(C)]
+pub struct bdh_model_logs {
+    _private: [u8; 0],
+}
+
 pub const BDH_OK: c_int = 0;
 pub const BDH_E_INVAL: c_int = -1;
 pub const BDH_E_SHAPE: c_int = -2;
@@ -149,12 +155,23 @@ extern "C" {
     pub fn bdh_model_forward_lazy(model: *mut bdh_model, tokens: *const i64, b: c_int, t: c_int,
         rho: *mut c_void, rho_dtype: c_int, stamps: *mut i32, position: i64, positions_dev: *const i32,
         logits: *mut f32, next_tokens: *mut i64, x_tap: *mut f32) -> c_int;
+    pub fn bdh_model_forward_layers(model: *mut bdh_model, tokens: *const i64, b: c_int, t: c_int,
+        rho_layers_host: *const *mut c_void, rho_dtype: c_int, stamps_layers_host: *const *mut i32, position: i64,
+        positions_dev: *const i32, logits: *mut f32, next_tokens: *mut i64, x_tap: *mut f32) -> c_int;
     pub fn bdh_rho_energy(ctx: *mut bdh_ctx, b: c_int, h: c_int, n: c_int, d: c_int, rho: *const c_void,
         rho_dtype: c_int, stamps: *const i32, clock: i64, clocks_dev: *const i32,
         alibi_slopes_host: *const f32, out: *mut f32) -> c_int;
     pub fn bdh_model_forward_viz(model: *mut bdh_model, tokens: *const i64, b: c_int, t: c_int,
         rho: *mut c_void, rho_dtype: c_int, stamps: *mut i32, position: i64, positions_dev: *const i32,
         logits: *mut f32, next_tokens: *mut i64, x_tap: *mut f32, viz: *mut f32) -> c_int;
+    pub fn bdh_model_logs_create(model: *mut bdh_model, b: c_int, rho_dtype: c_int, capacity: c_int,
+        out: *mut *mut bdh_model_logs) -> c_int;
+    pub fn bdh_model_logs_destroy(model: *mut bdh_model, logs: *mut bdh_model_logs) -> c_int;
+    pub fn bdh_model_logs_pending(logs: *const bdh_model_logs) -> c_int;
+    pub fn bdh_model_forward_deferred(model: *mut bdh_model, logs: *mut bdh_model_logs, tokens: *const i64, b: c_int,
+        rho: *mut c_void, rho_dtype: c_int, position: i64, positions_dev: *const i32, logits: *mut f32,
+        next_tokens: *mut i64) -> c_int;
+    pub fn bdh_model_flush(model: *mut bdh_model, logs: *mut bdh_model_logs, rho: *mut c_void) -> c_int;
     pub fn bdh_sample_top_k(ctx: *mut bdh_ctx, b: c_int, v: c_int, logits: *const f32, row_stride: i64,
         temperature: f32, top_k: c_int, uniforms: *const f32, next_tokens: *mut i64) -> c_int;
     pub fn bdh_probe_chunks(ctx: *mut bdh_ctx, region: *mut c_void, region_bytes: usize,
