@@ -207,7 +207,7 @@ def test_config5_step_against_oracle(bda, corc, B, density, dtype, tol):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
-@pytest.mark.parametrize("density", [0.01, 0.20])
+@pytest.mark.parametrize("density", [0.01, 0.02, 0.05, 0.10, 0.20])
 def test_config5_step_at_batch_64_properties(bda, corc, density, dtype, tol):
     """B=64 of the sweep (f32 state: 16 GiB): the step against an f32 torch statement of the same sums with q
     from the oracle's rotate, the index by-products against their definitions, and untouched rows bit-identical."""

@@ -350,6 +350,44 @@ def test_prefill_chunked_config3_shape_properties(bda, corc, unequal_pairs):
     assert rel_err(rho.cpu().numpy(), qtv.cpu().numpy()) < 2e-2
 
 
+def test_prefill_chunked_config3_at_its_own_batch(bda, corc):
+    """BASELINE config 3 at its full size (B=8, h=4, T=2048, N=8192, d=256, 5 % density, fresh state): the 32-slice
+    launch that bench.py times, checked without the oracle's token loop (too slow at this size):
+      - the first token of every slice reads a zero state: out[:, :, 0] == 0;
+      - the final state is Q^T V (src/model/bdh.rs:298 summed over the tokens), with Q = bf16(rope(x)) from the
+        oracle's rotate and the product by a device einsum, one batch entry at a time;
+      - slices are independent: (b=0, h=0..1) of this call hold the same bits as a B=1, h=2 call on those inputs
+        (the call test_prefill_chunked_config3_shape_properties checks against the oracle);
+      - out against the closed causal form tril(-1)(Q Q^T) V on the device for one slice."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h, T, N, d = 8, 4, 2048, 8192, 256
+    x, v, _ = _prefill_case(11, B, h, T, N, d, 0.05, 0.0)
+    freqs = corc.build_freqs(N)
+    ft = torch.from_numpy(freqs).to(DEV)
+    xt, vt = x.to(DEV), v.to(DEV)
+    rho = torch.zeros((B, h, N, d), device=DEV)
+    print("prefill config 3 at B=8, h=4", flush=True)
+    out = prefill_chunked(xt, vt, rho, ft, 0, state_is_zero=True)
+    torch.cuda.synchronize()
+    assert not out[:, :, 0].any()
+    for b in range(B):  # Q of one batch entry: [h, T, N] f32 = 256 MiB
+        q = torch.from_numpy(corc.rotate(x[b:b + 1].float().numpy(), freqs, orc.ROPE, 0)).to(DEV)
+        q = q.to(torch.bfloat16).float()  # the products take the rotated activations rounded to bf16
+        qtv = torch.einsum("htn,td->hnd", q[0], vt[b].float())
+        err = float((rho[b] - qtv).abs().max()) / float(qtv.abs().max())
+        assert err < 2e-2, f"batch entry {b}: {err}"
+        if b == 0:  # the causal closed form for one slice
+            s = torch.tril(q[0, 0] @ q[0, 0].T, -1)
+            o = s @ vt[0].float()
+            err_o = float((out[0, 0] - o).abs().max()) / float(o.abs().max())
+            assert err_o < 2e-2, err_o
+    rho2 = torch.zeros((1, 2, N, d), device=DEV)
+    out2 = prefill_chunked(xt[:1, :2].contiguous(), vt[:1].contiguous(), rho2, ft, 0, state_is_zero=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out2[0], out[0, :2]) and torch.equal(rho2[0], rho[0, :2])
+
+
 def test_prefill_chunked_argument_errors(bda):
     from burn_dragon_amd import ffi
 
