@@ -150,8 +150,10 @@ class Context:
     """bdh_ctx bound to a device and a HIP stream.  Without an explicit stream the context follows torch's
     current stream: every access to `.lib` (each wrapper fetches it right before its call) re-binds the context
     when the current stream has changed, so tensors torch allocates or fills on that stream and the library's
-    kernels stay ordered, also inside `with torch.cuda.stream(s)` and under graph capture.  A context created
-    with a stream, or given one through set_stream(..., pin=True), keeps it."""
+    kernels stay ordered, also inside `with torch.cuda.stream(s)` and under graph capture; on such a re-bind the
+    new stream first waits for what the old one still has queued (the context's workspace is shared by all calls).
+    A context created with a stream, or given one through set_stream(..., pin=True), keeps it.  Work that should
+    overlap on two streams needs two contexts."""
 
     def __init__(self, device_id: int = 0, stream: Optional[int] = None):
         self._lib = load_library()
@@ -173,8 +175,18 @@ class Context:
         if self._follow and getattr(self, "handle", None) and not sys.is_finalizing():
             import torch
 
-            current = torch.cuda.current_stream(self.device_id).cuda_stream
+            cur = torch.cuda.current_stream(self.device_id)
+            current = cur.cuda_stream
             if current != self._stream:
+                # The context's workspace and the model's activation scratch are shared by every call: work queued on
+                # the old stream may still use them, so the new stream waits for it (not under graph capture, where
+                # an event recorded outside the capture must not be waited on; a capture orders its own work).
+                if not torch.cuda.is_current_stream_capturing():
+                    old = (torch.cuda.ExternalStream(self._stream, device=self.device_id) if self._stream
+                           else torch.cuda.default_stream(self.device_id))
+                    done = torch.cuda.Event()
+                    done.record(old)
+                    cur.wait_event(done)
                 self._lib.bdh_ctx_set_stream(self.handle, current or None)
                 self._stream = current
         return self._lib

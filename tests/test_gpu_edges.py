@@ -243,6 +243,45 @@ def test_context_follows_torchs_current_stream(bda, corc):
     assert np.isfinite(out2.cpu().numpy()).all()
 
 
+def test_context_rebind_orders_the_shared_workspace_between_streams(bda, corc):
+    """Two calls through the default context on two different streams with no synchronisation in between: both use the
+    context's one workspace (the prefill's rotated activations, state copies and value layouts), so the second stream
+    must wait for the first stream's kernels at the re-bind.  Each call against the same call run alone."""
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h, T, N, d = 2, 4, 1024, 2048, 256
+    g = torch.Generator().manual_seed(3)
+    cases = []
+    for _ in range(2):
+        x = torch.relu(torch.randn((B, h, T, N), generator=g) - 1.3).to(torch.bfloat16).to(DEV)
+        v = torch.randn((B, T, d), generator=g).to(torch.bfloat16).to(DEV)
+        cases.append((x, v))
+    ft = torch.from_numpy(corc.build_freqs(N)).to(DEV)
+    alone = []
+    for x, v in cases:
+        rho = torch.zeros((B, h, N, d), device=DEV)
+        out = prefill_chunked(x, v, rho, ft, 0, state_is_zero=True)
+        torch.cuda.synchronize()
+        alone.append((out.clone(), rho.clone()))
+    s1, s2 = torch.cuda.Stream(device=DEV), torch.cuda.Stream(device=DEV)
+    rhos = [torch.zeros((B, h, N, d), device=DEV) for _ in range(2)]
+    torch.cuda.synchronize()
+    outs = []
+    for _ in range(3):  # a few rounds: the calls of the two streams alternate back to back
+        outs.clear()
+        for rho in rhos:
+            rho.zero_()
+        torch.cuda.synchronize()
+        for (x, v), rho, stream in zip(cases, rhos, (s1, s2)):
+            with torch.cuda.stream(stream):
+                outs.append(prefill_chunked(x, v, rho, ft, 0, state_is_zero=True))
+        torch.cuda.synchronize()
+        for (out, rho), (out_a, rho_a) in zip(zip(outs, rhos), alone):
+            assert torch.equal(out, out_a) and torch.equal(rho, rho_a)
+    assert ffi.default_context(0)._stream == s2.cuda_stream
+
+
 def test_probe_chunks_moves_exactly_the_listed_chunks(bda):
     """bdh_probe_chunks (the decode step's memory traffic without its arithmetic): mode 0 reads the listed chunks,
     scales by 1 and writes them back -- the region is unchanged; mode 1 only reads; mode 2 writes zeros into the
