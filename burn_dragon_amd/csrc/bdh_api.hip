@@ -83,9 +83,10 @@ int bdh_ctx_create(int device_id, void *hip_stream, bdh_ctx **out) {
 
 int bdh_ctx_destroy(bdh_ctx *ctx) {
   if (!ctx) return BDH_OK;
-  if (ctx->ws || ctx->fsa_mask) (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->ws || ctx->fsa_mask || ctx->lat_mask) (void)hipStreamSynchronize(ctx->stream);
   if (ctx->ws) (void)hipFree(ctx->ws);
   if (ctx->fsa_mask) (void)hipFree(ctx->fsa_mask);
+  if (ctx->lat_mask) (void)hipFree(ctx->lat_mask);
   delete ctx;
   return BDH_OK;
 }

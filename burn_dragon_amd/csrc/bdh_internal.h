@@ -35,6 +35,10 @@ struct bdh_ctx {
   void *fsa_mask = nullptr;
   size_t fsa_mask_bytes = 0;
   std::vector<int> fsa_mask_key;
+  // latent block mask of the last relu_lowrank call that had one (device) and the bytes it was built from
+  void *lat_mask = nullptr;
+  size_t lat_mask_bytes = 0;
+  std::vector<uint8_t> lat_mask_key;
   char err[512] = {0};
 };
 

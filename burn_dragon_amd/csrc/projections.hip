@@ -4,6 +4,7 @@
 // :346-350, :370-384, :436-449.
 #include "bdh_internal.h"
 
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 
@@ -946,15 +947,29 @@ int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p) {
   if (M > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "B*T too large");
   const unsigned char *mask_dev = nullptr;
   if (p.active_blocks_host) {
-    int rc = bdh_ws_reserve(ctx, (size_t)p.n_blocks + 256);
-    if (rc != BDH_OK) return rc;
-    // the caller's host buffer may go away on return: finish the copy before returning
-    if (p.n_blocks > 0) {
-      BDH_HIP_CHECK(ctx, hipMemcpyAsync(ctx->ws, p.active_blocks_host, (size_t)p.n_blocks,
-                                        hipMemcpyHostToDevice, ctx->stream));
+    // The device copy of the mask is kept with the bytes it was made from: the two projections of every layer of
+    // a call (and the calls after it) pass the same pattern, and only a new pattern costs a copy and a wait (the
+    // caller's host buffer may go away on return, and kernels still queued may read the old copy).
+    const size_t nb = (size_t)std::max(p.n_blocks, 0);
+    const bool same = ctx->lat_mask && ctx->lat_mask_key.size() == nb &&
+                      (nb == 0 || memcmp(ctx->lat_mask_key.data(), p.active_blocks_host, nb) == 0);
+    if (!same) {
       BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+      if (ctx->lat_mask_bytes < nb + 256) {
+        if (ctx->lat_mask) BDH_HIP_CHECK(ctx, hipFree(ctx->lat_mask));
+        ctx->lat_mask = nullptr;
+        ctx->lat_mask_bytes = 0;
+        ctx->lat_mask_key.clear();
+        if (hipMalloc(&ctx->lat_mask, nb + 256) != hipSuccess) {
+          (void)hipGetLastError();
+          return bdh_fail(ctx, BDH_E_NOMEM, "latent block mask of %zu bytes", nb);
+        }
+        ctx->lat_mask_bytes = nb + 256;
+      }
+      if (nb > 0) BDH_HIP_CHECK(ctx, hipMemcpy(ctx->lat_mask, p.active_blocks_host, nb, hipMemcpyHostToDevice));
+      ctx->lat_mask_key.assign(p.active_blocks_host, p.active_blocks_host + nb);
     }
-    mask_dev = static_cast<const unsigned char *>(ctx->ws);
+    mask_dev = static_cast<const unsigned char *>(ctx->lat_mask);
   }
   const bool aligned16 = bdh_aligned(p.in, 16) && bdh_aligned(p.weight, 16) && bdh_aligned(p.out, 16) &&
                          bdh_aligned(p.bias, 16) && bdh_aligned(p.gate, 16);

@@ -23,6 +23,12 @@
  *   - Entry points may grow the context's workspace (hipMalloc) the first time a shape is seen: run a
  *     step of each shape once before capturing calls in a HIP graph.
  *   - There is no CPU fallback: without a HIP device every compute entry point fails.
+ *   - State (`rho`) and output (`out`) buffers are ordinary device memory (hipMalloc: coarse-grained).  Calls
+ *     of many tokens add their products into them with the L2's no-return f32 adder (one add per element and call,
+ *     so no ordering question); fine-grained or host-coherent allocations may not perform such an add and would
+ *     lose updates silently.  Sums of that path below the smallest normal float are flushed to zero.
+ *   - bdh_ctx_set_stream only swaps the stream: the context's workspace is shared by all of its calls, so the
+ *     caller orders the old stream's queued work before the new stream's (an event), or uses one context per stream.
  */
 #ifndef BDH_MI355X_H
 #define BDH_MI355X_H
@@ -187,7 +193,8 @@ int bdh_state_step(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const f
  * for RoPE at d in {256,512}, N/128 when that grid would leave CUs idle, N/64 for the other kernels).
  * BASELINE configs 2 and 4 need 2 and 16 MiB.  All calls on one device share the array: calls that overlap on one device (two streams, two
  * contexts) race; calls ordered on one stream do not.  Nothing in the array has to start at zero: every
- * element that is read was written by the same call. */
+ * element that is read was written by the same call.  The array's address is kept for device ids 0..63; a context
+ * on a device beyond that returns BDH_E_UNSUPPORTED here. */
 int bdh_state_step_noalloc(bdh_ctx *ctx, int B, int h, int N, int d, int rotary, const float *x,
                            const float *v, const float *freqs, int64_t position,
                            const int32_t *positions_dev, const float *alibi_slopes_host, void *rho,

@@ -152,11 +152,14 @@ def test_relu_lowrank_on_the_matrix_cores_with_every_option(bda, corc, M, d, N, 
     assert 0.05 < (ref > 0).mean() < 0.6
 
 
-@pytest.mark.parametrize("B,T,h_in,d,N", [(2, 100, 1, 256, 640), (1, 300, 3, 72, 203), (3, 64, 1, 512, 1024)])
+@pytest.mark.parametrize("B,T,h_in,d,N", [(2, 100, 1, 256, 640), (1, 300, 3, 72, 203), (3, 64, 1, 512, 1024),
+                                          (4, 130, 1, 64, 8192)])
 def test_relu_lowrank_as_a_matrix_core_product_per_sequence(bda, corc, B, T, h_in, d, N):
     """Many tokens per sequence: one f32 matrix-core product per (sequence, head) whose k order is that of a scalar
     loop, so the outputs are again the bits of the oracle's fmaf chain -- with bias, threshold, block mask and gate,
-    ragged tiles in rows, columns and k (K = 72 is not a multiple of the 16-wide stage), wide value ranges."""
+    ragged tiles in rows, columns and k (K = 72 is not a multiple of the 16-wide stage), wide value ranges.  The last
+    case (N a multiple of 256, 768 tiles of 128 x 256) takes the wide-tile instance that long prompts of a large
+    model run on."""
     from burn_dragon_amd.kernel import relu_lowrank
 
     h = 3

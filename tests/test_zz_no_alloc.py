@@ -26,7 +26,7 @@ def _inputs(seed, B, h, N, d, density, Nq):
     return x, v, rho
 
 
-def _call(ffi, ctx, fn, x, v, rho, freqs, position, rotary, dtype):
+def _call(ffi, ctx, fn, x, v, rho, freqs, position, rotary, dtype, check_no_allocation=False):
     dev = "cuda:0"
     B, h, N = x.shape
     d = v.shape[1]
@@ -38,9 +38,12 @@ def _call(ffi, ctx, fn, x, v, rho, freqs, position, rotary, dtype):
     torch.cuda.synchronize()
     ctx.set_stream(torch.cuda.current_stream(0).cuda_stream)
     print(f"{fn.__name__} B={B} h={h} N={N} d={d} rotary={rotary} dtype={dtype}", flush=True)
+    free_before = torch.cuda.mem_get_info(0)[0]  # every tensor of the call exists already
     ctx.check(fn(ctx.handle, B, h, N, d, rotary, ffi.ptr(xt), ffi.ptr(vt), ffi.ptr(ft), position, None, None,
                  ffi.ptr(rt), ffi.F32 if dtype == torch.float32 else ffi.BF16, ffi.ptr(out), ffi.ptr(bm), ffi.ptr(rows)))
     torch.cuda.synchronize()
+    if check_no_allocation:  # the driver's count of free device memory has not moved: no hipMalloc, no workspace growth
+        assert torch.cuda.mem_get_info(0)[0] == free_before
     return out.cpu().numpy(), rt.float().cpu().numpy(), bm.cpu().numpy(), rows.cpu().numpy()
 
 
@@ -53,14 +56,16 @@ def test_noalloc_step_equals_the_allocating_step_twice_in_a_row(corc, rotary, dt
 
     lib = ffi.load_library()
     ctx = ffi.Context(0)  # a fresh context: its workspace is empty, and the new entry point never grows it
+    ctx_ref = ffi.Context(0)  # the allocating entry point runs on a context of its own
     try:
         # first call large (many workgroups per slice), second call smaller in every dimension
         for seed, (B, h, N, d, density) in enumerate([(4, 4, 4096, 256, 0.05), (2, 2, 640, 256, 0.3)]):
             x, v, rho = _inputs(40 + seed, B, h, N, d, density, 2 * N if rotary == orc.POPE else N)
             freqs = corc.build_freqs(N, rotary=rotary) if rotary != orc.ALIBI else np.zeros(N, np.float32)
             position = 777 + seed
-            got = _call(ffi, ctx, lib.bdh_state_step_noalloc, x, v, rho, freqs, position, rotary, dtype)
-            ref = _call(ffi, ctx, lib.bdh_state_step, x, v, rho, freqs, position, rotary, dtype)
+            got = _call(ffi, ctx, lib.bdh_state_step_noalloc, x, v, rho, freqs, position, rotary, dtype,
+                        check_no_allocation=True)
+            ref = _call(ffi, ctx_ref, lib.bdh_state_step, x, v, rho, freqs, position, rotary, dtype)
             for a, b, name in zip(got, ref, ("out", "rho", "bitmask", "rows_touched")):
                 assert np.array_equal(a, b), (name, seed)
             if dtype == torch.float32:
@@ -71,6 +76,7 @@ def test_noalloc_step_equals_the_allocating_step_twice_in_a_row(corc, rotary, dt
                 assert np.abs(got[1] - rho_ref).max() <= 1e-3 * np.abs(rho_ref).max()
     finally:
         ctx.close()
+        ctx_ref.close()
 
 
 def test_noalloc_step_rejects_a_shape_beyond_its_scratch():
