@@ -28,6 +28,15 @@ __device__ __forceinline__ unsigned short f32_to_bf16(float f) {  // round to ne
   return static_cast<unsigned short>(u >> 16);
 }
 
+// two floats rounded to bf16 by the hardware conversion (v_cvt_pk_bf16_f32: nearest even, the bits of f32_to_bf16
+// for every finite value), packed low | high
+__device__ __forceinline__ unsigned int pack_bf16_rne(float lo, float hi) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t a = {lo, hi};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(a, bf16x2_t));
+}
+
 // spread the 32 bits of v to the even bit positions of a 64-bit word
 __device__ __forceinline__ unsigned long long spread_bits(unsigned int v) {
   unsigned long long x = v;

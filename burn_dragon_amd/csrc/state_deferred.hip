@@ -20,6 +20,7 @@
 //   scores [unit][128]     this step's partial dot products q_t . q_s over the unit's pairs (scratch)
 #include <algorithm>
 #include <new>
+#include <type_traits>
 
 #include "bdh_internal.h"
 #include "state_common.h"
@@ -57,15 +58,21 @@ struct PairFrag {
     return kF32 ? ((g % (D / 256)) * 64 + lane) * 4 : ((g * 64 + lane) * 8) % D;
   }
   // Rows are streamed: every access is non-temporal, so that the lines of the log, which are read again on the
-  // next step, are the ones the caches keep.
-  __device__ static __forceinline__ void load_nt(const RhoT *pair, int g, int lane, float (&f)[GW]) {
-    typedef float v4f __attribute__((ext_vector_type(4)));
-    typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+  // next step, are the ones the caches keep.  A group travels as one 16-byte register quad (Raw) and is widened to
+  // floats where it is used, so that many groups can be in flight per lane.
+  typedef float v4f __attribute__((ext_vector_type(4)));
+  typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+  using Raw = typename std::conditional<kF32, v4f, v4u>::type;
+  __device__ static __forceinline__ Raw load_raw(const RhoT *pair, int g, int lane) {
+    if constexpr (kF32)
+      return __builtin_nontemporal_load(reinterpret_cast<const v4f *>(pair + row(g, lane) * D + col(g, lane)));
+    else
+      return __builtin_nontemporal_load(reinterpret_cast<const v4u *>(pair + (g * 64 + lane) * 8));
+  }
+  __device__ static __forceinline__ void expand(const Raw &t, float (&f)[GW]) {
     if constexpr (kF32) {
-      const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(pair + row(g, lane) * D + col(g, lane)));
       f[0] = t.x; f[1] = t.y; f[2] = t.z; f[3] = t.w;
     } else {
-      const v4u t = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(pair + (g * 64 + lane) * 8));
       const unsigned int w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -74,18 +81,38 @@ struct PairFrag {
       }
     }
   }
+  __device__ static __forceinline__ void load_nt(const RhoT *pair, int g, int lane, float (&f)[GW]) {
+    expand(load_raw(pair, g, lane), f);
+  }
+  // two floats rounded to bf16 (nearest even, the hardware conversion; the bits of f32_to_bf16 for every finite
+  // value), packed low | high
+  __device__ static __forceinline__ unsigned int pack_bf16(float lo, float hi) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const f32x2 a = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(a, bf16x2));
+  }
+  // a bf16 state holds bf16 values after every step: the floats of a group rounded in place
+  __device__ static __forceinline__ void round_in_place(float (&f)[GW]) {
+    if constexpr (!kF32) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const unsigned int pk = pack_bf16(f[2 * k], f[2 * k + 1]);
+        f[2 * k] = __uint_as_float(pk << 16);
+        f[2 * k + 1] = __uint_as_float(pk & 0xffff0000u);
+      }
+    }
+  }
   __device__ static __forceinline__ void store_nt(RhoT *pair, int g, int lane, const float (&f)[GW]) {
-    typedef float v4f __attribute__((ext_vector_type(4)));
-    typedef unsigned int v4u __attribute__((ext_vector_type(4)));
     if constexpr (kF32) {
       v4f t; t.x = f[0]; t.y = f[1]; t.z = f[2]; t.w = f[3];
       __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(pair + row(g, lane) * D + col(g, lane)));
     } else {
       v4u o;
-      o.x = (unsigned int)f32_to_bf16(f[0]) | ((unsigned int)f32_to_bf16(f[1]) << 16);
-      o.y = (unsigned int)f32_to_bf16(f[2]) | ((unsigned int)f32_to_bf16(f[3]) << 16);
-      o.z = (unsigned int)f32_to_bf16(f[4]) | ((unsigned int)f32_to_bf16(f[5]) << 16);
-      o.w = (unsigned int)f32_to_bf16(f[6]) | ((unsigned int)f32_to_bf16(f[7]) << 16);
+      o.x = pack_bf16(f[0], f[1]);
+      o.y = pack_bf16(f[2], f[3]);
+      o.z = pack_bf16(f[4], f[5]);
+      o.w = pack_bf16(f[6], f[7]);
       __builtin_nontemporal_store(o, reinterpret_cast<v4u *>(pair + (g * 64 + lane) * 8));
     }
   }
@@ -229,16 +256,14 @@ __global__ __launch_bounds__(256) void k_step_deferred(DeferArgs a, const RhoT *
     for (int e = 0; e < GW; ++e) acc[g][e] = 0.0f;
   const RhoT *base = rho + ((long)slice * a.N + 2L * seg * kUnitPairs) * D;
   for (int i0 = wave; i0 < total; i0 += 4 * U) {
-    float r[U][NG][GW];
+    typename F::Raw r[U][NG];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int i = i0 + u * 4;
       if (i < total) {
         const RhoT *pp = base + (long)s_idx[i] * (2 * D);
 #pragma unroll
-        for (int g = 0; g < NG; ++g) {
-          F::load_nt(pp, g, lane, r[u][g]);
-        }
+        for (int g = 0; g < NG; ++g) r[u][g] = F::load_raw(pp, g, lane);
       }
     }
 #pragma unroll
@@ -249,8 +274,10 @@ __global__ __launch_bounds__(256) void k_step_deferred(DeferArgs a, const RhoT *
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
           const float qf = F::row(g, lane) ? qq.y : qq.x;
+          float f[GW];
+          F::expand(r[u][g], f);
 #pragma unroll
-          for (int e = 0; e < GW; ++e) acc[g][e] = __builtin_fmaf(r[u][g][e], qf, acc[g][e]);
+          for (int e = 0; e < GW; ++e) acc[g][e] = __builtin_fmaf(f[e], qf, acc[g][e]);
         }
       }
     }
@@ -476,10 +503,7 @@ __device__ __forceinline__ void flush_apply(float (&r)[NG_][GW_], const float *v
       t = qf * v4.z; r[g][e4 + 2] = r[g][e4 + 2] + t;
       t = qf * v4.w; r[g][e4 + 3] = r[g][e4 + 3] + t;
     }
-    if constexpr (!F::kF32) {  // the eager step stores bf16 after every token
-#pragma unroll
-      for (int e = 0; e < F::GW; ++e) r[g][e] = bf16_to_f32(f32_to_bf16(r[g][e]));
-    }
+    F::round_in_place(r[g]);  // the eager step stores bf16 after every token
   }
 }
 
@@ -669,7 +693,7 @@ int bdh_launch_state_step_deferred(bdh_ctx *ctx, bdh_state_log *log, const float
   if (log->rho_dtype == BDH_F32) {
     if (d == 256) BDH_STEP(float, 256, 2); else BDH_STEP(float, 512, 2);
   } else {
-    if (d == 256) BDH_STEP(unsigned short, 256, 4); else BDH_STEP(unsigned short, 512, 2);
+    if (d == 256) BDH_STEP(unsigned short, 256, 8); else BDH_STEP(unsigned short, 512, 4);
   }
 #undef BDH_STEP
   BDH_LAUNCH_CHECK(ctx, "k_step_deferred");

@@ -491,7 +491,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_step_rope_bf16(StepPtrs a, unsig
             const float t0 = qf * vv[j][2 * k], t1 = qf * vv[j][2 * k + 1];
             lo = lo + t0;
             hi = hi + t1;
-            o[k] = (unsigned int)f32_to_bf16(lo) | ((unsigned int)f32_to_bf16(hi) << 16);
+            o[k] = pack_bf16_rne(lo, hi);
           }
           wp[j * 64 + lane] = make_uint4(o[0], o[1], o[2], o[3]);
         }
@@ -1129,7 +1129,7 @@ int bdh_launch_state_steps_in(bdh_ctx *ctx, const StateStepParams &p, float *out
       } else {
         unsigned short *rho = static_cast<unsigned short *>(p.rho);
         if (d == 256 && !split)
-          hipLaunchKernelGGL((k_step_rope_bf16<256, 4, 4, 1>), dim3(blocks), dim3(256), 0, ctx->stream, a, rho);
+          hipLaunchKernelGGL((k_step_rope_bf16<256, 4, 8, 1>), dim3(blocks), dim3(256), 0, ctx->stream, a, rho);
         if (d == 256 && split)
           hipLaunchKernelGGL((k_step_rope_bf16<256, 8, 4, 8>), dim3(blocks), dim3(512), 0, ctx->stream, a, rho);
         if (d == 512 && !split)
