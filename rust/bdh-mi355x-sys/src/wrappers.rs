@@ -112,15 +112,111 @@ pub fn fused_state_aligned<B: HipPointers>(ctx: &Ctx, query: Tensor<B, 4>, value
     out
 }
 
-/// drop-in for BDH::forward_with_state (src/model/bdh.rs:309-450): `rho` holds all layers [L,B,h,Nq,d]
-pub fn forward_with_state<B: HipPointers>(ctx: &Ctx, model: *mut bdh_model, tokens: Tensor<B, 2, Int>,
-    rho: &Tensor<B, 5>, position: &mut usize, vocab: usize) -> Tensor<B, 3> {
-    let [b, t] = tokens.dims();
-    let logits = Tensor::<B, 3>::empty([b, t, vocab], &tokens.device());
-    ctx.check(unsafe {
-        bdh_model_forward(model, B::int_device_ptr(&tokens), b as i32, t as i32, B::device_ptr(rho) as *mut c_void,
-            BDH_F32, *position as i64, B::device_ptr(&logits), std::ptr::null_mut(), std::ptr::null_mut())
-    });
-    *position = position.saturating_add(t); // src/model/bdh.rs:445
-    logits
+/// src/model/state.rs:10-15: one independent state tensor per layer and the shared position
+pub struct ModelState<B: Backend> {
+    pub layers: Vec<LayerState<B>>,
+    pub position: usize,
+}
+
+impl<B: Backend> ModelState<B> {
+    /// src/model/state.rs:27-38
+    pub fn new(num_layers: usize) -> Self {
+        ModelState { layers: (0..num_layers).map(|_| LayerState { rho: None }).collect(), position: 0 }
+    }
+    /// src/model/state.rs:40-45
+    pub fn reset(&mut self) {
+        for layer in self.layers.iter_mut() {
+            layer.rho = None;
+        }
+        self.position = 0;
+    }
+}
+
+/// The model's shapes as BDHConfig gives them (src/model/config.rs:113-164)
+#[derive(Clone, Copy)]
+pub struct ModelDims {
+    pub n_layer: usize,
+    pub n_embd: usize,
+    pub n_head: usize,
+    pub latent: usize,
+    pub vocab: usize,
+    pub rotary: RotaryEmbedding,
+    pub rope_theta: f32,
+    pub relu_threshold: f32,
+}
+
+/// Owns a `bdh_model` (destroyed on drop) together with the parameter tensors it points into and the context it
+/// launches on: the inference half of BDH<B> (src/model/bdh.rs:27-33).
+pub struct Model<B: HipPointers> {
+    raw: *mut bdh_model,
+    ctx: Ctx,
+    dims: ModelDims,
+    // the record order of the reference module; kept alive because the library holds their device pointers
+    _embed: Tensor<B, 2>,
+    _encoder: Tensor<B, 3>,
+    _encoder_v: Tensor<B, 3>,
+    _decoder: Tensor<B, 2>,
+    _lm_head: Tensor<B, 2>,
+}
+
+impl<B: HipPointers> Model<B> {
+    /// BDH::new as far as inference needs it (src/model/bdh.rs:37-84): `embed [V,d]`, `encoder`/`encoder_v [h,d,N]`,
+    /// `decoder [h*N,d]`, `lm_head [d,V]` are the Param values of the reference module (`.val()`, bdh.rs:324-331).
+    pub fn new(device: &B::Device, dims: ModelDims, embed: Tensor<B, 2>, encoder: Tensor<B, 3>,
+        encoder_v: Tensor<B, 3>, decoder: Tensor<B, 2>, lm_head: Tensor<B, 2>, alibi_slopes: Option<&[f32]>) -> Self {
+        let ctx = Ctx::new::<B>(device);
+        let config = bdh_model_config {
+            n_layer: dims.n_layer as i32, n_embd: dims.n_embd as i32, n_head: dims.n_head as i32,
+            latent: dims.latent as i32, vocab: dims.vocab as i32, rotary: dims.rotary as i32,
+            rope_theta: dims.rope_theta, relu_threshold: dims.relu_threshold,
+            alibi_slopes_host: alibi_slopes.map_or(std::ptr::null(), |s| s.as_ptr()),
+        };
+        let weights = bdh_model_weights {
+            embed: B::device_ptr(&embed), encoder: B::device_ptr(&encoder), encoder_v: B::device_ptr(&encoder_v),
+            decoder: B::device_ptr(&decoder), lm_head: B::device_ptr(&lm_head),
+        };
+        let mut raw = std::ptr::null_mut();
+        ctx.check(unsafe { bdh_model_create(ctx.raw, &config, &weights, &mut raw) });
+        Model { raw, ctx, dims, _embed: embed, _encoder: encoder, _encoder_v: encoder_v, _decoder: decoder,
+            _lm_head: lm_head }
+    }
+
+    /// src/model/bdh.rs:254-256
+    pub fn init_state(&self) -> ModelState<B> {
+        ModelState::new(self.dims.n_layer)
+    }
+
+    /// Drop-in for BDH::forward_with_state (src/model/bdh.rs:309-313): the reference's signature.  Every layer's
+    /// state is taken out of its LayerState (zeros on first use or on a shape change, :274-284), handed to the
+    /// library as one pointer per layer (bdh_model_forward_layers: no copy into one allocation) and put back (:304);
+    /// `state.position` advances by T (:445).
+    pub fn forward_with_state(&self, tokens: Tensor<B, 2, Int>, state: &mut ModelState<B>) -> Tensor<B, 3> {
+        assert_eq!(state.layers.len(), self.dims.n_layer, "model state layers mismatch"); // :314-318
+        let [b, t] = tokens.dims();
+        let (h, d, n) = (self.dims.n_head, self.dims.n_embd, self.dims.latent);
+        let nq = if self.dims.rotary == RotaryEmbedding::Pope { 2 * n } else { n };
+        let device = tokens.device();
+        let rhos: Vec<Tensor<B, 4>> = state.layers.iter_mut().map(|layer| match layer.rho.take() {
+            Some(r) if r.dims() == [b, h, nq, d] => r,
+            _ => Tensor::<B, 4>::zeros([b, h, nq, d], &device),
+        }).collect();
+        let ptrs: Vec<*mut c_void> = rhos.iter().map(|r| B::device_ptr(r) as *mut c_void).collect();
+        let logits = Tensor::<B, 3>::empty([b, t, self.dims.vocab], &device);
+        self.ctx.check(unsafe {
+            bdh_model_forward_layers(self.raw, B::int_device_ptr(&tokens), b as i32, t as i32, ptrs.as_ptr(), BDH_F32,
+                std::ptr::null(), state.position as i64, std::ptr::null(), B::device_ptr(&logits),
+                std::ptr::null_mut(), std::ptr::null_mut())
+        });
+        for (layer, rho) in state.layers.iter_mut().zip(rhos) {
+            layer.rho = Some(rho);
+        }
+        state.position = state.position.saturating_add(t); // :445
+        logits
+    }
+}
+
+impl<B: HipPointers> Drop for Model<B> {
+    fn drop(&mut self) {
+        unsafe { bdh_model_destroy(self.raw) };
+    }
 }

@@ -73,3 +73,20 @@ def test_python_binding_lists_every_header_symbol():
 
     c, _ = _c_prototypes()
     assert sorted(n for n, _, _ in c) == sorted(ffi.EXPORTS)
+
+
+def test_wrappers_use_declared_symbols_and_the_reference_signature():
+    """rust/bdh-mi355x-sys/src/wrappers.rs (uncompiled here): every bdh_* function it calls is declared in the
+    extern block, the model is an owner with Drop, and forward_with_state has the signature of
+    src/model/bdh.rs:309-313 over a ModelState of independent per-layer tensors (src/model/state.rs:5-15)."""
+    _, rtext = _rust_prototypes()
+    declared = set(re.findall(r"pub fn (bdh_[a-z0-9_]+)\(", rtext))
+    wtext = open(os.path.join(ROOT, "rust", "bdh-mi355x-sys", "src", "wrappers.rs")).read()
+    called = set(re.findall(r"\b(bdh_[a-z0-9_]+)\(", wtext))
+    assert called and called <= declared, called - declared
+    assert "bdh_model_forward_layers" in called and "bdh_model_destroy" in called
+    assert re.search(r"impl<B: HipPointers> Drop for Model<B>", wtext)
+    sig = re.search(r"pub fn forward_with_state\(&self, tokens: Tensor<B, 2, Int>, state: &mut ModelState<B>\)\s*->\s*Tensor<B, 3>",
+                    wtext)
+    assert sig, "forward_with_state must keep the reference's signature"
+    assert re.search(r"pub struct ModelState<B: Backend> \{\s*pub layers: Vec<LayerState<B>>,\s*pub position: usize,", wtext)
