@@ -231,7 +231,10 @@ def bench_prefill(args):
                    "algorithmic_flop_per_step": flop, "executed_flop_per_step": executed},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "frac_is": "algorithmic (all-scores) FLOP of the workload / time / peak: a utilisation figure "
+                                "for the workload, not matrix-pipe busy time; executed_frac counts what is issued",
                      "executed_tflops": (executed / (ms * 1e-3) / 1e12) if executed else None,
+                     "executed_frac": (executed / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS) if executed else None,
                      "traffic": prefill_traffic_bytes(B, h, N, d, T) if chunked else None,
                      "traffic_source": "buffer sizes of the chunk-recurrent form (x, Q written once and read twice, one "
                                        "bf16 state copy per 256 tokens written and read, rho, out); counters in "
@@ -853,14 +856,17 @@ def main():
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain copy of
             # known size; measured for the default workload only, by the profile named in traffic_source
             "traffic": 216.06e6 if default_workload else None,
-            "traffic_source": "profiles/state_step_config2_f32_pmc_traffic.md" if default_workload else None,
+            "traffic_source": ("profiles/state_step_config2_f32_pmc_traffic.md (a constant copied from that "
+                               "summary, not re-measured by this run)") if default_workload else None,
             "kernel": f"k_step_rope_{args.rho_dtype} (+ k_step_finalize); achieved = algorithmic bytes / ms_per_step "
                       "(both kernels of the step, the slower of the HIP-event and the host clock)",
             "launch_us": ms_per_step * 1e3,
             "event_us": event_us,
             # the dominant kernel alone, from the committed rocprofv3 kernel trace of this command
             "kernel_us": 42.3 if default_workload else None,
-            "kernel_us_source": "profiles/state_step_config2_f32_kernel_trace.md" if default_workload else None,
+            "kernel_us_source": ("profiles/state_step_config2_f32_kernel_trace.md (a constant copied from that "
+                                 "summary; event_us is this run's own clock for both kernels of the step)")
+            if default_workload else None,
             # bdh_probe_chunks in this run: in-place read-modify-write of random 2 KiB chunks (9.75 % of 1 GiB)
             # from ready-made lists: what this access pattern reaches with no arithmetic at all
             "ceiling_measured_gbs": ceiling,
@@ -882,8 +888,11 @@ def main():
                         "5% active, fresh state, 5 timed calls",
             "ms": p_ms, "tokens_per_s": 8 * 2048 / (p_ms * 1e-3),
             "algorithmic_flop": p_flop, "tflops": p_flop / (p_ms * 1e-3) / 1e12,
+            # frac: algorithmic (all-scores) FLOP / time / peak, the utilisation the workload's target is stated in;
+            # executed_frac: the FLOP the chunk-recurrent form actually issues / time / peak
             "frac": p_flop / (p_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
             "executed_flop": p_exec, "executed_tflops": p_exec / (p_ms * 1e-3) / 1e12,
+            "executed_frac": p_exec / (p_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
             # what bounds this form: its HBM traffic (buffer sizes; the counters of the profile read the same within 1 %)
             "hbm_traffic_bytes": prefill_traffic_bytes(8, 4, 8192, 256, 2048),
             "hbm_gbs": prefill_traffic_bytes(8, 4, 8192, 256, 2048) / (p_ms * 1e-3) / 1e9,
