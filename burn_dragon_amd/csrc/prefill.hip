@@ -20,6 +20,8 @@
 // column swizzle on every other group of eight k rows keeps the two half-waves on different banks.
 #include <algorithm>
 #include <atomic>
+#include <cmath>
+#include <cstring>
 #include <type_traits>
 
 #include "bdh_internal.h"
@@ -121,10 +123,97 @@ __global__ __launch_bounds__(256) void k_transpose_to_bf16(const TIn *__restrict
   }
 }
 
+struct HeadPar {
+  float v[64];
+};
+
+// V^T per (b,h) slice for a decaying state (src/model/bdh.rs:299-301): in bf16 [B][R][C] -> out bf16
+// [B*h][C][ldo] with row r (token r of R) scaled by exp((R - r) * log_decay[head]) -- the decay a token's update
+// has seen by the end of the pass.  Columns R..ldo-1 of the output are zero-filled.
+__global__ __launch_bounds__(256) void k_transpose_decay_bf16(const unsigned short *__restrict__ in,
+                                                              unsigned short *__restrict__ out, int R, int C, int ldo,
+                                                              long in_batch, int h, HeadPar log_decay) {
+  __shared__ unsigned short tile[64][66];
+  const long slice = blockIdx.z;
+  const float ld = log_decay.v[slice % h];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const unsigned short *src = in + (slice / h) * in_batch;
+  unsigned short *dst = out + slice * (long)C * ldo;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int rr = ty; rr < 64; rr += 4) {
+    const int r = r0 + rr, c = c0 + tx;
+    unsigned short v = 0;
+    if (r < R && c < C) v = f32_to_bf16_bits(bf16_bits_to_f32(src[(long)r * C + c]) * expf((float)(R - r) * ld));
+    tile[rr][tx] = v;
+  }
+  __syncthreads();
+  for (int cc = ty; cc < 64; cc += 4) {
+    const int c = c0 + cc, r = r0 + tx;
+    if (c < C && r < ldo) dst[(long)c * ldo + r] = tile[tx][cc];
+  }
+}
+
+// PoPE (src/model/attention.rs:323-330): x bf16 [S, T, N] -> q bf16 [S, T, 2N] = cat(softplus(x) cos, softplus(x) sin).
+// thread = (t, group of 8 neurons); loops over the slices
+__global__ __launch_bounds__(256) void k_pope_bf16(const uint4 *__restrict__ x, uint4 *__restrict__ q,
+                                                   const float *__restrict__ freqs, int S, int T, int N,
+                                                   long x_slice_groups, long pos0) {
+  const int groups = N >> 3;
+  const long gid = (long)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= (long)T * groups) return;
+  const int t = (int)(gid / groups), g = (int)(gid - (long)t * groups);
+  const float pos = (float)(pos0 + t);
+  float cs[8], sn[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float raw = pos * freqs[g * 8 + e];
+    sincosf((raw - floorf(raw)) * kTwoPi, &sn[e], &cs[e]);
+  }
+  for (int s = 0; s < S; ++s) {
+    const uint4 in = x[(long)s * x_slice_groups + (long)t * groups + g];
+    const unsigned int w[4] = {in.x, in.y, in.z, in.w};
+    unsigned int re[4], im[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const float m0 = logf(expf(bf16_bits_to_f32((unsigned short)(w[p] & 0xffffu))) + 1.0f);
+      const float m1 = logf(expf(bf16_bits_to_f32((unsigned short)(w[p] >> 16))) + 1.0f);
+      re[p] = (unsigned int)f32_to_bf16_bits(m0 * cs[2 * p]) | ((unsigned int)f32_to_bf16_bits(m1 * cs[2 * p + 1]) << 16);
+      im[p] = (unsigned int)f32_to_bf16_bits(m0 * sn[2 * p]) | ((unsigned int)f32_to_bf16_bits(m1 * sn[2 * p + 1]) << 16);
+    }
+    uint4 *row = q + ((long)s * T + t) * (2 * groups);
+    row[g] = make_uint4(re[0], re[1], re[2], re[3]);
+    row[groups + g] = make_uint4(im[0], im[1], im[2], im[3]);
+  }
+}
+
+// denom[slice][row] = sum over the column tiles of norm_part + eps (src/kernel/linear_attention.rs:8,108), in tile
+// order; tri: only the tiles up to the row's own exist
+__global__ __launch_bounds__(256) void k_norm_reduce(const float *__restrict__ norm_part, float *__restrict__ denom,
+                                                     int M, int nt, int tri, float eps) {
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  const long slice = blockIdx.y;
+  if (row >= M) return;
+  const int last = tri ? row / BM : nt - 1;
+  float sum = 0.0f;
+  for (int tj = 0; tj <= last; ++tj) sum += norm_part[(slice * nt + tj) * M + row];
+  denom[slice * M + row] = sum + eps;
+}
+
 // ------------------------------------------------------------------------------------
 // batched GEMM  C[m,n] (+)= sum_k A[m,k] B[n,k]
 // ------------------------------------------------------------------------------------
-enum { EPI_SCORES = 0, EPI_ACC = 1 };
+// EPI_SCORES / EPI_ACC: the two epilogues of the RoPE path.  The _X variants add what ALiBi, the row
+// normalisation of kernel::linear_attention::fused_state_aligned and a decaying state need (GemmArgs::mode).
+enum { EPI_SCORES = 0, EPI_ACC = 1, EPI_SCORES_X = 2, EPI_ACC_X = 3 };
+enum {
+  GM_DECAY_SCORES = 1,  // scores:  S[t,s] *= exp((t - s) * par)            (src/model/bdh.rs:299-301 unrolled)
+  GM_ADD_ALIBI = 2,     // scores:  S[t,s] += par * (s - t) on every element of the causal time blocks
+                        //          (src/kernel/linear_attention.rs:97-100: whole blocks, the diagonal one included)
+  GM_ROWNORM = 4,       // scores:  also write sum_s |S[t,s]| of this tile's columns to norm_part
+  GM_DECAY_ROWS = 8,    // acc:     row t *= exp(t * par)                   (the Q rho0 term of a decaying state)
+  GM_DECAY_STATE = 16,  // acc:     C = exp(K * par) * C + acc              (the state after K decaying tokens)
+  GM_DIVNORM = 32       // acc:     C = acc / denom[row]                    (src/kernel/linear_attention.rs:108-109)
+};
 
 struct GemmArgs {
   const void *A;  // bf16
@@ -139,7 +228,80 @@ struct GemmArgs {
   int tri;             // 1: tiles enumerate the lower triangle (row tile >= col tile) of an mt x mt grid
   int mt, nt;          // tile grid (rows, cols); rows are visited from the last (largest causal K) down
   int n_tiles, n_slices;
+  // _X epilogues only
+  int mode;            // GM_* bits
+  int h;               // heads: slice % h selects head_par
+  int block_size;      // GM_ADD_ALIBI: tokens per time block of the causal layout
+  float *norm_part;    // GM_ROWNORM: [slice][nt][M] sums of |S| per column tile
+  const float *denom;  // GM_DIVNORM: [slice][M]
+  float head_par[64];  // per head: log of the per-token decay factor, or the additive slope
 };
+
+// Epilogues of the _X variants.  Accumulator element e of lane l in a 32x32 tile: row = (e/4)*8 + (l/32)*4 +
+// (e%4), col = l%32.  s_red: 1024 floats of LDS that no wave reads any more (GM_ROWNORM only).
+template <int EPI>
+__device__ __forceinline__ void gemm_epilogue_x(const GemmArgs &g, f32x16 (&acc)[4][2], int slice, int m0, int n0,
+                                                int tj, int wm, int wn, int lane, int tid, float *s_red) {
+  const float par = g.head_par[slice % g.h];
+  if constexpr (EPI == EPI_SCORES_X) {
+    unsigned short *C = static_cast<unsigned short *>(g.C) + (long)slice * g.c_batch;
+    const int bs = g.block_size > 0 ? g.block_size : 1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        const int rblk = (g.mode & GM_ADD_ALIBI) ? row / bs : 0;
+        float rsum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+          float v = col < row ? acc[i][j][e] : 0.0f;  // tril(-1)
+          if ((g.mode & GM_DECAY_SCORES) && col < row) v *= expf((float)(row - col) * par);
+          if ((g.mode & GM_ADD_ALIBI) && col / bs <= rblk) v += par * (float)(col - row);
+          if (col >= g.N) v = 0.0f;  // padding columns of the score matrix
+          const unsigned short bits = f32_to_bf16_bits(v);
+          if (row < g.M && col < g.ldc) C[(long)row * g.ldc + col] = bits;
+          rsum += fabsf(bf16_bits_to_f32(bits));  // what the next product multiplies with
+        }
+        if (g.mode & GM_ROWNORM) {
+#pragma unroll
+          for (int off = 16; off >= 1; off >>= 1) rsum += __shfl_xor(rsum, off);  // the 32 columns of a half-wave
+          if ((lane & 31) == 0) s_red[wn * 256 + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3)] = rsum;
+        }
+      }
+    if (g.mode & GM_ROWNORM) {
+      __syncthreads();
+      if (tid < 256 && m0 + tid < g.M) {
+        const float sum = ((s_red[tid] + s_red[256 + tid]) + s_red[512 + tid]) + s_red[768 + tid];
+        g.norm_part[((long)slice * g.nt + tj) * g.M + m0 + tid] = sum;
+      }
+    }
+  } else {
+    float *C = static_cast<float *>(g.C) + (long)slice * g.c_batch;
+    const float sdecay = (g.mode & GM_DECAY_STATE) ? expf((float)g.K * par) : 1.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * 128 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row >= g.M) continue;
+        const float rscale = (g.mode & GM_DECAY_ROWS) ? expf((float)row * par) : 1.0f;
+        const float dn = (g.mode & GM_DIVNORM) ? g.denom[(long)slice * g.M + row] : 1.0f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+          if (col >= g.N) continue;
+          float v = acc[i][j][e];
+          if (g.mode & GM_DECAY_ROWS) v *= rscale;
+          if (g.mode & GM_DIVNORM) v = v / dn;
+          float *p = C + (long)row * g.ldc + col;
+          if (g.beta) v = ((g.mode & GM_DECAY_STATE) ? *p * sdecay : *p) + v;
+          *p = v;
+        }
+      }
+  }
+}
 
 // bf16 elements per k row of a k-major tile in LDS: 576 bytes = 64 mod 256, so the four k rows of 64 bytes
 // that 32 lanes of a transposing read touch fall on disjoint quarters of the 64 banks
@@ -280,6 +442,11 @@ __global__ __launch_bounds__(512) void k_gemm(GemmArgs g) {
     }
   }
 
+  if constexpr (EPI == EPI_SCORES_X || EPI == EPI_ACC_X) {
+    __syncthreads();  // every wave is past its fragment reads: s_a can hold the row sums
+    gemm_epilogue_x<EPI>(g, acc, slice, m0, n0, tj, wm, wn, lane, tid, reinterpret_cast<float *>(s_a));
+    return;
+  }
   // epilogue.  Accumulator element e of lane l in a 32x32 tile:
   //   row = (e/4)*8 + (l/32)*4 + (e%4), col = l%32
 #pragma unroll
@@ -366,7 +533,8 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
     pb[c] = Bh + (long)(n0 + bi * 8 + lr) * g.ldb + lc * 8;
   }
   // scores: A and B are the same matrix, so a tile on the diagonal needs its rows only once
-  const bool same_ab = EPI == EPI_SCORES && g.tri && ti == tj && g.A == g.B && g.b_div == 1;
+  const bool same_ab = (EPI == EPI_SCORES || EPI == EPI_SCORES_X) && ti == tj && g.A == g.B && g.b_div == 1 &&
+                       g.a_batch == g.b_batch;
 #define BDH_ISSUE_TILE(buf, k0)                                                                              \
   _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                            \
     const int bi = c * 8 + wave;                                                                             \
@@ -406,6 +574,10 @@ __global__ __launch_bounds__(512) void k_gemm_direct(GemmArgs g) {
     cur ^= 1;
   }
 #undef BDH_ISSUE_TILE
+  if constexpr (EPI == EPI_SCORES_X || EPI == EPI_ACC_X) {  // the loop ended with a barrier: s_dyn is free
+    gemm_epilogue_x<EPI>(g, acc, slice, m0, n0, tj, wm, wn, lane, tid, reinterpret_cast<float *>(s_dyn));
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -1052,7 +1224,7 @@ template <bool AK, int EPI>
 hipError_t launch_gemm(hipStream_t st, const GemmArgs &g) {
   const int groups = (g.n_slices + 7) / 8;
   const bool full = !AK && g.M % BM == 0 && g.N % BN == 0 && g.K % BK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 &&
-                    (EPI != EPI_SCORES || g.ldc == g.N);
+                    ((EPI != EPI_SCORES && EPI != EPI_SCORES_X) || g.ldc == g.N);
   if constexpr (!AK) {
     if (full) {
       constexpr int lds = 4 * 256 * 64 * 2;  // two buffers of two 32 KiB tiles
@@ -1076,92 +1248,163 @@ hipError_t launch_gemm(hipStream_t st, const GemmArgs &g) {
   return hipSuccess;
 }
 
-// One pass of the all-scores form (any T, N, d that are multiples of 8): tokens [0, T) of the pointers given,
-// x / out slices x_slice / out_slice elements apart.
+// What a pass of the all-scores form does beyond the RoPE recurrence.
+struct PassMode {
+  int rotary = BDH_ROPE;
+  bool decay = false;       // ALiBi, recurrent semantics: rho <- (rho + q (x) v) * exp(-slope) per token
+  bool row_norm = false;    // the stateless, row-normalised form of kernel::linear_attention::fused_state_aligned
+  bool add_alibi = false;   // row_norm only: + slope * (s - t) on the causal time blocks
+  int block_size = 1;       // row_norm + add_alibi: tokens per time block
+  float head_par[64] = {};  // per head: log of the decay factor (decay) or the slope (add_alibi)
+  bool extended() const { return rotary != BDH_ROPE || decay || row_norm; }
+};
+
+// One pass of the all-scores form (any T; N and d multiples of 8): tokens [0, T) of the pointers given,
+// x / out slices x_slice / out_slice elements apart.  rho [S, Nq, d], Nq = 2N for PoPE.
 static int prefill_pass_scores(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16, long x_slice,
                                const uint16_t *v_bf16, long v_batch, const float *freqs, int64_t position,
-                               int state_is_zero, float *rho, float *out, long out_slice) {
+                               int state_is_zero, float *rho, float *out, long out_slice,
+                               const PassMode &pm = PassMode()) {
   const int S = B * h;
+  const int Nq = pm.rotary == BDH_POPE ? 2 * N : N;
+  const bool ext = pm.extended();
+  const bool stateless = pm.row_norm;
   const int Tp = (T + 7) / 8 * 8;  // leading dimension of the score matrix
   const int mt = (T + BM - 1) / BM;  // row/col tiles of the score matrix
-  const int nt_rho = (N + BM - 1) / BM, nt_d = (d + BN - 1) / BN;
-  const int n_score_tiles = mt * (mt + 1) / 2;
+  const int nt_rho = (Nq + BM - 1) / BM, nt_d = (d + BN - 1) / BN;
+  // a time block that straddles two score tiles has additive terms above the tile diagonal: all tiles then
+  const bool full_grid = pm.row_norm && pm.add_alibi && (BM % pm.block_size) != 0;
+  const int n_score_tiles = full_grid ? mt * mt : mt * (mt + 1) / 2;
   const int n_out_tiles = mt * nt_d, n_rho_tiles = nt_rho * nt_d;
+  const bool own_q = pm.rotary != BDH_ALIBI;  // ALiBi does not rotate: the products read x itself
 
-  // workspace: Q bf16 [S,T,N] | scores bf16 [S,T,Tp] | V^T bf16 [B,d,Tp] | rho0^T bf16 [S,d,N]
-  const size_t q_bytes = bdh_align_up((size_t)S * T * N * 2, 256);
+  // workspace: Q bf16 [S,T,Nq] | scores bf16 [S,T,Tp] | V^T bf16 [B or S,d,Tp] | rho0^T bf16 [S,d,Nq] |
+  //            norm partials f32 [S,mt,T] | denominators f32 [S,T]
+  const size_t q_bytes = own_q ? bdh_align_up((size_t)S * T * Nq * 2, 256) : 0;
   const size_t s_bytes = bdh_align_up((size_t)S * T * Tp * 2, 256);
-  const size_t vt_bytes = bdh_align_up((size_t)B * d * Tp * 2, 256);
-  const size_t rt_bytes = state_is_zero ? 0 : bdh_align_up((size_t)S * d * N * 2, 256);
-  int rc = bdh_ws_reserve(ctx, q_bytes + s_bytes + vt_bytes + rt_bytes);
+  const size_t vt_bytes = bdh_align_up((size_t)(pm.decay ? S : B) * d * Tp * 2, 256);
+  const size_t vs_bytes = pm.decay ? bdh_align_up((size_t)B * d * Tp * 2, 256) : 0;  // undecayed V^T for S V
+  const size_t rt_bytes = (state_is_zero || stateless) ? 0 : bdh_align_up((size_t)S * d * Nq * 2, 256);
+  const size_t np_bytes = pm.row_norm ? bdh_align_up((size_t)S * mt * T * 4, 256) : 0;
+  const size_t dn_bytes = pm.row_norm ? bdh_align_up((size_t)S * T * 4, 256) : 0;
+  int rc = bdh_ws_reserve(ctx, q_bytes + s_bytes + vt_bytes + vs_bytes + rt_bytes + np_bytes + dn_bytes);
   if (rc != BDH_OK) return rc;
   char *ws = static_cast<char *>(ctx->ws);
-  unsigned short *Q = reinterpret_cast<unsigned short *>(ws);
-  unsigned short *Sc = reinterpret_cast<unsigned short *>(ws + q_bytes);
-  unsigned short *Vt = reinterpret_cast<unsigned short *>(ws + q_bytes + s_bytes);
-  unsigned short *Rt = reinterpret_cast<unsigned short *>(ws + q_bytes + s_bytes + vt_bytes);
+  size_t off = 0;
+  auto take = [&](size_t bytes) { char *p = ws + off; off += bytes; return p; };
+  unsigned short *Qw = reinterpret_cast<unsigned short *>(take(q_bytes));
+  unsigned short *Sc = reinterpret_cast<unsigned short *>(take(s_bytes));
+  unsigned short *Vt = reinterpret_cast<unsigned short *>(take(vt_bytes));   // decayed per slice when pm.decay
+  unsigned short *Vs = pm.decay ? reinterpret_cast<unsigned short *>(take(vs_bytes)) : Vt;  // plain, per batch entry
+  unsigned short *Rt = reinterpret_cast<unsigned short *>(take(rt_bytes));
+  float *norm_part = reinterpret_cast<float *>(take(np_bytes));
+  float *denom = reinterpret_cast<float *>(take(dn_bytes));
+  const unsigned short *Q = own_q ? Qw : reinterpret_cast<const unsigned short *>(x_bf16);
+  const long q_slice = own_q ? (long)T * Nq : x_slice;
   if ((long)S * n_score_tiles > 0x7fffffffL / 16 || (long)S * n_rho_tiles > 0x7fffffffL / 16)
     return bdh_fail(ctx, BDH_E_SHAPE, "too many tiles (T=%d N=%d)", T, N);
+  auto with_mode = [&](GemmArgs &g, int mode) {
+    g.mode = mode; g.h = h; g.block_size = pm.block_size; g.norm_part = norm_part; g.denom = denom;
+    memcpy(g.head_par, pm.head_par, sizeof(g.head_par));
+  };
 
   // 0. V^T (and rho0^T): make every B operand k-contiguous
   hipLaunchKernelGGL(k_transpose_to_bf16<unsigned short>, dim3((d + 63) / 64, (Tp + 63) / 64, B), dim3(256), 0,
-                     ctx->stream, v_bf16, Vt, T, d, Tp, v_batch);
+                     ctx->stream, v_bf16, Vs, T, d, Tp, v_batch);
   BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<V>");
-  if (!state_is_zero) {
-    hipLaunchKernelGGL(k_transpose_to_bf16<float>, dim3((d + 63) / 64, (N + 63) / 64, S), dim3(256), 0, ctx->stream,
-                       rho, Rt, N, d, N, (long)N * d);
+  if (pm.decay) {
+    HeadPar hp;
+    memcpy(hp.v, pm.head_par, sizeof(hp.v));
+    hipLaunchKernelGGL(k_transpose_decay_bf16, dim3((d + 63) / 64, (Tp + 63) / 64, S), dim3(256), 0, ctx->stream,
+                       v_bf16, Vt, T, d, Tp, v_batch, h, hp);
+    BDH_LAUNCH_CHECK(ctx, "k_transpose_decay_bf16");
+  }
+  if (!state_is_zero && !stateless) {
+    hipLaunchKernelGGL(k_transpose_to_bf16<float>, dim3((d + 63) / 64, (Nq + 63) / 64, S), dim3(256), 0, ctx->stream,
+                       rho, Rt, Nq, d, Nq, (long)Nq * d);
     BDH_LAUNCH_CHECK(ctx, "k_transpose_to_bf16<rho0>");
   }
   // 1. rotation
-  {
+  if (own_q) {
     const long work = (long)T * (N / 8);
-    hipLaunchKernelGGL(k_rope_bf16, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, ctx->stream,
-                       reinterpret_cast<const uint4 *>(x_bf16), reinterpret_cast<uint4 *>(Q), freqs, S, T, N,
-                       x_slice / 8, (long)position);
-    BDH_LAUNCH_CHECK(ctx, "k_rope_bf16");
+    if (pm.rotary == BDH_POPE)
+      hipLaunchKernelGGL(k_pope_bf16, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, ctx->stream,
+                         reinterpret_cast<const uint4 *>(x_bf16), reinterpret_cast<uint4 *>(Qw), freqs, S, T, N,
+                         x_slice / 8, (long)position);
+    else
+      hipLaunchKernelGGL(k_rope_bf16, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, ctx->stream,
+                         reinterpret_cast<const uint4 *>(x_bf16), reinterpret_cast<uint4 *>(Qw), freqs, S, T, N,
+                         x_slice / 8, (long)position);
+    BDH_LAUNCH_CHECK(ctx, "k_rope_bf16 / k_pope_bf16");
   }
   // 2. scores = tril(-1)(Q Q^T), lower tiles only
   {
     GemmArgs g{};
     g.A = Q; g.B = Q; g.C = Sc;
-    g.a_batch = (long)T * N; g.b_batch = (long)T * N; g.c_batch = (long)T * Tp;
-    g.lda = N; g.ldb = N; g.ldc = Tp;
-    g.M = T; g.N = T; g.K = N; g.b_div = 1; g.beta = 0; g.causal_k = 0;
-    g.tri = 1; g.mt = mt; g.nt = mt; g.n_tiles = n_score_tiles; g.n_slices = S;
-    BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_SCORES>(ctx->stream, g)));
+    g.a_batch = q_slice; g.b_batch = q_slice; g.c_batch = (long)T * Tp;
+    g.lda = Nq; g.ldb = Nq; g.ldc = Tp;
+    g.M = T; g.N = T; g.K = Nq; g.b_div = 1; g.beta = 0; g.causal_k = 0;
+    g.tri = full_grid ? 0 : 1; g.mt = mt; g.nt = mt; g.n_tiles = n_score_tiles; g.n_slices = S;
+    if (ext) {
+      with_mode(g, (pm.decay ? GM_DECAY_SCORES : 0) | (pm.add_alibi ? GM_ADD_ALIBI : 0) | (pm.row_norm ? GM_ROWNORM : 0));
+      BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_SCORES_X>(ctx->stream, g)));
+    } else {
+      BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_SCORES>(ctx->stream, g)));
+    }
     BDH_LAUNCH_CHECK(ctx, "k_gemm<scores>");
   }
-  // 3a. out = Q rho0 (skipped for a fresh state)
-  if (!state_is_zero) {
+  if (pm.row_norm) {
+    hipLaunchKernelGGL(k_norm_reduce, dim3((T + 255) / 256, S), dim3(256), 0, ctx->stream, norm_part, denom, T, mt,
+                       full_grid ? 0 : 1, 1e-6f);
+    BDH_LAUNCH_CHECK(ctx, "k_norm_reduce");
+  }
+  // 3a. out = Q rho0 (skipped for a fresh state; a decaying state has lost exp(-slope)^t by row t)
+  if (!state_is_zero && !stateless) {
     GemmArgs g{};
     g.A = Q; g.B = Rt; g.C = out;
-    g.a_batch = (long)T * N; g.b_batch = (long)d * N; g.c_batch = out_slice;
-    g.lda = N; g.ldb = N; g.ldc = d;
-    g.M = T; g.N = d; g.K = N; g.b_div = 1; g.beta = 0; g.causal_k = 0;
+    g.a_batch = q_slice; g.b_batch = (long)d * Nq; g.c_batch = out_slice;
+    g.lda = Nq; g.ldb = Nq; g.ldc = d;
+    g.M = T; g.N = d; g.K = Nq; g.b_div = 1; g.beta = 0; g.causal_k = 0;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
-    BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC>(ctx->stream, g)));
+    if (pm.decay) {
+      with_mode(g, GM_DECAY_ROWS);
+      BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC_X>(ctx->stream, g)));
+    } else {
+      BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC>(ctx->stream, g)));
+    }
     BDH_LAUNCH_CHECK(ctx, "k_gemm<Q rho0>");
   }
-  // 3b. out (+)= scores V
+  // 3b. out (+)= scores V   (row-normalised form: divided by the row's sum of |scores| + eps)
   {
     GemmArgs g{};
-    g.A = Sc; g.B = Vt; g.C = out;
+    g.A = Sc; g.B = Vs; g.C = out;
     g.a_batch = (long)T * Tp; g.b_batch = (long)d * Tp; g.c_batch = out_slice;
     g.lda = Tp; g.ldb = Tp; g.ldc = d;
-    g.M = T; g.N = d; g.K = T; g.b_div = h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 1;
+    g.M = T; g.N = d; g.K = T; g.b_div = h; g.beta = (state_is_zero || stateless) ? 0 : 1;
+    g.causal_k = full_grid ? 0 : 1;
     g.tri = 0; g.mt = mt; g.nt = nt_d; g.n_tiles = n_out_tiles; g.n_slices = S;
-    BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC>(ctx->stream, g)));
+    if (pm.row_norm) {
+      with_mode(g, GM_DIVNORM);
+      BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC_X>(ctx->stream, g)));
+    } else {
+      BDH_HIP_CHECK(ctx, (launch_gemm<false, EPI_ACC>(ctx->stream, g)));
+    }
     BDH_LAUNCH_CHECK(ctx, "k_gemm<S V>");
   }
-  // 4. rho (+)= Q^T V   (A = Q read k-major)
-  {
+  // 4. rho (+)= Q^T V   (A = Q read k-major; a decaying state: rho = g^T rho + sum_s g^(T-s) q_s (x) v_s)
+  if (!stateless) {
     GemmArgs g{};
     g.A = Q; g.B = Vt; g.C = rho;
-    g.a_batch = (long)T * N; g.b_batch = (long)d * Tp; g.c_batch = (long)N * d;
-    g.lda = N; g.ldb = Tp; g.ldc = d;
-    g.M = N; g.N = d; g.K = T; g.b_div = h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 0;
+    g.a_batch = q_slice; g.b_batch = (long)d * Tp; g.c_batch = (long)Nq * d;
+    g.lda = Nq; g.ldb = Tp; g.ldc = d;
+    g.M = Nq; g.N = d; g.K = T; g.b_div = pm.decay ? 1 : h; g.beta = state_is_zero ? 0 : 1; g.causal_k = 0;
     g.tri = 0; g.mt = nt_rho; g.nt = nt_d; g.n_tiles = n_rho_tiles; g.n_slices = S;
-    BDH_HIP_CHECK(ctx, (launch_gemm<true, EPI_ACC>(ctx->stream, g)));
+    if (pm.decay) {
+      with_mode(g, GM_DECAY_STATE);
+      BDH_HIP_CHECK(ctx, (launch_gemm<true, EPI_ACC_X>(ctx->stream, g)));
+    } else {
+      BDH_HIP_CHECK(ctx, (launch_gemm<true, EPI_ACC>(ctx->stream, g)));
+    }
     BDH_LAUNCH_CHECK(ctx, "k_gemm<Q^T V>");
   }
   return BDH_OK;
@@ -1242,28 +1485,36 @@ static int prefill_pass_chunks(bdh_ctx *ctx, int B, int h, int Tc, int N, const 
 
 }  // namespace
 
-extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
-                                   const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk,
-                                   int flags, float *rho, float *out) {
-  if (!ctx) return BDH_E_INVAL;
+// Shared body of the two entry points.  pm: what goes beyond the RoPE recurrence (all-scores form only).
+static int prefill_chunked_impl(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
+                                const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk, int flags,
+                                float *rho, float *out, const PassMode &pm) {
   if (B < 0 || h < 0 || T < 0 || N < 0 || d < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative dimension");
   if (position < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative position");
   if (chunk < 0) return bdh_fail(ctx, BDH_E_INVAL, "negative chunk length");
-  if (flags & ~(BDH_PREFILL_STATE_IS_ZERO | BDH_PREFILL_STATE_HILO | BDH_PREFILL_ALL_SCORES))
-    return bdh_fail(ctx, BDH_E_INVAL, "unknown flag bits 0x%x", flags);
   if (B == 0 || h == 0 || T == 0) return BDH_OK;
-  if ((N & 7) || (d & 7) || N == 0 || d == 0)
-    return bdh_fail(ctx, BDH_E_SHAPE, "chunked prefill needs N and d to be positive multiples of 8 (N=%d d=%d)", N, d);
-  if (!x_bf16 || !v_bf16 || !freqs || !rho || !out) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
-  if (!bdh_aligned(x_bf16, 16) || !bdh_aligned(v_bf16, 16) || !bdh_aligned(rho, 16) || !bdh_aligned(out, 16))
+  // RoPE keeps the contract of bdh_prefill_chunked (N and d multiples of 8); the other forms only read x in
+  // 16-byte pieces
+  if ((N & 7) || N == 0 || d == 0 || (!pm.extended() && (d & 7)))
+    return bdh_fail(ctx, BDH_E_SHAPE, "chunked prefill needs N%s to be positive multiples of 8 (N=%d d=%d)",
+                    pm.extended() ? "" : " and d", N, d);
+  const bool stateless = pm.row_norm;
+  if (!x_bf16 || !v_bf16 || !out || (!stateless && !rho) || (pm.rotary != BDH_ALIBI && !freqs))
+    return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  if (!bdh_aligned(x_bf16, 16) || !bdh_aligned(v_bf16, 16) || (rho && !bdh_aligned(rho, 16)) || !bdh_aligned(out, 16))
     return bdh_fail(ctx, BDH_E_ALIGN, "x, v, rho and out need 16-byte alignment");
   if (B > 65535 || B * h > 65535) return bdh_fail(ctx, BDH_E_SHAPE, "batch too large for the transpose grid");
   // tokens per pass: the workspace holds the rotated activations (and, in the all-scores form, the score
   // matrix) of one pass only; the state is carried from pass to pass in the caller's f32 rho
   const int pass_default = 2048;
   int pass = chunk > 0 ? chunk : pass_default;
-  const bool aligned = !(flags & BDH_PREFILL_ALL_SCORES) && d == 256 && N % 256 == 0;
-  int zero = (flags & BDH_PREFILL_STATE_IS_ZERO) ? 1 : 0;
+  if (stateless) {  // the normaliser needs whole score rows: one pass
+    if ((double)B * h * T * T * 2.0 > 64.0 * 1024 * 1024 * 1024)
+      return bdh_fail(ctx, BDH_E_SHAPE, "row-normalised form: the score matrix of B*h=%d, T=%d exceeds 64 GiB", B * h, T);
+    pass = T;
+  }
+  const bool aligned = !pm.extended() && !(flags & BDH_PREFILL_ALL_SCORES) && d == 256 && N % 256 == 0;
+  int zero = ((flags & BDH_PREFILL_STATE_IS_ZERO) || stateless) ? 1 : 0;
   const int hilo = (flags & BDH_PREFILL_STATE_HILO) ? 1 : 0;
   for (int t0 = 0; t0 < T;) {
     int Tc = std::min(pass, T - t0);
@@ -1277,11 +1528,53 @@ extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int
                                op, (long)T * d);
     } else {
       rc = prefill_pass_scores(ctx, B, h, Tc, N, d, xp, (long)T * N, vp, (long)T * d, freqs, position + t0, zero, rho,
-                               op, (long)T * d);
+                               op, (long)T * d, pm);
     }
     if (rc != BDH_OK) return rc;
     zero = 0;
     t0 += Tc;
   }
   return BDH_OK;
+}
+
+extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
+                                   const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk,
+                                   int flags, float *rho, float *out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (flags & ~(BDH_PREFILL_STATE_IS_ZERO | BDH_PREFILL_STATE_HILO | BDH_PREFILL_ALL_SCORES))
+    return bdh_fail(ctx, BDH_E_INVAL, "unknown flag bits 0x%x", flags);
+  return prefill_chunked_impl(ctx, B, h, T, N, d, x_bf16, v_bf16, freqs, position, chunk, flags, rho, out, PassMode());
+}
+
+extern "C" int bdh_prefill_chunked_ex(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary,
+                                      const uint16_t *x_bf16, const uint16_t *v_bf16, const float *freqs,
+                                      const float *alibi_slopes_host, int64_t position, int chunk, int flags,
+                                      int block_size, float *rho, float *out) {
+  if (!ctx) return BDH_E_INVAL;
+  if (flags & ~(BDH_PREFILL_STATE_IS_ZERO | BDH_PREFILL_STATE_HILO | BDH_PREFILL_ALL_SCORES | BDH_PREFILL_ROW_NORMALIZE))
+    return bdh_fail(ctx, BDH_E_INVAL, "unknown flag bits 0x%x", flags);
+  if (rotary != BDH_ROPE && rotary != BDH_ALIBI && rotary != BDH_POPE)
+    return bdh_fail(ctx, BDH_E_INVAL, "unknown rotary mode %d", rotary);
+  PassMode pm;
+  pm.rotary = rotary;
+  pm.row_norm = (flags & BDH_PREFILL_ROW_NORMALIZE) != 0;
+  pm.block_size = block_size > 0 ? block_size : 1;
+  float slopes[64];
+  if (pm.row_norm) {
+    // kernel::linear_attention::fused_state_aligned: the additive term exists when slopes are given (:44-51)
+    pm.add_alibi = alibi_slopes_host != nullptr;
+    if (pm.add_alibi) {
+      if (h > 64) return bdh_fail(ctx, BDH_E_SHAPE, "at most 64 heads with ALiBi slopes (h=%d)", h);
+      memcpy(pm.head_par, alibi_slopes_host, sizeof(float) * h);
+    }
+  } else if (rotary == BDH_ALIBI) {
+    // BDH::recurrent_attention: the state decays by exp(-slope) after every token (src/model/bdh.rs:299-301)
+    if (h > 64) return bdh_fail(ctx, BDH_E_SHAPE, "at most 64 heads with ALiBi slopes (h=%d)", h);
+    if (alibi_slopes_host) memcpy(slopes, alibi_slopes_host, sizeof(float) * h);
+    else bdh_default_alibi_slopes(h, slopes);
+    pm.decay = true;
+    // log of the ROUNDED per-token factor (src/model/attention.rs:181-186), as the lazily decayed step uses it
+    for (int i = 0; i < h; ++i) pm.head_par[i] = (float)log((double)expf(-slopes[i]));
+  }
+  return prefill_chunked_impl(ctx, B, h, T, N, d, x_bf16, v_bf16, freqs, position, chunk, flags, rho, out, pm);
 }

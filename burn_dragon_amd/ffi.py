@@ -18,14 +18,14 @@ LIB_PATH = os.path.join(PKG, "libbdh_mi355x.so")
 OK, E_INVAL, E_SHAPE, E_ALIGN, E_HIP, E_NOMEM, E_UNSUPPORTED = 0, -1, -2, -3, -4, -5, -6
 ROPE, ALIBI, POPE = 0, 1, 2
 F32, BF16 = 0, 1
-PREFILL_STATE_IS_ZERO, PREFILL_STATE_HILO, PREFILL_ALL_SCORES = 1, 2, 4
+PREFILL_STATE_IS_ZERO, PREFILL_STATE_HILO, PREFILL_ALL_SCORES, PREFILL_ROW_NORMALIZE = 1, 2, 4, 8
 
 # every symbol include/bdh_mi355x.h declares
 EXPORTS = [
     "bdh_version", "bdh_status_string", "bdh_ctx_create", "bdh_ctx_destroy", "bdh_ctx_set_stream",
     "bdh_ctx_synchronize", "bdh_last_error", "bdh_ctx_set_option", "bdh_build_freqs", "bdh_default_alibi_slopes",
     "bdh_recurrent_attention", "bdh_state_step", "bdh_relu_lowrank", "bdh_layer_norm",
-    "bdh_fused_state_aligned", "bdh_prefill_chunked", "bdh_model_create", "bdh_model_destroy",
+    "bdh_fused_state_aligned", "bdh_prefill_chunked", "bdh_prefill_chunked_ex", "bdh_model_create", "bdh_model_destroy",
     "bdh_model_state_bytes", "bdh_model_forward", "bdh_model_forward_ex", "bdh_advance_positions",
     "bdh_sample_top_k", "bdh_recurrent_attention_lazy_alibi", "bdh_alibi_materialize", "bdh_model_forward_lazy",
     "bdh_rho_energy", "bdh_model_forward_viz", "bdh_rotate",
@@ -111,6 +111,8 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_fused_state_aligned.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, P, c_int, P, c_int, c_int,
                                             c_int, P]
     lib.bdh_prefill_chunked.argtypes = [P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int64, c_int, c_int, P, P]
+    lib.bdh_prefill_chunked_ex.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, P, c_int64, c_int,
+                                           c_int, c_int, P, P]
     lib.bdh_model_create.argtypes = [P, POINTER(ModelConfigC), POINTER(ModelWeightsC), POINTER(P)]
     lib.bdh_model_destroy.argtypes = [P]
     lib.bdh_model_state_bytes.restype = c_size_t

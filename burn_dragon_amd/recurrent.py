@@ -143,6 +143,37 @@ def prefill_chunked(x_bf16: torch.Tensor, v_bf16: torch.Tensor, rho: torch.Tenso
     return out
 
 
+def prefill_chunked_ex(x_bf16: torch.Tensor, v_bf16: torch.Tensor, rho: Optional[torch.Tensor], freqs: torch.Tensor,
+                       position: int, rotary: RotaryEmbedding = RotaryEmbedding.ROPE,
+                       alibi_slopes=None, row_normalize: bool = False,
+                       block_size: int = 1, state_is_zero: bool = False, chunk: int = 0, hilo: bool = False,
+                       all_scores: bool = False, ctx: Optional[ffi.Context] = None) -> torch.Tensor:
+    """prefill_chunked for all three positional schemes (PoPE: rho [B,h,2N,d]; ALiBi: the state decays by
+    exp(-slope) per token, src/model/bdh.rs:299-301), and with row_normalize the bf16 matrix-core form of
+    kernel::linear_attention::fused_state_aligned (src/kernel/linear_attention.rs:11-115, dense causal layout with
+    time blocks of block_size; stateless: rho is not used and may be None; the additive ALiBi term whenever
+    alibi_slopes is given).  Returns out [B,h,T,d] float32."""
+    ctx = ctx or ffi.default_context(x_bf16.device.index or 0)
+    B, h, T, N = x_bf16.shape
+    d = v_bf16.shape[-1]
+    rotary = RotaryEmbedding(rotary)
+    nq = 2 * N if rotary == RotaryEmbedding.POPE else N
+    assert x_bf16.dtype == torch.bfloat16 and x_bf16.is_contiguous()
+    v_bf16 = v_bf16.reshape(B, T, d)
+    assert v_bf16.dtype == torch.bfloat16 and v_bf16.is_contiguous()
+    if rho is not None:
+        assert rho.dtype == torch.float32 and rho.is_contiguous() and tuple(rho.shape) == (B, h, nq, d)
+    out = torch.empty((B, h, T, d), device=x_bf16.device, dtype=torch.float32)
+    freqs_ptr = ffi.ptr(freqs.reshape(-1)) if freqs is not None else None
+    slopes = None if alibi_slopes is None else np.ascontiguousarray(alibi_slopes, np.float32)
+    flags = ((ffi.PREFILL_STATE_IS_ZERO if state_is_zero else 0) | (ffi.PREFILL_STATE_HILO if hilo else 0) |
+             (ffi.PREFILL_ALL_SCORES if all_scores else 0) | (ffi.PREFILL_ROW_NORMALIZE if row_normalize else 0))
+    ctx.check(ctx.lib.bdh_prefill_chunked_ex(ctx.handle, B, h, T, N, d, int(rotary), ffi.ptr(x_bf16), ffi.ptr(v_bf16),
+                                             freqs_ptr, ffi.ptr(slopes), int(position), int(chunk), flags, int(block_size),
+                                             ffi.ptr(rho) if rho is not None else None, ffi.ptr(out)))
+    return out
+
+
 class StateLog:
     """The pending rank-1 updates of ONE state tensor rho [B,h,N,d] (bdh_state_log): the deferred decode step
     reads its active state rows and logs its update; `flush` (called by the step itself when `capacity` steps are

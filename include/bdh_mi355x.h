@@ -310,13 +310,46 @@ int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N, int dv,
  *                 BDH_PREFILL_ALL_SCORES: always the all-scores form (every causal 256x256 score tile of
  *                 the pass, no state copies).
  *   rho [B,h,N,d] f32 in/out,  out [B,h,T,d] f32
- * N and d must be multiples of 8.  There is no row-normalised variant: the normaliser of
- * kernel::linear_attention::fused_state_aligned needs whole score rows (bdh_fused_state_aligned).
+ * N and d must be multiples of 8.  ALiBi, PoPE and the row-normalised form: bdh_prefill_chunked_ex below.
  */
-enum bdh_prefill_flags { BDH_PREFILL_STATE_IS_ZERO = 1, BDH_PREFILL_STATE_HILO = 2, BDH_PREFILL_ALL_SCORES = 4 };
+enum bdh_prefill_flags {
+  BDH_PREFILL_STATE_IS_ZERO = 1,
+  BDH_PREFILL_STATE_HILO = 2,
+  BDH_PREFILL_ALL_SCORES = 4,
+  BDH_PREFILL_ROW_NORMALIZE = 8 /* bdh_prefill_chunked_ex only */
+};
 int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
                         const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk,
                         int flags, float *rho, float *out);
+
+/*
+ * bdh_prefill_chunked for all three positional schemes, and the bf16 matrix-core form of the row-normalised
+ * attention.  Same arguments, plus:
+ *   rotary             BDH_ROPE: exactly bdh_prefill_chunked.
+ *                      BDH_POPE: Q = bf16(cat(softplus(x) cos, softplus(x) sin)) (src/model/attention.rs:323-330),
+ *                      rho [B,h,2N,d].
+ *                      BDH_ALIBI: Q = x, and the state decays by g_h = exp(-slope_h) after every token
+ *                      (src/model/bdh.rs:299-301):  out_t = g^t q_t rho0 + sum_{s<t} g^(t-s) (q_t . q_s) v_s,
+ *                      rho = g^T rho0 + sum_s g^(T-s) q_s (x) v_s, the powers as exp(k * log(g_f32)) like the lazily
+ *                      decayed step.  alibi_slopes_host: host float[h], NULL = the default slopes.  rho is an
+ *                      eagerly decayed f32 state (bdh_alibi_materialize first for a lazily decayed one).
+ *                      PoPE and ALiBi take the all-scores form (every causal 256x256 score tile of a pass).
+ *   flags              | BDH_PREFILL_ROW_NORMALIZE: the stateless function of
+ *                      kernel::linear_attention::fused_state_aligned (src/kernel/linear_attention.rs:11-115) with the
+ *                      dense causal layout, as bdh_fused_state_aligned computes it in f32:
+ *                        out = (S' V) / (sum_s |S'[t,s]| + 1e-6),  S' = tril(-1)(Q Q^T) [+ slope_h (s - t)]
+ *                      rho is neither read nor written (may be NULL), the whole call is one pass (chunk is ignored;
+ *                      the bf16 score matrix [B*h,T,T] lives in the workspace), positions start at `position`
+ *                      (the reference: 0).  The additive term is applied when alibi_slopes_host is given, whatever
+ *                      the rotary mode, on every element of the causal time blocks of block_size tokens -- the
+ *                      diagonal block included, where it reaches the elements above the diagonal (:97-100).
+ *                      The normaliser sums the bf16-rounded scores, the values the product multiplies with.
+ *   block_size         tokens per time block (BDH_PREFILL_ROW_NORMALIZE with slopes only; <= 0 means 1).
+ * Tolerance class of the bf16 forms: 2e-2 of the output scale.  At most 64 heads when slopes are in use.
+ */
+int bdh_prefill_chunked_ex(bdh_ctx *ctx, int B, int h, int T, int N, int d, int rotary, const uint16_t *x_bf16,
+                           const uint16_t *v_bf16, const float *freqs, const float *alibi_slopes_host,
+                           int64_t position, int chunk, int flags, int block_size, float *rho, float *out);
 
 /* ---- a1: the whole cached step ------------------------------------------------------- */
 /* src/model/config.rs:113-164 (BDHConfig) + :10-31 (FusedKernelConfig), as plain scalars */

@@ -58,6 +58,7 @@ pub const BDH_BF16: c_int = 1;
 pub const BDH_PREFILL_STATE_IS_ZERO: c_int = 1;
 pub const BDH_PREFILL_STATE_HILO: c_int = 2;
 pub const BDH_PREFILL_ALL_SCORES: c_int = 4;
+pub const BDH_PREFILL_ROW_NORMALIZE: c_int = 8;
 
 /// src/model/config.rs:113-164 (BDHConfig) + :10-31 (FusedKernelConfig), as plain scalars
 #[repr(C)]
@@ -129,6 +130,9 @@ extern "C" {
     pub fn bdh_prefill_chunked(ctx: *mut bdh_ctx, b: c_int, h: c_int, t: c_int, n: c_int, d: c_int,
         x_bf16: *const u16, v_bf16: *const u16, freqs: *const f32, position: i64, chunk: c_int, flags: c_int,
         rho: *mut f32, out: *mut f32) -> c_int;
+    pub fn bdh_prefill_chunked_ex(ctx: *mut bdh_ctx, b: c_int, h: c_int, t: c_int, n: c_int, d: c_int, rotary: c_int,
+        x_bf16: *const u16, v_bf16: *const u16, freqs: *const f32, alibi_slopes_host: *const f32, position: i64,
+        chunk: c_int, flags: c_int, block_size: c_int, rho: *mut f32, out: *mut f32) -> c_int;
     pub fn bdh_model_create(ctx: *mut bdh_ctx, config: *const bdh_model_config,
         weights: *const bdh_model_weights, out: *mut *mut bdh_model) -> c_int;
     pub fn bdh_model_destroy(model: *mut bdh_model) -> c_int;

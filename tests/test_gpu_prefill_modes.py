@@ -1,0 +1,195 @@
+"""GPU parity of bdh_prefill_chunked_ex: the bf16 matrix-core prefill for PoPE and ALiBi (recurrent semantics,
+src/model/bdh.rs:288-302) and the row-normalised form of kernel::linear_attention::fused_state_aligned
+(src/kernel/linear_attention.rs:11-115), through the C ABI, against the CPU oracle on the bf16-rounded inputs.
+Tolerance class of the bf16 forms: 2e-2 of the output's max-norm (Q, the scores and the state copy that enters a
+product are rounded to bf16 once; accumulation is f32)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bdh_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def bda():
+    if not torch.cuda.is_available():
+        pytest.fail("no HIP device: the GPU tests must run on the MI355X box")
+    import burn_dragon_amd
+
+    return burn_dragon_amd
+
+
+def rel_err(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+def _case(seed, B, h, T, N, d, nq, rho0_scale, relu=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((B, h, T, N), generator=g)
+    if relu:
+        x = torch.relu(x - 0.5)
+    x = x.to(torch.bfloat16)
+    v = torch.randn((B, T, d), generator=g).to(torch.bfloat16)
+    rho0 = (rho0_scale * torch.randn((B, h, nq, d), generator=g)).float()
+    return x, v, rho0
+
+
+ROT = {"rope": orc.ROPE, "alibi": orc.ALIBI, "pope": orc.POPE}
+
+
+@pytest.mark.parametrize("rotary", ["pope", "alibi"])
+@pytest.mark.parametrize("T,N,d,rho0_scale,position,chunk", [
+    (70, 24, 40, 0.05, 5, 0),        # ragged against every tile
+    (300, 264, 72, 0.0, 0, 0),       # fresh state, two score tiles
+    (512, 256, 256, 0.05, 33, 0),    # full tiles: operands straight from global memory into LDS
+    (600, 128, 64, 0.05, 9, 256),    # three passes: the state (and its decay) carried between them
+])
+def test_recurrent_prefill_pope_and_alibi(bda, corc, rotary, T, N, d, rho0_scale, position, chunk):
+    """Oracle = the sequential loop of src/model/bdh.rs:288-302 (PoPE rotation of attention.rs:323-330; ALiBi decay of
+    :299-301 with the reference's default slopes)."""
+    from burn_dragon_amd.recurrent import prefill_chunked_ex
+
+    B, h = 2, 3
+    rot = ROT[rotary]
+    nq = 2 * N if rotary == "pope" else N
+    x, v, rho0 = _case(T + N, B, h, T, N, d, nq, rho0_scale)
+    freqs = corc.build_freqs(N, rotary=rot)
+    slopes = corc.default_alibi_slopes(h) if rotary == "alibi" else None
+    q = corc.rotate(x.float().numpy(), freqs, rot, position)
+    decay = None if slopes is None else corc.alibi_decay(slopes)
+    out_ref, rho_ref = corc.recurrent_attention(q, v.float().numpy(), rho0.numpy(), decay=decay)
+    rho = rho0.clone().to(DEV)
+    out = prefill_chunked_ex(x.to(DEV), v.to(DEV), rho, torch.from_numpy(freqs).to(DEV), position,
+                             rotary=bda.RotaryEmbedding.parse(rotary), alibi_slopes=slopes,
+                             state_is_zero=(rho0_scale == 0.0), chunk=chunk)
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), out_ref) < TOL
+    assert rel_err(rho.cpu().numpy(), rho_ref) < TOL
+    if rho0_scale == 0.0:
+        assert not out[:, :, 0].any()  # token 0 reads only the initial state
+
+
+def test_alibi_prefill_custom_slopes_then_decode_steps(bda, corc):
+    """Caller-given slopes; and the state the call leaves continues under the eager ALiBi decode step
+    (bdh_recurrent_attention) like the oracle's token loop over prompt + steps."""
+    from burn_dragon_amd.recurrent import prefill_chunked_ex, recurrent_attention
+
+    B, h, T, N, d, steps = 2, 4, 200, 64, 48, 6
+    x, v, rho0 = _case(11, B, h, T + steps, N, d, N, 0.0)
+    slopes = np.array([0.9, 0.3, 0.05, 0.0], np.float32)
+    zeros = np.zeros(N, np.float32)
+    out_ref, rho_ref = corc.recurrent_attention(x.float().numpy(), v.float().numpy(), rho0.numpy(),
+                                                decay=corc.alibi_decay(slopes))
+    rho = rho0.clone().to(DEV)
+    out_p = prefill_chunked_ex(x[:, :, :T].contiguous().to(DEV), v[:, :T].contiguous().to(DEV), rho, None, 0,
+                               rotary=bda.RotaryEmbedding.ALIBI, alibi_slopes=slopes, state_is_zero=True)
+    out_d = recurrent_attention(x[:, :, T:].float().contiguous().to(DEV), v[:, T:].float().contiguous().to(DEV), rho,
+                                torch.from_numpy(zeros).to(DEV), T, bda.RotaryEmbedding.ALIBI, alibi_slopes=slopes)
+    torch.cuda.synchronize()
+    assert rel_err(out_p.cpu().numpy(), out_ref[:, :, :T]) < TOL
+    assert rel_err(out_d.cpu().numpy(), out_ref[:, :, T:]) < TOL
+    assert rel_err(rho.cpu().numpy(), rho_ref) < TOL
+
+
+def test_rope_through_the_extended_entry_point_is_the_plain_call(bda, corc):
+    """rotary = RoPE without row normalisation is bdh_prefill_chunked, bit for bit (chunk-recurrent form included)."""
+    from burn_dragon_amd.recurrent import prefill_chunked, prefill_chunked_ex
+
+    B, h, T, N, d = 2, 2, 520, 256, 256
+    x, v, rho0 = _case(3, B, h, T, N, d, N, 0.05)
+    ft = torch.from_numpy(corc.build_freqs(N)).to(DEV)
+    rho_a, rho_b = rho0.clone().to(DEV), rho0.clone().to(DEV)
+    out_a = prefill_chunked(x.to(DEV), v.to(DEV), rho_a, ft, 7)
+    out_b = prefill_chunked_ex(x.to(DEV), v.to(DEV), rho_b, ft, 7, rotary=bda.RotaryEmbedding.ROPE)
+    torch.cuda.synchronize()
+    assert torch.equal(out_a, out_b) and torch.equal(rho_a, rho_b)
+
+
+@pytest.mark.parametrize("rotary,seed", [("rope", 1337), ("pope", 2024)])
+def test_row_normalised_reference_recipes(bda, corc, rotary, seed):
+    """tests/fused_kernel_tests.rs:70-170 on the bf16 path: B=1, h=2, T=6, N=8, dv=6, BlockPattern2d::dense(3);
+    fused == dense tril(-1) + row-normalise.  The reference compares f32 paths at 1e-4; this path rounds Q and the
+    scores to bf16: 2e-2."""
+    from burn_dragon_amd.recurrent import prefill_chunked_ex
+
+    rot = ROT[rotary]
+    g = torch.Generator().manual_seed(seed)
+    query = torch.randn((1, 2, 6, 8), generator=g).to(torch.bfloat16)
+    value = torch.randn((1, 6, 6), generator=g).to(torch.bfloat16)
+    freqs = corc.build_freqs(8, rotary=rot)
+    got = prefill_chunked_ex(query.to(DEV), value.to(DEV), None, torch.from_numpy(freqs).to(DEV), 0,
+                             rotary=bda.RotaryEmbedding.parse(rotary), row_normalize=True, block_size=3)
+    torch.cuda.synchronize()
+    q = orc.rotate(query.double().numpy(), freqs.astype(np.float64), rot, 0)
+    scores = np.tril(q @ np.swapaxes(q, 2, 3), -1)
+    scores = scores / (np.abs(scores).sum(3, keepdims=True) + 1e-6)
+    reference = scores @ value.double().numpy()[:, None]
+    assert rel_err(got.cpu().numpy(), reference) < TOL
+    ref_c = corc.fused_state_aligned(query.float().numpy(), value.float().numpy(), freqs, None, 3, rot)
+    assert rel_err(got.cpu().numpy(), ref_c) < TOL
+
+
+@pytest.mark.parametrize("rotary", ["rope", "alibi", "pope"])
+@pytest.mark.parametrize("T,N,dv,bs", [(300, 200, 70, 48),    # time blocks straddle the 256-wide score tiles
+                                       (520, 64, 40, 64),     # time blocks aligned with them
+                                       (512, 256, 256, 128)]) # full tiles
+def test_row_normalised_medium_shapes(bda, corc, rotary, T, N, dv, bs):
+    """Against the oracle's blocked form (src/kernel/linear_attention.rs:54-112): ALiBi adds slope * (s - t) to whole
+    time blocks, the diagonal one included."""
+    from burn_dragon_amd.recurrent import prefill_chunked_ex
+
+    B, h = 2, 3
+    rot = ROT[rotary]
+    x, v, _ = _case(T + bs, B, h, T, N, dv, N, 0.0)
+    slopes = corc.default_alibi_slopes(h) if rotary == "alibi" else None
+    freqs = corc.build_freqs(N, rotary=rot)
+    got = prefill_chunked_ex(x.to(DEV), v.to(DEV), None, torch.from_numpy(freqs).to(DEV), 0,
+                             rotary=bda.RotaryEmbedding.parse(rotary), alibi_slopes=slopes, row_normalize=True,
+                             block_size=bs)
+    torch.cuda.synchronize()
+    ref = corc.fused_state_aligned(x.float().numpy(), v.float().numpy(), freqs, slopes, bs, rot)
+    assert rel_err(got.cpu().numpy(), ref) < TOL
+
+
+def test_row_normalised_matches_the_f32_entry_point_at_a_long_sequence(bda, corc):
+    """T = 1100 with 16 slices, ragged against the tiles and the time block of 100: the bf16 form against
+    bdh_fused_state_aligned (f32 on the same bf16-rounded inputs), RoPE and ALiBi."""
+    from burn_dragon_amd.kernel import linear_attention
+    from burn_dragon_amd.recurrent import prefill_chunked_ex
+
+    B, h, T, N, dv, bs = 4, 4, 1100, 64, 40, 100
+    x, v, _ = _case(9, B, h, T, N, dv, N, 0.0)
+    for rotary, rot in (("rope", orc.ROPE), ("alibi", orc.ALIBI)):
+        slopes = corc.default_alibi_slopes(h) if rotary == "alibi" else None
+        freqs = torch.from_numpy(corc.build_freqs(N, rotary=rot))
+        want = linear_attention.fused_state_aligned(x.float().to(DEV), v.float()[:, None].to(DEV), freqs,
+                                                    None if slopes is None else torch.from_numpy(slopes),
+                                                    bda.BlockPattern2d.dense(bs), bda.RotaryEmbedding.parse(rotary))
+        got = prefill_chunked_ex(x.to(DEV), v.to(DEV), None, freqs.to(DEV), 0, rotary=bda.RotaryEmbedding.parse(rotary),
+                                 alibi_slopes=slopes, row_normalize=True, block_size=bs)
+        torch.cuda.synchronize()
+        assert rel_err(got.cpu().numpy(), want.cpu().numpy()) < TOL
+
+
+def test_extended_prefill_contract_errors(bda):
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.recurrent import prefill_chunked_ex
+
+    x = torch.zeros((1, 2, 8, 16), dtype=torch.bfloat16, device=DEV)
+    v = torch.zeros((1, 8, 8), dtype=torch.bfloat16, device=DEV)
+    ft = torch.zeros(16, device=DEV)
+    ctx = ffi.default_context(0)
+    out = torch.empty((1, 2, 8, 8), device=DEV)
+    call = lambda rotary, flags, rho, h=2: ctx.lib.bdh_prefill_chunked_ex(
+        ctx.handle, 1, h, 8, 16, 8, rotary, ffi.ptr(x), ffi.ptr(v), ffi.ptr(ft), None, 0, 0, flags, 1, rho, ffi.ptr(out))
+    assert call(7, 0, None) == -1                       # unknown rotary mode
+    assert call(0, 16, None) == -1                      # unknown flag bit
+    assert call(1, 0, None) == -1                       # a recurrent call needs rho
+    assert call(1, ffi.PREFILL_ROW_NORMALIZE, None) == 0  # the row-normalised form does not
+    with pytest.raises(AssertionError):                 # PoPE state has 2N rows
+        prefill_chunked_ex(x, v, torch.zeros((1, 2, 16, 8), device=DEV), ft, 0, rotary=bda.RotaryEmbedding.POPE)
