@@ -32,6 +32,24 @@ int bdh_ws_reserve(bdh_ctx *ctx, size_t bytes) {
   return BDH_OK;
 }
 
+int bdh_stage_reserve(bdh_ctx *ctx, size_t bytes) {
+  if (bytes <= ctx->stage_bytes) return BDH_OK;
+  bytes = bdh_align_up(bytes, size_t(1) << 20);
+  if (ctx->stage) {
+    BDH_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    BDH_HIP_CHECK(ctx, hipFree(ctx->stage));
+    ctx->stage = nullptr;
+    ctx->stage_bytes = 0;
+  }
+  hipError_t e = hipMalloc(&ctx->stage, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return bdh_fail(ctx, BDH_E_NOMEM, "staging buffer of %zu bytes: %s", bytes, hipGetErrorString(e));
+  }
+  ctx->stage_bytes = bytes;
+  return BDH_OK;
+}
+
 extern "C" {
 
 const char *bdh_version(void) { return "bdh_mi355x 0.1.0 (gfx950)"; }
@@ -83,7 +101,8 @@ int bdh_ctx_create(int device_id, void *hip_stream, bdh_ctx **out) {
 
 int bdh_ctx_destroy(bdh_ctx *ctx) {
   if (!ctx) return BDH_OK;
-  if (ctx->ws || ctx->fsa_mask || ctx->lat_mask) (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->ws || ctx->fsa_mask || ctx->lat_mask || ctx->stage) (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->stage) (void)hipFree(ctx->stage);
   if (ctx->ws) (void)hipFree(ctx->ws);
   if (ctx->fsa_mask) (void)hipFree(ctx->fsa_mask);
   if (ctx->lat_mask) (void)hipFree(ctx->lat_mask);
@@ -168,6 +187,11 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
   if (strcmp(name, "fused_state_aligned.path") == 0) {
     if (value < -1 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "fused_state_aligned.path takes -1, 0 or 1");
     ctx->opt_fsa_path = value;
+    return BDH_OK;
+  }
+  if (strcmp(name, "state_step.prompt_bf16") == 0) {
+    if (value < 0) return bdh_fail(ctx, BDH_E_INVAL, "state_step.prompt_bf16 takes 0 (never) or a token count");
+    ctx->opt_step_prompt_bf16 = value;
     return BDH_OK;
   }
   return bdh_fail(ctx, BDH_E_INVAL, "unknown option '%s'", name);

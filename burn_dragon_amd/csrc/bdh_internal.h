@@ -17,6 +17,9 @@ struct bdh_ctx {
   // growable device workspace (partials, counters); owned by the context
   void *ws = nullptr;
   size_t ws_bytes = 0;
+  // a second growable buffer for inputs a launcher converts before it calls a path that sizes ctx->ws itself
+  void *stage = nullptr;
+  size_t stage_bytes = 0;
   int n_cu = 0;
   int opt_step_split = -1;  // -1 choose by grid size, 0 / 1 force the 256- / 64-pair workgroup
   int opt_step_dense = -1;  // many-token state step as dense f32 products: -1 from T = 128, 0 never, 1 always
@@ -31,6 +34,7 @@ struct bdh_ctx {
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on
   int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
+  int opt_step_prompt_bf16 = 0;  // many-token state step on the bf16 matrix cores from this many tokens on (0: never)
   // time-block mask of the last sparse fused_state_aligned pattern (device) and the pattern it was built from
   void *fsa_mask = nullptr;
   size_t fsa_mask_bytes = 0;
@@ -73,6 +77,8 @@ int bdh_launch_model_small(bdh_model *m, const int64_t *tokens, int B, void *rho
 
 // Grows ctx->ws to at least `bytes` (synchronises the stream before freeing the old one).
 int bdh_ws_reserve(bdh_ctx *ctx, size_t bytes);
+// The same for ctx->stage.
+int bdh_stage_reserve(bdh_ctx *ctx, size_t bytes);
 
 #define BDH_HIP_CHECK(ctx, call)                                                        \
   do {                                                                                  \
@@ -123,6 +129,9 @@ size_t bdh_step_scratch_bytes();
 // The same T steps as four dense products per chunk on the f32 matrix cores (attention_parallel.hip):
 // RoPE / PoPE, f32 state, no bitmask or row counts.
 int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
+// prefill.hip: the same T steps on the bf16 matrix cores (x, v and the scores rounded to bf16, f32 accumulation and
+// f32 state; tolerance class 2e-2): any rotary, a lazily decayed state is brought up to date first; host position only.
+int bdh_launch_state_prefill_bf16(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
 // rho <- the up-to-date state, stamps <- clock, for a lazily decayed ALiBi state
 int bdh_launch_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, const float *slopes_host, int64_t clock,
                                  const int32_t *clocks_dev, void *rho, int rho_dtype, int32_t *stamps);

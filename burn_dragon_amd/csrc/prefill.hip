@@ -1537,6 +1537,70 @@ static int prefill_chunked_impl(bdh_ctx *ctx, int B, int h, int T, int N, int d,
   return BDH_OK;
 }
 
+namespace {
+
+// in f32 [n] -> out bf16 [n], rounded to nearest even
+__global__ __launch_bounds__(256) void k_f32_to_bf16(const float *__restrict__ in, unsigned short *__restrict__ out, size_t n) {
+  const size_t n4 = n / 4;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
+    const float4 v = reinterpret_cast<const float4 *>(in)[i];
+    uint2 o;
+    o.x = (unsigned int)f32_to_bf16_bits(v.x) | ((unsigned int)f32_to_bf16_bits(v.y) << 16);
+    o.y = (unsigned int)f32_to_bf16_bits(v.z) | ((unsigned int)f32_to_bf16_bits(v.w) << 16);
+    reinterpret_cast<uint2 *>(out)[i] = o;
+  }
+  if (blockIdx.x == 0 && threadIdx.x < n - n4 * 4) out[n4 * 4 + threadIdx.x] = f32_to_bf16_bits(in[n4 * 4 + threadIdx.x]);
+}
+
+__global__ __launch_bounds__(256) void k_fill_i32(int32_t *__restrict__ p, long n, int32_t v) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+}  // namespace
+
+int bdh_launch_state_prefill_bf16(bdh_ctx *ctx, const StateStepParams &p, float *out_ln) {
+  const int B = p.B, h = p.h, T = p.T, N = p.N, d = p.d;
+  if (p.rho_dtype != BDH_F32 || p.positions_dev || p.bitmask || p.rows_touched)
+    return bdh_fail(ctx, BDH_E_UNSUPPORTED, "the bf16 prompt form takes an f32 state, a host position and no by-products");
+  if (p.stamps && p.rotary != BDH_ALIBI) return bdh_fail(ctx, BDH_E_INVAL, "decay stamps only apply to ALiBi");
+  if (p.stamps && p.position + T > 0x7fffffffLL) return bdh_fail(ctx, BDH_E_INVAL, "position beyond the stamp range");
+  PassMode pm;
+  pm.rotary = p.rotary;
+  if (p.rotary == BDH_ALIBI) {
+    if (h > 64) return bdh_fail(ctx, BDH_E_SHAPE, "at most 64 heads with ALiBi slopes (h=%d)", h);
+    pm.decay = true;
+    for (int i = 0; i < h; ++i) pm.head_par[i] = (float)log((double)expf(-p.slopes_host[i]));
+  }
+  if (p.stamps) {  // a lazily decayed state: apply what is pending, the products decay every row themselves
+    const int rc0 = bdh_launch_alibi_materialize(ctx, B, h, N, d, p.slopes_host, p.position, nullptr, p.rho, p.rho_dtype,
+                                                 p.stamps);
+    if (rc0 != BDH_OK) return rc0;
+  }
+  const size_t nx = (size_t)B * h * T * N, nv = (size_t)B * T * d;
+  const size_t x_bytes = bdh_align_up(nx * 2, 256);
+  int rc = bdh_stage_reserve(ctx, x_bytes + bdh_align_up(nv * 2, 256));
+  if (rc != BDH_OK) return rc;
+  unsigned short *xb = static_cast<unsigned short *>(ctx->stage);
+  unsigned short *vb = reinterpret_cast<unsigned short *>(static_cast<char *>(ctx->stage) + x_bytes);
+  hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)std::min<size_t>((nx / 4 + 255) / 256 + 1, 1u << 16)), dim3(256), 0,
+                     ctx->stream, p.x, xb, nx);
+  BDH_LAUNCH_CHECK(ctx, "k_f32_to_bf16<x>");
+  hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)std::min<size_t>((nv / 4 + 255) / 256 + 1, 1u << 16)), dim3(256), 0,
+                     ctx->stream, p.v, vb, nv);
+  BDH_LAUNCH_CHECK(ctx, "k_f32_to_bf16<v>");
+  rc = prefill_chunked_impl(ctx, B, h, T, N, d, xb, vb, p.freqs, p.position, 0, 0, static_cast<float *>(p.rho), p.out, pm);
+  if (rc != BDH_OK) return rc;
+  if (p.stamps) {  // every row is now up to date as of the end of the call
+    const long rows = (long)B * h * N;
+    hipLaunchKernelGGL(k_fill_i32, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, ctx->stream, p.stamps, rows,
+                       (int32_t)(p.position + T));
+    BDH_LAUNCH_CHECK(ctx, "k_fill_i32");
+  }
+  if (out_ln) return bdh_launch_layer_norm_rows(ctx, (int64_t)B * h * T, d, p.out, out_ln);
+  return BDH_OK;
+}
+
 extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
                                    const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk,
                                    int flags, float *rho, float *out) {

@@ -1031,6 +1031,12 @@ int bdh_launch_state_steps_in(bdh_ctx *ctx, const StateStepParams &p, float *out
     }
     return BDH_OK;
   }
+  // opt-in ("state_step.prompt_bf16" = T0): calls of T0+ tokens on an f32 state, positions given by the host and no
+  // per-token by-products run on the bf16 matrix cores (inputs and scores rounded to bf16: tolerance class 2e-2)
+  if (!fixed && !p.bitmask && !p.rows_touched && ctx->opt_step_prompt_bf16 > 0 && T >= ctx->opt_step_prompt_bf16 &&
+      p.rho_dtype == BDH_F32 && !p.positions_dev && N % 8 == 0 && (p.rotary != BDH_ROPE || d % 8 == 0) &&
+      (p.rotary != BDH_ALIBI || h <= 64))
+    return bdh_launch_state_prefill_bf16(ctx, p, out_ln);
   // many tokens, no per-token by-products: the dense form on the f32 matrix cores (a bf16 state is widened for the call)
   // (not when even a 128-token chunk of rotated activations would pass 16 GiB of workspace)
   const bool chunk_fits = sizeof(float) * (size_t)slices * Nq * 128 <= (size_t(16) << 30) &&

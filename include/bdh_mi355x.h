@@ -80,6 +80,13 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       from 8 tokens on for an f32 state that every token streams in full -- PoPE,
  *                       eager ALiBi -- or that is at most 64 MiB),
  *                       0 = always token by token, 1 = dense products for any T.
+ *   "state_step.prompt_bf16": 0 (default) never; T0 > 0: a call of T0 or more tokens on an f32 state, with the
+ *                       position given by the host and no bitmask / row-count outputs, runs as
+ *                       bdh_prefill_chunked_ex does: on the bf16 matrix cores, activations, values and scores
+ *                       rounded to bf16, f32 accumulation and f32 state (any rotary; a lazily decayed ALiBi state
+ *                       is brought up to date first and stamped with the end of the call).  Tolerance class
+ *                       2e-2 instead of 1e-3, which is why it is opt-in; applies to bdh_recurrent_attention and
+ *                       to the prompt calls of bdh_model_forward*.
  *   "state_step.dense_kernel": 1 (default) PoPE and eagerly decayed ALiBi steps at d in {256,512} take
  *                       the dense streaming kernel, 0 = the generic kernel (same values).
  *   "relu_lowrank.mfma_rows": 8 (default) calls with this many rows and at most 64 (N a multiple of 4, d a

@@ -193,3 +193,83 @@ def test_extended_prefill_contract_errors(bda):
     assert call(1, ffi.PREFILL_ROW_NORMALIZE, None) == 0  # the row-normalised form does not
     with pytest.raises(AssertionError):                 # PoPE state has 2N rows
         prefill_chunked_ex(x, v, torch.zeros((1, 2, 16, 8), device=DEV), ft, 0, rotary=bda.RotaryEmbedding.POPE)
+
+
+# ------------------------------------------------- the option that routes prompt calls to the bf16 form
+@pytest.fixture
+def prompt_bf16(bda):
+    from burn_dragon_amd import ffi
+
+    ctx = ffi.default_context(0)
+    ctx.set_option("state_step.prompt_bf16", 64)
+    yield ctx
+    ctx.set_option("state_step.prompt_bf16", 0)
+
+
+@pytest.mark.parametrize("rotary", ["rope", "alibi", "pope"])
+def test_recurrent_attention_takes_the_bf16_form_when_asked(bda, corc, prompt_bf16, rotary):
+    """bdh_recurrent_attention with "state_step.prompt_bf16": f32 inputs, rounded to bf16 inside; against the oracle's
+    token loop on the f32 inputs at the bf16 tolerance, and different from the default f32 path (so the option took)."""
+    from burn_dragon_amd.recurrent import recurrent_attention
+
+    B, h, T, N, d = 2, 3, 200, 128, 72
+    rot = ROT[rotary]
+    nq = 2 * N if rotary == "pope" else N
+    g = torch.Generator().manual_seed(21)
+    x = torch.relu(torch.randn((B, h, T, N), generator=g) - 0.5)
+    v = torch.randn((B, T, d), generator=g)
+    rho0 = 0.05 * torch.randn((B, h, nq, d), generator=g)
+    freqs = corc.build_freqs(N, rotary=rot)
+    slopes = corc.default_alibi_slopes(h) if rotary == "alibi" else None
+    decay = None if slopes is None else corc.alibi_decay(slopes)
+    out_ref, rho_ref = corc.recurrent_attention(corc.rotate(x.numpy(), freqs, rot, 40), v.numpy(), rho0.numpy(),
+                                                decay=decay)
+    ft = torch.from_numpy(freqs).to(DEV)
+    rho = rho0.clone().to(DEV)
+    out = recurrent_attention(x.to(DEV), v.to(DEV), rho, ft, 40, bda.RotaryEmbedding.parse(rotary), alibi_slopes=slopes)
+    prompt_bf16.set_option("state_step.prompt_bf16", 0)
+    rho32 = rho0.clone().to(DEV)
+    out32 = recurrent_attention(x.to(DEV), v.to(DEV), rho32, ft, 40, bda.RotaryEmbedding.parse(rotary),
+                                alibi_slopes=slopes)
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), out_ref) < TOL and rel_err(rho.cpu().numpy(), rho_ref) < TOL
+    assert rel_err(out32.cpu().numpy(), out_ref) < 1e-3
+    assert not torch.equal(out, out32)
+
+
+@pytest.mark.parametrize("lazy", [False, True], ids=["eager-decay", "lazy-decay"])
+def test_trained_checkpoint_prompt_on_the_bf16_form(bda, corc, prompt_bf16, lazy):
+    """The reference's trained ALiBi checkpoint (tests/golden/tiny_shakespeare): a 160-character prompt through
+    forward_with_state with the state path of every layer on the bf16 matrix cores, then greedy decode steps on the
+    state it left.  Logits against the oracle at the bf16 tolerance; the model still predicts the text."""
+    import os
+
+    from burn_dragon_amd import record
+
+    ckpt = os.path.join(os.path.dirname(__file__), "golden", "tiny_shakespeare")
+    text = ("First Citizen:\nBefore we proceed any further, hear me speak.\n\nAll:\nSpeak, speak.\n\n"
+            "First Citizen:\nYou are all resolved rather to die than to famish?\n\nAll:\nResolved. resolved.\n")
+    model, tok, _ = bda.BDH.from_checkpoint_dir(ckpt, DEV, alibi_lazy=lazy)
+    _, weights, _, _ = record.load_checkpoint_dir(ckpt)
+    shape = orc.BDHShape(n_layer=4, n_embd=128, n_head=4, mlp_internal_dim_multiplier=4, vocab_size=69, rotary=orc.ALIBI)
+    w = orc.BDHWeights(**weights)
+    ids = np.array([tok.encode(text)])
+    n_prompt = 160
+    assert ids.shape[1] > n_prompt + 4
+    state = model.init_state()
+    logits = model.forward_with_state(torch.from_numpy(ids[:, :n_prompt]), state).cpu().numpy()
+    rho_ref = np.zeros((4, 1, 4, 128, 128), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, ids[:, :n_prompt], rho_ref, 0, sparse_state=False)
+    assert rel_err(logits, logits_ref) < TOL
+    z = logits[0].astype(np.float64)
+    logp = z - z.max(-1, keepdims=True)
+    logp -= np.log(np.exp(logp).sum(-1, keepdims=True))
+    loss = float(-logp[np.arange(n_prompt - 1), ids[0, 1:n_prompt]].mean())
+    assert loss < 1.4, loss  # uniform would be ln 69 = 4.23
+    # decode steps (single tokens: the f32 step kernels) continue from the state the bf16 prompt left
+    for t in range(n_prompt, n_prompt + 4):
+        step = model.forward_with_state(torch.from_numpy(ids[:, t:t + 1]), state).cpu().numpy()
+        step_ref, pos, _, _ = corc.forward_with_state(shape, w, ids[:, t:t + 1], rho_ref, pos, sparse_state=False)
+        assert rel_err(step, step_ref) < TOL
+    model.materialize_state(state)
+    assert rel_err(state.storage.cpu().numpy(), rho_ref) < TOL and state.position == pos
