@@ -110,16 +110,19 @@ def cpu_baseline_model(cfg, B, prompt, budget_s=20.0, max_tokens=256):
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
-def measure_prefill(B=8, h=4, N=8192, d=256, T=2048, density=0.05, steps=10, warmup=3):
+def measure_prefill(B=8, h=4, N=8192, d=256, T=2048, density=0.05, steps=10, warmup=3, rotary="rope",
+                    row_normalize=False, all_scores=False):
     """BASELINE config 3: chunked prefill, B=8, T=2048, h=4, N=8192, d=256, bf16 inputs, f32
-    accumulate, 5 % density, positions 0..T, fresh state.  One step = one bdh_prefill_chunked.
+    accumulate, 5 % density, positions 0..T, fresh state.  One step = one bdh_prefill_chunked (RoPE), or one
+    bdh_prefill_chunked_ex for PoPE (2N state rows), ALiBi (decaying state, default slopes) and the row-normalised
+    stateless form (time blocks of 64; ALiBi then adds its term to the scores).
     Returns (ms per call, algorithmic FLOP per call)."""
     import torch
     from scipy.stats import norm
 
     from burn_dragon_amd.kernel.linear_attention import build_freqs
     from burn_dragon_amd.positional import RotaryEmbedding
-    from burn_dragon_amd.recurrent import prefill_chunked
+    from burn_dragon_amd.recurrent import prefill_chunked, prefill_chunked_ex
 
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(4)
@@ -128,21 +131,31 @@ def measure_prefill(B=8, h=4, N=8192, d=256, T=2048, density=0.05, steps=10, war
     for b in range(B):  # generated per batch entry to bound the f32 temporary
         x[b] = torch.relu(torch.randn((h, T, N), device=dev, generator=g) + mu).to(torch.bfloat16)
     v = torch.randn((B, T, d), device=dev, generator=g).to(torch.bfloat16)
-    freqs = build_freqs(N, 65536.0, RotaryEmbedding.ROPE).reshape(-1).to(dev)
-    rho = torch.zeros((B, h, N, d), device=dev)
+    rot = RotaryEmbedding.parse(rotary)
+    nq = 2 * N if rot == RotaryEmbedding.POPE else N
+    freqs = build_freqs(N, 65536.0, rot).reshape(-1).to(dev)
+    rho = None if row_normalize else torch.zeros((B, h, nq, d), device=dev)
+    if rot == RotaryEmbedding.ROPE and not row_normalize:
+        call = lambda: prefill_chunked(x, v, rho, freqs, 0, state_is_zero=True, all_scores=all_scores)
+    else:
+        slopes = None
+        if rot == RotaryEmbedding.ALIBI and row_normalize:  # the additive term needs explicit slopes
+            slopes = [1.0 / 2.0 ** (i / h) for i in range(h)]
+        call = lambda: prefill_chunked_ex(x, v, rho, freqs, 0, rotary=rot, alibi_slopes=slopes,
+                                          row_normalize=row_normalize, block_size=64, state_is_zero=True)
     for _ in range(warmup):
-        prefill_chunked(x, v, rho, freqs, 0, state_is_zero=True)
+        call()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
     for _ in range(steps):
-        prefill_chunked(x, v, rho, freqs, 0, state_is_zero=True)
+        call()
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms = max(start.elapsed_time(stop), wall * 1e3) / steps
-    flop = float(B * h) * (T * (T - 1.0) * N + T * (T - 1.0) * d + 2.0 * T * N * d)
+    flop = float(B * h) * (T * (T - 1.0) * nq + T * (T - 1.0) * d + (0.0 if row_normalize else 2.0 * T * nq * d))
     return ms, flop
 
 
@@ -217,9 +230,11 @@ def bench_prefill(args):
     h, N, d, T = args.heads, args.latent, args.embd, args.time
     steps = min(args.steps, 20) if args.steps == 1000 else args.steps
     warmup = min(args.warmup, 3) if args.warmup == 50 else args.warmup
-    ms, flop = measure_prefill(B, h, N, d, T, args.density, steps, warmup)
+    ms, flop = measure_prefill(B, h, N, d, T, args.density, steps, warmup, args.rotary, args.row_normalize,
+                               args.all_scores)
     achieved = flop / (ms * 1e-3) / 1e12
-    chunked = d == 256 and N % 256 == 0 and T % 256 == 0
+    plain = args.rotary == "rope" and not args.row_normalize
+    chunked = plain and not args.all_scores and d == 256 and N % 256 == 0 and T % 256 == 0
     executed = prefill_executed_flop(B, h, N, d, T) if chunked else None
     print(json.dumps({
         "metric": "prefill tokens/sec (chunked dense linear attention) + bf16 MFMA utilisation",
@@ -227,7 +242,9 @@ def bench_prefill(args):
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"BASELINE config 3: chunked prefill B={B} T={T} h={h} N={N} d={d}, bf16 in / f32 "
-                               f"accumulate, {args.density:.0%} active, RoPE positions 0..T, fresh state",
+                               f"accumulate, {args.density:.0%} active, {args.rotary} positions 0..T, fresh state"
+                               + (", row-normalised stateless form (time blocks of 64)" if args.row_normalize else "")
+                               + ("" if chunked else ", all-scores form"),
                    "algorithmic_flop_per_step": flop, "executed_flop_per_step": executed},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
@@ -733,6 +750,10 @@ def main():
     ap.add_argument("--defer", type=int, default=0, metavar="K",
                     help="model (c1, c4): decode with deferred state updates, a log of K steps per layer")
     ap.add_argument("--time", type=int, default=2048, help="prefill: tokens per sequence")
+    ap.add_argument("--rotary", choices=["rope", "alibi", "pope"], default="rope", help="prefill: positional scheme")
+    ap.add_argument("--row-normalize", action="store_true",
+                    help="prefill: the row-normalised stateless form of fused_state_aligned on the bf16 matrix cores")
+    ap.add_argument("--all-scores", action="store_true", help="prefill: never the chunk-recurrent form")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="library launch-shape option set on the context before the run (repeatable)")
     args = ap.parse_args()
