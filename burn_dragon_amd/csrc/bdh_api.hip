@@ -189,6 +189,17 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     ctx->opt_fsa_path = value;
     return BDH_OK;
   }
+  if (strcmp(name, "model.fused_rows") == 0) {
+    if (value < 0 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "model.fused_rows takes 0 or 1");
+    ctx->opt_model_fused_rows = value;
+    return BDH_OK;
+  }
+  if (strcmp(name, "model.fused_kb") == 0) {
+    if (value != 128 && value != 256 && value != 512 && value != 1024 && value != 2048)
+      return bdh_fail(ctx, BDH_E_INVAL, "model.fused_kb takes 128, 256, 512, 1024 or 2048");
+    ctx->opt_model_fused_kb = value;
+    return BDH_OK;
+  }
   if (strcmp(name, "state_step.prompt_bf16") == 0) {
     if (value < 0) return bdh_fail(ctx, BDH_E_INVAL, "state_step.prompt_bf16 takes 0 (never) or a token count");
     ctx->opt_step_prompt_bf16 = value;

@@ -34,6 +34,8 @@ struct bdh_ctx {
   int opt_step_dense_kernel = 1;  // 0: PoPE / eager ALiBi at d in {256,512} take the generic kernel
   int opt_decoder_splitk_rows = 24;  // decode-step encoder on the matrix cores from this many sequences on
   int opt_fsa_path = -1;    // fused_state_aligned: -1 choose by T, 0 row kernel, 1 f32 matrix cores
+  int opt_model_fused_rows = 1;  // 0: a one-sequence decode step never folds its reductions into the projections
+  int opt_model_fused_kb = 256;  // rows of E per workgroup of the encoder's first stage in that form
   int opt_step_prompt_bf16 = 0;  // many-token state step on the bf16 matrix cores from this many tokens on (0: never)
   // time-block mask of the last sparse fused_state_aligned pattern (device) and the pattern it was built from
   void *fsa_mask = nullptr;
@@ -113,6 +115,13 @@ struct StateStepParams {
   uint64_t *bitmask;
   int32_t *rows_touched;
   int32_t *stamps = nullptr;  // ALiBi only: [B,h,N] decay stamps of a lazily decayed state, or null
+  // T = 1 on the RoPE kernels (d in {256, 512}) only: leave the readout as the per-workgroup partial sums
+  // [B*h][S][d] in the context's workspace (the caller's next kernel adds them up): no second stage, `out` unused
+  struct StepPartials *partials_out = nullptr;
+};
+struct StepPartials {
+  const float *partial = nullptr;
+  int S = 0;
 };
 int bdh_launch_state_steps(bdh_ctx *ctx, const StateStepParams &p);
 
@@ -156,6 +165,34 @@ struct ReluLowrankParams {
 int bdh_launch_relu_lowrank(bdh_ctx *ctx, const ReluLowrankParams &p);
 // the same on the f32 matrix cores for many rows per (sequence, head); csrc/attention_parallel.hip
 int bdh_launch_relu_lowrank_gemm(bdh_ctx *ctx, const ReluLowrankParams &p, const unsigned char *mask_dev);
+// relu_lowrank for ONE input row per head whose values are made by the kernel itself from the partial sums an earlier
+// kernel left (a decode step of one sequence: the two reductions of a layer whose inputs come from other CUs ride in
+// front of the projection that consumes them, behind its first weight loads):
+//   mode 1 (D_y, src/model/bdh.rs:359,370-381): row of head hh = LN(sum_g partial[hh][g][:]), g < S
+//   mode 2 (D_x of the next layer, :436-441 then :346-350): row = LN(cur_old + LN(sum_kb dpart[kb][:])), kb < KBN,
+//           shared by the heads; the workgroup (0, 0) also writes it to cur_new
+//   mode 3 (D_x of the first layer, :319-322 then :346-350): row = LN(embed[tokens[0]]), written to cur_new too
+struct ReluLowrankRowParams {
+  int mode, h, N, d;
+  const float *weight;
+  float threshold;
+  const float *gate;  // [h][N] or null
+  float *out;         // [h][N]
+  const float *partial;  // mode 1: [h][S][d]; mode 2: [KBN][d]
+  int rows;              // S or KBN
+  const float *cur_old;  // mode 2
+  float *cur_new;        // modes 2 and 3
+  const int64_t *tokens = nullptr;  // mode 3: device, the one token; partial = the embedding table, rows = V
+};
+int bdh_launch_relu_lowrank_row(bdh_ctx *ctx, const ReluLowrankRowParams &p);
+bool bdh_relu_lowrank_row_fits(int d, int rows);
+// The first stage of the encoder for one row (M = 1): partial[kb][:] = sum over k-block kb of xy[k] E[k,:], KB rows
+// per block; *KBN_out = number of blocks.  partial must hold KBN * d floats.
+int bdh_launch_decoder_partial_row(bdh_ctx *ctx, int h, int N, int d, const float *xy, const float *decoder, int KB,
+                                   float *partial, int *KBN_out);
+// cur[m,:] = LN(cur[m,:] + LN(sum_kb partial[kb][m][:])) and, with head, the output head of the finished rows
+int bdh_launch_decoder_finalize_head(bdh_ctx *ctx, const float *partial, int KBN, int M, int d, float *cur,
+                                     const struct DecoderHead *head);
 int bdh_launch_layer_norm(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);
 // the same for internal many-row use: statistics by wave reduction, not bit-identical to the index-order sums
 int bdh_launch_layer_norm_rows(bdh_ctx *ctx, int64_t rows, int d, const float *in, float *out);

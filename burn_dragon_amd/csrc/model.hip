@@ -4,6 +4,7 @@
 #include <vector>
 
 #include "bdh_internal.h"
+#include <utility>
 
 namespace {
 
@@ -241,6 +242,50 @@ int model_forward_impl(bdh_model *m, const int64_t *tokens, int B, int T, StateR
       if (rc2 != BDH_OK) return rc2;
       return bdh_launch_lm_head(ctx, B, 1, d, V, cur_final, m->w.lm_head, logits, next_tokens);
     }
+  }
+
+  // A decode step of ONE sequence through a RoPE model too large for the fused forms above (BASELINE config 1): four
+  // launches per layer instead of six.  The two reductions whose inputs come from other CUs -- the readout partials with
+  // their LayerNorm, the encoder partials with the two LayerNorms and the residual -- are redone by every workgroup of the
+  // projection that consumes the result (D_y, the next layer's D_x), behind its first weight loads.
+  if (B == 1 && T == 1 && !x_tap && !viz && !logs && ctx->opt_model_fused_rows != 0 && c.rotary == BDH_ROPE &&
+      (d == 256 || d == 512) && N >= 2 && (N % 2) == 0) {
+    const int KB = ctx->opt_model_fused_kb;
+    const size_t K = (size_t)h * N;
+    const size_t kbn_max = (K + KB - 1) / KB;
+    const size_t n_row = bdh_align_up((size_t)d, 64), n_lat = bdh_align_up(K, 64);
+    int rc2 = ensure_act(m, sizeof(float) * (2 * n_row + 2 * n_lat + kbn_max * d));
+    if (rc2 != BDH_OK) return rc2;
+    float *cur_a = static_cast<float *>(m->act);
+    float *cur_b = cur_a + n_row;
+    float *xr = cur_b + n_row;
+    float *xyr = xr + n_lat;
+    float *dpart = xyr + n_lat;
+    int KBN = 0;
+    for (int l = 0; l < L; ++l) {
+      if (l == 0) {  // :319-322, then :346-350
+        ReluLowrankRowParams px{3, h, N, d, m->w.encoder, c.relu_threshold, nullptr, xr, m->w.embed, V, nullptr, cur_a, tokens};
+        rc2 = bdh_launch_relu_lowrank_row(ctx, px);
+      } else {  // :436-441 of the previous layer, then :346-350
+        ReluLowrankRowParams px{2, h, N, d, m->w.encoder, c.relu_threshold, nullptr, xr, dpart, KBN, cur_a, cur_b};
+        rc2 = bdh_launch_relu_lowrank_row(ctx, px);
+        std::swap(cur_a, cur_b);
+      }
+      if (rc2 != BDH_OK) return rc2;
+      StepPartials sp;
+      StateStepParams ps{1, h, 1, N, d, c.rotary, rho_dtype, xr, cur_a, m->freqs, position, positions_dev, nullptr,
+                         st.rho(l), nullptr, nullptr, nullptr, nullptr, &sp};
+      rc2 = bdh_launch_state_steps(ctx, ps);
+      if (rc2 != BDH_OK) return rc2;
+      // :359,370-381  xy = x * relu(LN(sum of the readout partials) . encoder_v - thr)
+      ReluLowrankRowParams py{1, h, N, d, m->w.encoder_v, c.relu_threshold, xr, xyr, sp.partial, sp.S, nullptr, nullptr};
+      rc2 = bdh_launch_relu_lowrank_row(ctx, py);
+      if (rc2 != BDH_OK) return rc2;
+      rc2 = bdh_launch_decoder_partial_row(ctx, h, N, d, xyr, m->w.decoder, KB, dpart, &KBN);  // :383
+      if (rc2 != BDH_OK) return rc2;
+    }
+    const DecoderHead head{m->w.lm_head, 1, V, logits, next_tokens};
+    return bdh_launch_decoder_finalize_head(ctx, dpart, KBN, 1, d, cur_a, &head);  // :436-449
   }
 
   // activation scratch: cur [M,d] | x [B,h,T,N] | xy [B,h,T,N] | attn [B,h,T,d] | attn_ln [B,h,T,d] | last [h,d]

@@ -106,6 +106,177 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank(const float *__restrict__
   }
 }
 
+// One input row per head that the kernel makes itself (a decode step of one sequence).  The reductions of a layer whose
+// inputs come from other CUs -- the sum of the state step's readout partials with its LayerNorm (src/model/bdh.rs:359),
+// the sum of the encoder's partials with the two LayerNorms and the residual (:436-441) -- run in front of the
+// projection that consumes their result, in every workgroup, behind the workgroup's first UK weight loads: as launches
+// of their own each is a launch gap plus a chain of dependent trips to memory.
+//   MODE 1: row(hh) = LN(sum_g partial[hh][g][:])                      rows = S partial rows per head
+//   MODE 2: row     = LN(cur_old + LN(sum_kb partial[kb][:]))          rows = KBN, the same row for every head;
+//           workgroup (0, 0) writes it to cur_new (another buffer than cur_old: other workgroups still read that)
+//   MODE 3: row     = LN(embed[tokens[0]][:])   (src/model/bdh.rs:319-322; a token outside [0, V) gives a NaN row, as
+//           k_embed_ln does)                      partial = the embedding table, rows = V; written to cur_new too
+// The NW waves split the partial rows, a lane owns four adjacent columns of up to four column groups (d <= 1024),
+// every wave then finishes the row on its own with wave shuffles (the same arithmetic in every wave and workgroup, so
+// all of them hold the same bits).  Then k_relu_lowrank's one k-sequential fmaf chain per output.
+struct RowArgs {
+  const float *partial;
+  int rows;
+  const float *cur_old;
+  float *cur_new;
+  const int64_t *tokens;  // MODE 3
+};
+
+template <int MODE, int UK, int NTHR>
+__global__ __launch_bounds__(NTHR) void k_relu_lowrank_row1(RowArgs a, int d, const float *__restrict__ w, int h, int N,
+                                                           float thr, const float *__restrict__ gate,
+                                                           float *__restrict__ out) {
+  constexpr int NW = NTHR / 64;
+  extern __shared__ float s_row[];  // [d] the finished row | [NW][d] the waves' partial sums
+  float *s_in = s_row;
+  float *s_grp = s_row + d;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int hh = blockIdx.y;
+  const int n = blockIdx.x * NTHR + tid;
+  const bool col = n < N;
+  const float *wp = w + (long)hh * d * N + (col ? n : 0);
+  // the first UK weight rows are on their way while the row is made (d >= UK)
+  float wv[UK];
+#pragma unroll
+  for (int u = 0; u < UK; ++u) wv[u] = wp[(long)u * N];
+
+  const float *src = a.partial + (MODE == 1 ? (long)hh * a.rows * d : 0);
+  int n_rows = a.rows;
+  bool bad_token = false;
+  if (MODE == 3) {
+    const long tok = a.tokens[0];
+    bad_token = tok < 0 || tok >= a.rows;
+    src = a.partial + (bad_token ? 0 : tok) * d;
+    n_rows = 1;
+  }
+  const int per = (n_rows + NW - 1) / NW;
+  const int r0 = min(n_rows, wave * per), r1 = min(n_rows, r0 + per);
+  float4 res[4];
+  if (MODE == 2) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = (j * 64 + lane) * 4;
+      res[j] = c < d ? *reinterpret_cast<const float4 *>(a.cur_old + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = (j * 64 + lane) * 4;
+    if (c < d) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      int r = r0;
+      for (; r + 32 <= r1; r += 32) {  // 32 rows in flight: the sum is a chain of trips to the L2
+        float4 t[32];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) t[u] = *reinterpret_cast<const float4 *>(src + (long)(r + u) * d + c);
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+          v.x += t[u].x; v.y += t[u].y; v.z += t[u].z; v.w += t[u].w;
+        }
+      }
+      if (r < r1) {  // up to 31 rows left: all asked for at once
+        float4 t[31];
+#pragma unroll
+        for (int u = 0; u < 31; ++u)
+          t[u] = r + u < r1 ? *reinterpret_cast<const float4 *>(src + (long)(r + u) * d + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 31; ++u)
+          if (r + u < r1) {
+            v.x += t[u].x; v.y += t[u].y; v.z += t[u].z; v.w += t[u].w;
+          }
+      }
+      if (MODE == 3 && bad_token) v = make_float4(NAN, NAN, NAN, NAN);
+      *reinterpret_cast<float4 *>(s_grp + wave * d + c) = v;
+    }
+  }
+  __syncthreads();
+  {
+    auto wave_sum = [](float v) {
+      for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+      return v;
+    };
+    float4 vals[4];
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = (j * 64 + lane) * 4;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c < d) {
+        v = *reinterpret_cast<const float4 *>(s_grp + c);
+#pragma unroll
+        for (int g = 1; g < NW; ++g) {
+          const float4 t = *reinterpret_cast<const float4 *>(s_grp + g * d + c);
+          v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+        }
+        s += (v.x + v.y) + (v.z + v.w);
+      }
+      vals[j] = v;
+    }
+    auto layer_norm4 = [&](float total) {  // vals <- (vals - mean) / sqrt(var + eps) over the d columns
+      const float mean = wave_sum(total) / (float)d;
+      float q = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if ((j * 64 + lane) * 4 < d) {
+          const float tx = vals[j].x - mean, ty = vals[j].y - mean, tz = vals[j].z - mean, tw = vals[j].w - mean;
+          q += (tx * tx + ty * ty) + (tz * tz + tw * tw);
+        }
+      const float den = sqrtf(wave_sum(q) / (float)d + kLnEps);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        vals[j].x = (vals[j].x - mean) / den; vals[j].y = (vals[j].y - mean) / den;
+        vals[j].z = (vals[j].z - mean) / den; vals[j].w = (vals[j].w - mean) / den;
+      }
+    };
+    layer_norm4(s);
+    if (MODE == 2) {
+      s = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if ((j * 64 + lane) * 4 < d) {
+          vals[j].x += res[j].x; vals[j].y += res[j].y; vals[j].z += res[j].z; vals[j].w += res[j].w;
+          s += (vals[j].x + vals[j].y) + (vals[j].z + vals[j].w);
+        }
+      layer_norm4(s);
+    }
+    if (wave == 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int c = (j * 64 + lane) * 4;
+        if (c < d) {
+          *reinterpret_cast<float4 *>(s_in + c) = vals[j];
+          if (MODE != 1 && blockIdx.x == 0 && hh == 0) *reinterpret_cast<float4 *>(a.cur_new + c) = vals[j];
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  float acc = 0.0f;
+#pragma unroll
+  for (int u = 0; u < UK; ++u) acc = __builtin_fmaf(s_in[u], wv[u], acc);
+  int k0 = UK;
+  for (; k0 + UK <= d; k0 += UK) {
+#pragma unroll
+    for (int u = 0; u < UK; ++u) wv[u] = wp[(long)(k0 + u) * N];
+#pragma unroll
+    for (int u = 0; u < UK; ++u) acc = __builtin_fmaf(s_in[k0 + u], wv[u], acc);
+  }
+  for (; k0 < d; ++k0) acc = __builtin_fmaf(s_in[k0], wp[(long)k0 * N], acc);
+  if (!col) return;
+  float pv = acc;
+  if (thr != 0.0f) pv = pv - thr;
+  float y = pv > 0.0f ? pv : 0.0f;
+  const long o = (long)hh * N + n;
+  if (gate) y = gate[o] * y;
+  out[o] = y;
+}
+
 // A few input rows against a SMALL weight matrix (a few MiB: it sits in the L2): with one thread per column there
 // are only a handful of workgroups and each thread walks k in rounds of loads.  Here NW waves share 64
 // columns: each wave asks for its own 64-row span of k at once, so every weight of the matrix is in flight
@@ -471,8 +642,8 @@ __global__ __launch_bounds__(256) void k_embed_ln(const int64_t *__restrict__ to
 // mixed[m = b*T+t, k = hh*N+n] = xy[b,hh,t,n].  Rows of E whose xy is zero for every row
 // of the tile are never loaded.
 // ------------------------------------------------------------------------------------
-template <int RT, int MAXV, int UF = 4>
-__global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict__ xy,
+template <int RT, int MAXV, int UF = 4, int NWV = 4>  // NWV waves per workgroup share a k-block
+__global__ __launch_bounds__(NWV * 64) void k_decoder_partial(const float *__restrict__ xy,
                                                          const float *__restrict__ E,
                                                          float *__restrict__ partial, int T, int h, int N,
                                                          int d, int KB, int M) {
@@ -484,7 +655,7 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
   const int K = h * N;
   const int nv = (d + 255) >> 8;  // float4 groups per lane
   float *s_xy = s_mem;
-  for (int i = tid; i < RT * KB; i += 256) {
+  for (int i = tid; i < RT * KB; i += NWV * 64) {
     const int r = i / KB, kk = i - r * KB;
     const int m = m0 + r, k = kb * KB + kk;
     float val = 0.0f;
@@ -503,14 +674,14 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) acc[r][j] = make_float4(0.f, 0.f, 0.f, 0.f);
 
-  // each wave takes k = wave, wave+4, ...; UF of its E rows are in flight at a time
-  for (int kk0 = wave; kk0 < KB; kk0 += 4 * UF) {
+  // each wave takes k = wave, wave+NWV, ...; UF of its E rows are in flight at a time
+  for (int kk0 = wave; kk0 < KB; kk0 += NWV * UF) {
     float xs[UF][RT];
     bool any[UF];
     float4 e[UF][MAXV];
 #pragma unroll
     for (int u = 0; u < UF; ++u) {
-      const int kk = kk0 + 4 * u;
+      const int kk = kk0 + NWV * u;
       const int k = kb * KB + kk;
       any[u] = false;
       if (kk < KB && k < K) {
@@ -549,7 +720,7 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
     }
   }
   __syncthreads();
-  // cross-wave reduction, one row of the tile at a time, through LDS [4][d]
+  // cross-wave reduction, one row of the tile at a time, through LDS [NWV][d]
   float *s_red = s_mem;
   for (int r = 0; r < RT; ++r) {
 #pragma unroll
@@ -560,8 +731,12 @@ __global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict
     __syncthreads();
     const int m = m0 + r;
     if (m < M)
-      for (int c = tid; c < d; c += 256)
-        partial[((long)kb * M + m) * d + c] = s_red[c] + s_red[d + c] + s_red[2 * d + c] + s_red[3 * d + c];
+      for (int c = tid; c < d; c += NWV * 64) {
+        float v = s_red[c] + s_red[d + c] + s_red[2 * d + c] + s_red[3 * d + c];
+#pragma unroll
+        for (int g = 4; g < NWV; ++g) v += s_red[g * d + c];
+        partial[((long)kb * M + m) * d + c] = v;
+      }
     __syncthreads();
   }
 }
@@ -1197,6 +1372,56 @@ int bdh_launch_decoder_residual(bdh_ctx *ctx, int B, int T, int h, int N, int d,
   }
 #undef BDH_DEC
   BDH_LAUNCH_CHECK(ctx, "k_decoder_partial");
+  launch_decoder_finalize(ctx, partial, KBN, M, d, cur, head);
+  BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
+  return BDH_OK;
+}
+
+bool bdh_relu_lowrank_row_fits(int d, int rows) { return d >= 64 && d <= 1024 && (d & 3) == 0 && rows >= 1; }
+
+int bdh_launch_relu_lowrank_row(bdh_ctx *ctx, const ReluLowrankRowParams &p) {
+  if (!bdh_relu_lowrank_row_fits(p.d, p.rows)) return bdh_fail(ctx, BDH_E_SHAPE, "fused row projection: d=%d rows=%d", p.d, p.rows);
+  constexpr int NTHR = 128, UK = 64;
+  const dim3 grid((p.N + NTHR - 1) / NTHR, p.h);
+  const size_t lds = sizeof(float) * (size_t)p.d * (1 + NTHR / 64);
+  const RowArgs a{p.partial, p.rows, p.cur_old, p.cur_new, p.tokens};
+  if (p.mode == 1)
+    hipLaunchKernelGGL((k_relu_lowrank_row1<1, UK, NTHR>), grid, dim3(NTHR), lds, ctx->stream, a, p.d, p.weight, p.h, p.N,
+                       p.threshold, p.gate, p.out);
+  else if (p.mode == 3)
+    hipLaunchKernelGGL((k_relu_lowrank_row1<3, UK, NTHR>), grid, dim3(NTHR), lds, ctx->stream, a, p.d, p.weight, p.h, p.N,
+                       p.threshold, p.gate, p.out);
+  else
+    hipLaunchKernelGGL((k_relu_lowrank_row1<2, UK, NTHR>), grid, dim3(NTHR), lds, ctx->stream, a, p.d, p.weight, p.h, p.N,
+                       p.threshold, p.gate, p.out);
+  BDH_LAUNCH_CHECK(ctx, "k_relu_lowrank_row1");
+  return BDH_OK;
+}
+
+int bdh_launch_decoder_partial_row(bdh_ctx *ctx, int h, int N, int d, const float *xy, const float *decoder, int KB,
+                                   float *partial, int *KBN_out) {
+  const long K = (long)h * N;
+  if (d > 1024 || (d & 3)) return bdh_fail(ctx, BDH_E_SHAPE, "decoder needs d %% 4 == 0 and d <= 1024, got %d", d);
+  const int KBN = (int)((K + KB - 1) / KB);
+  // 16 waves share a k-block: as many waves in flight as 128-row blocks of four waves give, a quarter of the partial rows
+  size_t lds = sizeof(float) * (size_t)KB;
+  if (lds < sizeof(float) * 16u * d) lds = sizeof(float) * 16u * d;
+  const dim3 grid(KBN, 1);
+  const int mv = d <= 256 ? 1 : (d <= 512 ? 2 : 4);
+  if (mv == 1)
+    hipLaunchKernelGGL((k_decoder_partial<1, 1, 16, 16>), grid, dim3(1024), lds, ctx->stream, xy, decoder, partial, 1, h, N, d, KB, 1);
+  else if (mv == 2)
+    hipLaunchKernelGGL((k_decoder_partial<1, 2, 8, 16>), grid, dim3(1024), lds, ctx->stream, xy, decoder, partial, 1, h, N, d, KB, 1);
+  else
+    hipLaunchKernelGGL((k_decoder_partial<1, 4, 4, 16>), grid, dim3(1024), lds, ctx->stream, xy, decoder, partial, 1, h, N, d, KB, 1);
+  BDH_LAUNCH_CHECK(ctx, "k_decoder_partial");
+  *KBN_out = KBN;
+  return BDH_OK;
+}
+
+int bdh_launch_decoder_finalize_head(bdh_ctx *ctx, const float *partial, int KBN, int M, int d, float *cur,
+                                     const DecoderHead *head) {
+  if (d > 1024 || (d & 3) != 0) return bdh_fail(ctx, BDH_E_SHAPE, "encoder second stage needs d %% 4 == 0 and d <= 1024");
   launch_decoder_finalize(ctx, partial, KBN, M, d, cur, head);
   BDH_LAUNCH_CHECK(ctx, "k_decoder_finalize");
   return BDH_OK;

@@ -1002,6 +1002,8 @@ int bdh_launch_state_steps_in(bdh_ctx *ctx, const StateStepParams &p, float *out
   if ((long)slices > 0x7fffffffL / 4096) return bdh_fail(ctx, BDH_E_SHAPE, "B*h too large");
 
   const bool fast = p.rotary == BDH_ROPE && (d == 256 || d == 512) && N >= 2;
+  if (p.partials_out && (!fast || T != 1 || fixed || p.bitmask || p.rows_touched))
+    return bdh_fail(ctx, BDH_E_UNSUPPORTED, "readout partials are only handed over by a single-token RoPE step at d in {256, 512}");
   // few slices (small batch): 64 pairs per workgroup of 8 waves, so the grid still covers the chip
   const int n_cu = ctx->n_cu > 0 ? ctx->n_cu : 256;
   const bool split = fast && (ctx->opt_step_split >= 0 ? ctx->opt_step_split == 1
@@ -1144,6 +1146,11 @@ int bdh_launch_state_steps_in(bdh_ctx *ctx, const StateStepParams &p, float *out
           hipLaunchKernelGGL((k_step_rope_bf16<512, 8, 2, 8>), dim3(blocks), dim3(512), 0, ctx->stream, a, rho);
       }
       BDH_LAUNCH_CHECK(ctx, "k_step_rope");
+      if (p.partials_out) {  // the caller's next kernel adds the partials up
+        p.partials_out->partial = partial;
+        p.partials_out->S = S;
+        return BDH_OK;
+      }
       launch_finalize(ctx->stream, slices, partial, pair_cnt, S, d, out_t, (long)T * d, out_ln_t, rows_t, (long)T, 2, nt,
                       a.partial_t_stride, a.cnt_t_stride);
       BDH_LAUNCH_CHECK(ctx, "k_step_finalize");

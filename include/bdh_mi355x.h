@@ -121,6 +121,13 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       workgroup per block, while batch x weights of a layer stay under 256 MiB.
  *                       2 = the one-launch step whenever the model fits it; 0 = kernel by kernel like any
  *                       other call (values agree to 1e-5: other summation trees).
+ *   "model.fused_rows": 1 (default) a decode step of ONE sequence (B = 1, T = 1, no x_tap / viz) through a RoPE
+ *                       model with n_embd in {256, 512} that is too large for the forms above takes four launches
+ *                       per layer instead of six: D_y sums the state step's readout partials and applies their
+ *                       LayerNorm itself, the next layer's D_x sums the encoder's partials and applies the two
+ *                       LayerNorms and the residual (the first layer's D_x makes its row from the embedding), each
+ *                       behind its first weight loads.  0 = kernel by kernel (values agree to 1e-5).
+ *   "model.fused_kb":   rows of E per workgroup of the encoder's first stage in that form (128 .. 2048, default 256).
  *   "model.phase_batch": the two-launch layer only for at most this many sequences (default: no limit
  *                       beyond the one above; 0 = never).
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,

@@ -237,11 +237,11 @@ def _shape_from_cfg(cfg):
                         relu_threshold=cfg.fused_kernels.relu_threshold, alibi_slopes=cfg.fused_kernels.alibi_slopes)
 
 
-def _model_pair(bda, cfg, seed):
+def _model_pair(bda, cfg, seed, **kw):
     shape = _shape_from_cfg(cfg)
     w = orc.init_weights(shape, seed)
     model = bda.BDH(cfg, DEV, weights={"embed": w.embed, "encoder": w.encoder, "encoder_v": w.encoder_v,
-                                       "decoder": w.decoder, "lm_head": w.lm_head})
+                                       "decoder": w.decoder, "lm_head": w.lm_head}, **kw)
     return shape, w, model
 
 
@@ -715,3 +715,47 @@ def test_decode_graph_replays_match_eager_steps(bda, d, mult):
         assert int(graph.positions[0]) == sg.position
         nxt_e = new_e
         del junk
+
+
+@pytest.mark.parametrize("d,mult,h,state", [(256, 32, 4, "f32"), (512, 16, 2, "f32"), (256, 32, 4, "bf16")])
+def test_single_sequence_decode_folds_the_reductions_into_the_projections(bda, corc, d, mult, h, state):
+    """A decode step of one sequence through a RoPE model with more than 64 blocks of 64 neurons takes four launches
+    per layer ("model.fused_rows"): D_y sums the readout partials and applies their LayerNorm itself, the next layer's
+    D_x the encoder partials with the two LayerNorms and the residual.  Against the kernel-by-kernel step (1e-5: other
+    summation trees; a bf16 state: one rounding step) and the oracle (1e-3 / 2e-2), over a prompt and 12 greedy steps;
+    the state both leave is compared too."""
+    from burn_dragon_amd import ffi
+
+    cfg = bda.BDHConfig(n_layer=3, n_embd=d, n_head=h, mlp_internal_dim_multiplier=mult, vocab_size=256)
+    cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
+    dt = ffi.BF16 if state == "bf16" else ffi.F32
+    shape, w, model = _model_pair(bda, cfg, seed=13, rho_dtype=dt)
+    N = model.latent
+    assert h * N // 64 > 64  # too many blocks for the two-launch layer
+    ctx = ffi.default_context(0)
+    prompt = np.random.default_rng(3).integers(0, 256, size=(1, 9))
+    runs = {}
+    for fused in (1, 0):
+        ctx.set_option("model.fused_rows", fused)
+        try:
+            st = model.init_state()
+            lg, nxt = model.forward_with_state(torch.from_numpy(prompt), st, want_next=True)
+            steps = []
+            for _ in range(12):
+                lg, nxt2 = model.forward_with_state(nxt.reshape(1, 1), st, want_next=True)
+                steps.append((lg.cpu().numpy(), int(nxt[0])))
+                nxt = nxt2
+            torch.cuda.synchronize()
+            runs[fused] = (steps, st.storage.float().cpu().numpy())
+        finally:
+            ctx.set_option("model.fused_rows", 1)
+    tol_pair, tol_orc = (1e-5, 1e-3) if state == "f32" else (2e-2, 2e-2)
+    rho_ref = np.zeros((3, 1, h, N, d), np.float32)
+    logits_ref, pos, _, _ = corc.forward_with_state(shape, w, prompt, rho_ref, 0)
+    for (lg1, tok1), (lg0, tok0) in zip(*[runs[k][0] for k in (1, 0)]):
+        assert tok1 == tok0
+        assert rel_err(lg1, lg0) < tol_pair
+        logits_ref, pos, _, _ = corc.forward_with_state(shape, w, np.array([[tok1]]), rho_ref, pos)
+        assert rel_err(lg1, logits_ref) < tol_orc
+    assert rel_err(runs[1][1], runs[0][1]) < tol_pair
+    assert rel_err(runs[1][1], rho_ref) < tol_orc
