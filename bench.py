@@ -898,7 +898,9 @@ def main():
         # the same workload through the deferred-update step (flushes inside its timed region)
         del rho, xs, vs
         torch.cuda.empty_cache()
-        result["deferred"] = measure_deferred(steps=args.steps, warmup=max(args.warmup, 128))
+        # its own step count: at least eight log capacities, so that the flushes -- all of them inside its timed
+        # region, the final one included -- are amortised as in a decode loop, whatever --steps says for the line's value
+        result["deferred"] = measure_deferred(steps=max(args.steps, 8 * 128), warmup=max(args.warmup, 128))
         # BASELINE config 3 beside the headline: the chunked prefill, bf16 matrix cores (its own roofline)
         p_ms, p_flop = measure_prefill(steps=5, warmup=2)
         torch.cuda.empty_cache()
