@@ -399,3 +399,33 @@ def test_prefill_chunked_argument_errors(bda):
     assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 16, 8, p, p, p, 0, -1, 1, p, p) == ffi.E_INVAL  # chunk < 0
     assert ctx.lib.bdh_prefill_chunked(ctx.handle, 1, 1, 8, 16, 8, p, p, p, 0, 0, 64, p, p) == ffi.E_INVAL  # flag bits
     assert ctx.lib.bdh_prefill_chunked(ctx.handle, 0, 1, 8, 16, 8, None, None, None, 0, 0, 1, None, None) == ffi.OK
+
+
+def test_prefill_state_copies_tight_against_a_device_restatement(bda, corc):
+    """A tight check of the chunk-recurrent kernels' bf16 state copies (the stores of k_state_stream that need idle
+    cycles before their data registers are rewritten): the second and third 256-token chunks of a call read
+    bf16(rho_c) that the first kernel wrote.  The same quantities from plain f32 torch products on the device, with the
+    same roundings (Q = bf16 of the oracle's rotation, scores and state copies rounded to bf16 once, f32 accumulation),
+    must agree to 2e-3 of the output scale -- ten times tighter than the bf16 tolerance class, so a few corrupted
+    elements of a copy show."""
+    from burn_dragon_amd.recurrent import prefill_chunked
+
+    B, h, T, N, d = 1, 2, 768, 512, 256
+    x, v, _ = _prefill_case(77, B, h, T, N, d, 0.2, 0.0)
+    freqs = corc.build_freqs(N)
+    rho = torch.zeros((B, h, N, d), device=DEV)
+    out = prefill_chunked(x.to(DEV), v.to(DEV), rho, torch.from_numpy(freqs).to(DEV), 0, state_is_zero=True)
+    torch.cuda.synchronize()
+    q = torch.from_numpy(corc.rotate(x.float().numpy(), freqs, orc.ROPE, 0)).to(DEV).to(torch.bfloat16).float()
+    vf = v.float().to(DEV)
+    state = torch.zeros((B, h, N, d), device=DEV)
+    ref = torch.empty((B, h, T, d), device=DEV)
+    for c in range(T // 256):
+        sl = slice(c * 256, (c + 1) * 256)
+        qc, vc = q[:, :, sl], vf[:, None, sl]
+        scores = torch.tril(qc @ qc.transpose(2, 3), -1).to(torch.bfloat16).float()
+        ref[:, :, sl] = scores @ vc + qc @ state.to(torch.bfloat16).float()
+        state = state + qc.transpose(2, 3) @ vc
+    scale = ref.abs().max().item()
+    assert (out - ref).abs().max().item() < 2e-3 * scale
+    assert (rho - state).abs().max().item() < 2e-3 * state.abs().max().item()
