@@ -397,7 +397,12 @@ struct BDHWeightsHost {  // record order of the reference module
 
 class BDH {
  public:
-  BDH(const Context &ctx, const BDHConfig &config, const BDHWeightsHost &w) : ctx_(ctx), config_(config) {
+  // defer_updates = K > 0 (RoPE models with n_embd 256 or 512): single-token calls log their state updates and apply
+  // them every K tokens (bdh_model_forward_deferred); flush_state(), and every call that is not such a step, bring
+  // state.storage up to date first.  Logits and the flushed state agree with the eager step to f32 rounding (a layer
+  // fed the same inputs leaves the same bits; the readouts that feed deeper layers are reassociated sums).
+  BDH(const Context &ctx, const BDHConfig &config, const BDHWeightsHost &w, size_t defer_updates = 0)
+      : ctx_(ctx), config_(config), defer_updates_(defer_updates) {
     const size_t h = config.n_head, d = config.n_embd, N = config.latent_per_head(), V = config.vocab_size;
     embed_ = Tensor::from_host(w.embed, {V, d});
     encoder_ = Tensor::from_host(w.encoder, {h, d, N});
@@ -410,7 +415,16 @@ class BDH {
     bdh_model_weights mw{embed_.data(), encoder_.data(), encoder_v_.data(), decoder_.data(), lm_head_.data()};
     ctx_.check(bdh_model_create(ctx_.raw(), &c, &mw, &model_));
   }
-  ~BDH() { bdh_model_destroy(model_); }
+  ~BDH() {
+    if (logs_) bdh_model_logs_destroy(model_, logs_);
+    bdh_model_destroy(model_);
+  }
+
+  // applies the logged updates of a deferred state (no-op otherwise): afterwards state.storage is the reference's state
+  void flush_state(ModelState &state) {
+    if (logs_ && state.storage && bdh_model_logs_pending(logs_) > 0)
+      ctx_.check(bdh_model_flush(model_, logs_, state.storage->data()));
+  }
   BDH(const BDH &) = delete;
   BDH &operator=(const BDH &) = delete;
 
@@ -425,7 +439,18 @@ class BDH {
     const size_t h = config_.n_head, d = config_.n_embd, N = config_.latent_per_head();
     const size_t Nq = config_.fused_kernels.rotary_embedding == RotaryEmbedding::Pope ? 2 * N : N;
     const std::vector<size_t> want{config_.n_layer, batch, h, Nq, d};
-    if (!state.storage || state.storage->shape() != want) state.storage = Tensor::zeros(want);  // bdh.rs:274-284
+    if (!state.storage || state.storage->shape() != want) {  // bdh.rs:274-284
+      drop_logs();  // pending updates belong to the storage that is replaced
+      state.storage = Tensor::zeros(want);
+    }
+    const bool deferred = defer_updates_ > 0 && time == 1 && !viz && batch > 0;
+    if (deferred && (!logs_ || logs_batch_ != batch)) {
+      flush_state(state);
+      drop_logs();
+      ctx_.check(bdh_model_logs_create(model_, (int)batch, BDH_F32, (int)defer_updates_, &logs_));
+      logs_batch_ = batch;
+    }
+    if (!deferred) flush_state(state);
     int64_t *tok_dev = nullptr, *next_dev = nullptr;
     hip_check(hipMalloc(reinterpret_cast<void **>(&tok_dev), sizeof(int64_t) * std::max<size_t>(tokens.size(), 1)), "hipMalloc");
     hip_check(hipMalloc(reinterpret_cast<void **>(&next_dev), sizeof(int64_t) * std::max<size_t>(batch, 1)), "hipMalloc");
@@ -435,9 +460,13 @@ class BDH {
       hip_check(hipMemcpy(tok_dev, tokens.data(), sizeof(int64_t) * tokens.size(), hipMemcpyHostToDevice), "hipMemcpy");
       std::optional<Tensor> maps;
       if (viz) maps.emplace(std::vector<size_t>{config_.n_layer, 4, h, N});
-      rc = bdh_model_forward_viz(model_, tok_dev, (int)batch, (int)time, state.storage->data(), BDH_F32, nullptr,
-                                 (int64_t)state.position, nullptr, logits.data(), next_tokens ? next_dev : nullptr,
-                                 nullptr, maps ? maps->data() : nullptr);
+      if (deferred)
+        rc = bdh_model_forward_deferred(model_, logs_, tok_dev, (int)batch, state.storage->data(), BDH_F32,
+                                        (int64_t)state.position, nullptr, logits.data(), next_tokens ? next_dev : nullptr);
+      else
+        rc = bdh_model_forward_viz(model_, tok_dev, (int)batch, (int)time, state.storage->data(), BDH_F32, nullptr,
+                                   (int64_t)state.position, nullptr, logits.data(), next_tokens ? next_dev : nullptr,
+                                   nullptr, maps ? maps->data() : nullptr);
       if (rc == BDH_OK && maps) {
         ctx_.synchronize();
         const std::vector<float> host = maps->to_host();
@@ -502,10 +531,19 @@ class BDH {
   const BDHConfig &config() const { return config_; }
 
  private:
+  void drop_logs() {
+    if (logs_) bdh_model_logs_destroy(model_, logs_);
+    logs_ = nullptr;
+    logs_batch_ = 0;
+  }
+
   const Context &ctx_;
   BDHConfig config_;
   Tensor embed_, encoder_, encoder_v_, decoder_, lm_head_;
   bdh_model *model_ = nullptr;
+  size_t defer_updates_ = 0;
+  bdh_model_logs *logs_ = nullptr;  // one update log per layer, for a batch of logs_batch_ sequences
+  size_t logs_batch_ = 0;
 };
 
 }  // namespace bdh

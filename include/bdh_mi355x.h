@@ -513,7 +513,9 @@ int bdh_model_forward_viz(bdh_model *model, const int64_t *tokens, int B, int T,
  * layer logs one step per call, so all layers fill and flush together, the call that finds the logs full flushing
  * them first).  Until bdh_model_flush, rho [L,B,h,N,d] lags behind by the pending steps; flush before any other
  * entry point (a prompt call, bdh_model_forward*, bdh_rho_energy, an export) touches rho.  Logits agree with
- * bdh_model_forward_ex to f32 rounding of the reassociated readout; the flushed state holds its bits. */
+ * bdh_model_forward_ex to f32 rounding of the reassociated readout, and so does the flushed state: a layer applies
+ * its logged updates bit for bit as the eager step would (the first layer's state is bit-identical), but the
+ * readouts that feed the deeper layers differ by that rounding, and their updates with them. */
 typedef struct bdh_model_logs bdh_model_logs; /* opaque: one bdh_state_log per layer */
 int bdh_model_logs_create(bdh_model *model, int B, int rho_dtype, int capacity, bdh_model_logs **out);
 int bdh_model_logs_destroy(bdh_model *model, bdh_model_logs *logs);

@@ -140,6 +140,53 @@ static void inference_paths_run_across_configs(const Context &ctx) {
   }
 }
 
+// A decode loop with deferred state updates through the mirror (BDH(..., defer_updates)): logits against the oracle's
+// token loop, and the flushed state against the state an eager model leaves (layer 0: bit for bit).
+static void decode_with_deferred_updates(const Context &ctx) {
+  BDHConfig config;
+  config.n_layer = 2;
+  config.n_embd = 256;
+  config.n_head = 2;
+  config.mlp_internal_dim_multiplier = 4;  // N = 512 per head
+  config.vocab_size = 32;
+  config.dropout = 0.0;
+  config.fused_kernels.set_rotary_embedding(RotaryEmbedding::Rope);
+  std::mt19937 g(29);
+  const size_t h = 2, d = 256, N = config.latent_per_head(), V = 32, B = 2, steps = 11;
+  BDHWeightsHost w{randn(g, V * d, 1.0f), randn(g, h * d * N, 0.02f), randn(g, h * d * N, 0.02f), randn(g, h * N * d, 0.02f),
+                   randn(g, d * V, 0.02f)};
+  BDH eager(ctx, config, w), lazy(ctx, config, w, 4);  // a flush every 4 tokens
+  // the eager model kernel by kernel (a model of this size would take two launches per layer, whose state update
+  // is another instruction sequence): the deferred step logs what bdh_state_step would have written
+  ctx.check(bdh_ctx_set_option(ctx.raw(), "model.one_launch", 0));
+  ModelState se = eager.init_state(), sl = lazy.init_state();
+  std::vector<float> rho(2 * B * h * N * d, 0.0f), ref(B * V);
+  orc_model m{2, (int)d, (int)h, (int)N, (int)V, (int)RotaryEmbedding::Rope, 65536.0f, 0.0f, nullptr,
+              w.embed.data(), w.encoder.data(), w.encoder_v.data(), w.decoder.data(), w.lm_head.data()};
+  int64_t pos = 0;
+  double worst = 0.0;
+  for (size_t t = 0; t < steps; ++t) {
+    const std::vector<int64_t> tok{(int64_t)((3 * t + 1) % V), (int64_t)((5 * t + 2) % V)};
+    Tensor le = eager.forward_with_state(tok, B, 1, se);
+    Tensor ll = lazy.forward_with_state(tok, B, 1, sl);
+    EXPECT(orc_forward_with_state(&m, tok.data(), (int)B, 1, rho.data(), &pos, ref.data(), nullptr, nullptr, 0) == 0);
+    worst = std::max(worst, std::max(rel_err(ll.to_host(), ref), rel_err(ll.to_host(), le.to_host())));
+  }
+  std::printf("  deferred decode: worst logits rel err %.2e\n", worst);
+  EXPECT(worst < 1e-3);
+  EXPECT(sl.position == steps && (size_t)pos == steps);
+  lazy.flush_state(sl);
+  ctx.synchronize();
+  // the first layer sees the same inputs in both runs: its flushed state holds the eager step's bits; deeper layers
+  // receive readouts that differ by f32 rounding (the sums are reassociated), so their states agree to that level
+  const std::vector<float> a = sl.storage->to_host(), b = se.storage->to_host();
+  const size_t layer = B * h * N * d;
+  EXPECT(std::equal(a.begin(), a.begin() + layer, b.begin()));
+  EXPECT(rel_err(a, b) < 1e-5);
+  EXPECT(rel_err(a, rho) < 1e-3);
+  ctx.check(bdh_ctx_set_option(ctx.raw(), "model.one_launch", 1));
+}
+
 // src/model/attention.rs:383-432, the reference's own two known-answer tests, through the mirror
 static void attention_alibi_kats(const Context &ctx) {
   FusedKernelConfig kernel;
@@ -384,6 +431,8 @@ int main(int argc, char **argv) {
     }
     std::printf("inference_paths_run_across_configs\n");
     inference_paths_run_across_configs(ctx);
+    std::printf("decode_with_deferred_updates\n");
+    decode_with_deferred_updates(ctx);
     std::printf("attention_alibi_kats\n");
     attention_alibi_kats(ctx);
     std::printf("relu_lowrank_fused_matches_reference\n");
