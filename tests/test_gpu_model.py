@@ -688,22 +688,23 @@ def test_model_create_rejects_bad_configs(bda):
     assert err.value.status == ffi.E_SHAPE
 
 
-@pytest.mark.parametrize("d,mult", [(256, 16), (256, 128), (128, 4)], ids=["two-launch-layer", "kernel-by-kernel", "one-launch"])
-def test_decode_graph_replays_match_eager_steps(bda, d, mult):
+@pytest.mark.parametrize("d,mult,B", [(256, 16, 2), (256, 128, 2), (128, 4, 2), (256, 128, 1)],
+                         ids=["two-launch-layer", "kernel-by-kernel", "one-launch", "four-launch-layer"])
+def test_decode_graph_replays_match_eager_steps(bda, d, mult, B):
     """A captured decode step is replayed several times, with eager work and synchronisations of the
     same program between the replays, and every replay is checked against the eager path -- for each of
-    the three forms a decode step can take."""
+    the four forms a decode step can take."""
     cfg = bda.BDHConfig(n_layer=3, n_embd=d, n_head=4, mlp_internal_dim_multiplier=mult, vocab_size=64)
     cfg.fused_kernels.set_rotary_embedding(bda.RotaryEmbedding.ROPE)
     model = bda.BDH(cfg, DEV, seed=21)
-    prompt = torch.randint(0, 64, (2, 5), generator=torch.Generator().manual_seed(2))
+    prompt = torch.randint(0, 64, (B, 5), generator=torch.Generator().manual_seed(2))
     se, sg = model.init_state(), model.init_state()
     _, nxt_e = model.forward_with_state(prompt, se, want_next=True)
     _, nxt_g = model.forward_with_state(prompt, sg, want_next=True)
     graph = model.capture_decode_step(sg, nxt_g)
     assert torch.equal(sg.storage, se.storage)  # capture must not disturb the state
     for step in range(6):
-        logits_e, new_e = model.forward_with_state(nxt_e.reshape(2, 1), se, want_next=True)
+        logits_e, new_e = model.forward_with_state(nxt_e.reshape(B, 1), se, want_next=True)
         torch.cuda.synchronize()
         junk = torch.randn(1 << 16, device=DEV).sum()  # unrelated eager work between replays
         graph.replay()
