@@ -642,8 +642,8 @@ __global__ __launch_bounds__(256) void k_embed_ln(const int64_t *__restrict__ to
 // mixed[m = b*T+t, k = hh*N+n] = xy[b,hh,t,n].  Rows of E whose xy is zero for every row
 // of the tile are never loaded.
 // ------------------------------------------------------------------------------------
-template <int RT, int MAXV, int UF = 4, int NWV = 4>  // NWV waves per workgroup share a k-block
-__global__ __launch_bounds__(NWV * 64) void k_decoder_partial(const float *__restrict__ xy,
+template <int RT, int MAXV, int UF = 4>
+__global__ __launch_bounds__(256) void k_decoder_partial(const float *__restrict__ xy,
                                                          const float *__restrict__ E,
                                                          float *__restrict__ partial, int T, int h, int N,
                                                          int d, int KB, int M) {
@@ -655,7 +655,7 @@ __global__ __launch_bounds__(NWV * 64) void k_decoder_partial(const float *__res
   const int K = h * N;
   const int nv = (d + 255) >> 8;  // float4 groups per lane
   float *s_xy = s_mem;
-  for (int i = tid; i < RT * KB; i += NWV * 64) {
+  for (int i = tid; i < RT * KB; i += 256) {
     const int r = i / KB, kk = i - r * KB;
     const int m = m0 + r, k = kb * KB + kk;
     float val = 0.0f;
@@ -674,14 +674,14 @@ __global__ __launch_bounds__(NWV * 64) void k_decoder_partial(const float *__res
 #pragma unroll
     for (int j = 0; j < MAXV; ++j) acc[r][j] = make_float4(0.f, 0.f, 0.f, 0.f);
 
-  // each wave takes k = wave, wave+NWV, ...; UF of its E rows are in flight at a time
-  for (int kk0 = wave; kk0 < KB; kk0 += NWV * UF) {
+  // each wave takes k = wave, wave+4, ...; UF of its E rows are in flight at a time
+  for (int kk0 = wave; kk0 < KB; kk0 += 4 * UF) {
     float xs[UF][RT];
     bool any[UF];
     float4 e[UF][MAXV];
 #pragma unroll
     for (int u = 0; u < UF; ++u) {
-      const int kk = kk0 + NWV * u;
+      const int kk = kk0 + 4 * u;
       const int k = kb * KB + kk;
       any[u] = false;
       if (kk < KB && k < K) {
@@ -720,7 +720,7 @@ __global__ __launch_bounds__(NWV * 64) void k_decoder_partial(const float *__res
     }
   }
   __syncthreads();
-  // cross-wave reduction, one row of the tile at a time, through LDS [NWV][d]
+  // cross-wave reduction, one row of the tile at a time, through LDS [4][d]
   float *s_red = s_mem;
   for (int r = 0; r < RT; ++r) {
 #pragma unroll
@@ -731,13 +731,63 @@ __global__ __launch_bounds__(NWV * 64) void k_decoder_partial(const float *__res
     __syncthreads();
     const int m = m0 + r;
     if (m < M)
-      for (int c = tid; c < d; c += NWV * 64) {
-        float v = s_red[c] + s_red[d + c] + s_red[2 * d + c] + s_red[3 * d + c];
-#pragma unroll
-        for (int g = 4; g < NWV; ++g) v += s_red[g * d + c];
-        partial[((long)kb * M + m) * d + c] = v;
-      }
+      for (int c = tid; c < d; c += 256)
+        partial[((long)kb * M + m) * d + c] = s_red[c] + s_red[d + c] + s_red[2 * d + c] + s_red[3 * d + c];
     __syncthreads();
+  }
+}
+
+// The encoder's first stage for ONE row (a decode step of one sequence): partial[kb][:] = sum over the KB rows of
+// k-block kb of xy[k] * E[k,:], rows whose xy is zero never loaded.  Grid (k-blocks, column parts): a workgroup of NWV
+// waves owns 64 * VW adjacent columns, a lane VW of them; wave w takes k = w, w + NWV, ... with UF rows in flight.
+// More column parts mean fewer, larger k-blocks for the same number of waves in flight -- fewer partial rows for the
+// consumer to add.
+template <int VW, int UF, int NWV>
+__global__ __launch_bounds__(NWV * 64) void k_decoder_partial_row(const float *__restrict__ xy,
+                                                                  const float *__restrict__ E,
+                                                                  float *__restrict__ partial, long K, int d, int KB) {
+  extern __shared__ float s_mem[];  // [KB] xy of the block, then [NWV][64 * VW] for the wave reduction
+  typedef float vec_t __attribute__((ext_vector_type(VW)));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int kb = blockIdx.x;
+  const int c = (blockIdx.y * 64 + lane) * VW;
+  for (int i = tid; i < KB; i += NWV * 64) {
+    const long k = (long)kb * KB + i;
+    s_mem[i] = k < K ? xy[k] : 0.0f;
+  }
+  __syncthreads();
+  float acc[VW];
+#pragma unroll
+  for (int e = 0; e < VW; ++e) acc[e] = 0.0f;
+  for (int kk0 = wave; kk0 < KB; kk0 += NWV * UF) {
+    float xs[UF];
+    vec_t ev[UF];
+#pragma unroll
+    for (int u = 0; u < UF; ++u) {
+      const int kk = kk0 + NWV * u;
+      xs[u] = kk < KB ? s_mem[kk] : 0.0f;
+      if (xs[u] != 0.0f && c < d) ev[u] = *reinterpret_cast<const vec_t *>(E + ((long)kb * KB + kk) * d + c);
+    }
+#pragma unroll
+    for (int u = 0; u < UF; ++u)
+      if (xs[u] != 0.0f && c < d) {
+#pragma unroll
+        for (int e = 0; e < VW; ++e) acc[e] = __builtin_fmaf(xs[u], ev[u][e], acc[e]);
+      }
+  }
+  __syncthreads();
+  float *s_red = s_mem;
+#pragma unroll
+  for (int e = 0; e < VW; ++e) s_red[wave * 64 * VW + lane * VW + e] = acc[e];
+  __syncthreads();
+  for (int j = tid; j < 64 * VW; j += NWV * 64) {
+    const int cc = blockIdx.y * 64 * VW + j;
+    if (cc < d) {
+      float v = s_red[j];
+#pragma unroll
+      for (int g = 1; g < NWV; ++g) v += s_red[g * 64 * VW + j];
+      partial[(long)kb * d + cc] = v;
+    }
   }
 }
 
@@ -1403,18 +1453,16 @@ int bdh_launch_decoder_partial_row(bdh_ctx *ctx, int h, int N, int d, const floa
   const long K = (long)h * N;
   if (d > 1024 || (d & 3)) return bdh_fail(ctx, BDH_E_SHAPE, "decoder needs d %% 4 == 0 and d <= 1024, got %d", d);
   const int KBN = (int)((K + KB - 1) / KB);
-  // 16 waves share a k-block: as many waves in flight as 128-row blocks of four waves give, a quarter of the partial rows
-  size_t lds = sizeof(float) * (size_t)KB;
-  if (lds < sizeof(float) * 16u * d) lds = sizeof(float) * 16u * d;
-  const dim3 grid(KBN, 1);
-  const int mv = d <= 256 ? 1 : (d <= 512 ? 2 : 4);
-  if (mv == 1)
-    hipLaunchKernelGGL((k_decoder_partial<1, 1, 16, 16>), grid, dim3(1024), lds, ctx->stream, xy, decoder, partial, 1, h, N, d, KB, 1);
-  else if (mv == 2)
-    hipLaunchKernelGGL((k_decoder_partial<1, 2, 8, 16>), grid, dim3(1024), lds, ctx->stream, xy, decoder, partial, 1, h, N, d, KB, 1);
+  // 16 waves per workgroup; two columns per lane (128-column parts) up to d = 256, four beyond
+  constexpr int NWV = 16;
+  const int VW = d <= 256 ? 2 : 4;
+  const size_t lds = sizeof(float) * std::max<size_t>((size_t)KB, (size_t)NWV * 64 * VW);
+  const dim3 grid(KBN, (d + 64 * VW - 1) / (64 * VW));
+  if (VW == 2)
+    hipLaunchKernelGGL((k_decoder_partial_row<2, 16, NWV>), grid, dim3(NWV * 64), lds, ctx->stream, xy, decoder, partial, K, d, KB);
   else
-    hipLaunchKernelGGL((k_decoder_partial<1, 4, 4, 16>), grid, dim3(1024), lds, ctx->stream, xy, decoder, partial, 1, h, N, d, KB, 1);
-  BDH_LAUNCH_CHECK(ctx, "k_decoder_partial");
+    hipLaunchKernelGGL((k_decoder_partial_row<4, 16, NWV>), grid, dim3(NWV * 64), lds, ctx->stream, xy, decoder, partial, K, d, KB);
+  BDH_LAUNCH_CHECK(ctx, "k_decoder_partial_row");
   *KBN_out = KBN;
   return BDH_OK;
 }
