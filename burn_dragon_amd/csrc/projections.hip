@@ -140,11 +140,7 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank_row1(RowArgs a, int d, co
   const int n = blockIdx.x * NTHR + tid;
   const bool col = n < N;
   const float *wp = w + (long)hh * d * N + (col ? n : 0);
-  // the first UK weight rows are on their way while the row is made (d >= UK)
   float wv[UK];
-#pragma unroll
-  for (int u = 0; u < UK; ++u) wv[u] = wp[(long)u * N];
-
   const float *src = a.partial + (MODE == 1 ? (long)hh * a.rows * d : 0);
   int n_rows = a.rows;
   bool bad_token = false;
@@ -156,6 +152,17 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank_row1(RowArgs a, int d, co
   }
   const int per = (n_rows + NW - 1) / NW;
   const int r0 = min(n_rows, wave * per), r1 = min(n_rows, r0 + per);
+  // Order of the requests (a wavefront has at most 63 memory operations outstanding and they complete in issue order):
+  // the first 32 partial rows of the lane's first column group, then the first UK weight rows, so that the row is
+  // being made while the weights are on their way (d >= UK).
+  const bool head32 = r0 + 32 <= r1;  // uniform over the wave
+  float4 t0[32];
+  if (head32) {
+#pragma unroll
+    for (int u = 0; u < 32; ++u) t0[u] = *reinterpret_cast<const float4 *>(src + (long)(r0 + u) * d + lane * 4);
+  }
+#pragma unroll
+  for (int u = 0; u < UK; ++u) wv[u] = wp[(long)u * N];
   float4 res[4];
   if (MODE == 2) {
 #pragma unroll
@@ -170,6 +177,13 @@ __global__ __launch_bounds__(NTHR) void k_relu_lowrank_row1(RowArgs a, int d, co
     if (c < d) {
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       int r = r0;
+      if (j == 0 && head32) {
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+          v.x += t0[u].x; v.y += t0[u].y; v.z += t0[u].z; v.w += t0[u].w;
+        }
+        r += 32;
+      }
       for (; r + 32 <= r1; r += 32) {  // 32 rows in flight: the sum is a chain of trips to the L2
         float4 t[32];
 #pragma unroll
