@@ -273,3 +273,74 @@ def test_trained_checkpoint_prompt_on_the_bf16_form(bda, corc, prompt_bf16, lazy
         assert rel_err(step, step_ref) < TOL
     model.materialize_state(state)
     assert rel_err(state.storage.cpu().numpy(), rho_ref) < TOL and state.position == pos
+
+
+@pytest.mark.parametrize("mode", ["alibi-recurrent", "rope-rownorm", "alibi-rownorm"])
+def test_extended_prefill_at_the_config3_size(bda, corc, mode):
+    """BASELINE config 3's shape (B=8, h=4, T=2048, N=8192, d=256, 5 % density) through bdh_prefill_chunked_ex, checked
+    without the oracle's loops (too slow at this size):
+      ALiBi, recurrent: token 0 reads a zero state; the final state is sum_s g^(T-s) q_s (x) v_s (src/model/bdh.rs:298-301
+        summed over the tokens) by a device einsum per batch entry; out of one slice against the closed causal form with
+        the decay powers; slices (b=0, h=0..1) hold the bits of a B=1, h=2 call with those heads' slopes.
+      row-normalised: |out[t]| <= max|v| (a quotient of sum s_i v_i by sum |s_i|); one slice against the closed form
+        on the device; slices hold the bits of the reduced call."""
+    from burn_dragon_amd.recurrent import prefill_chunked_ex
+
+    B, h, T, N, d, bs = 8, 4, 2048, 8192, 256, 64
+    g = torch.Generator().manual_seed(17)
+    x = torch.empty((B, h, T, N), dtype=torch.bfloat16)
+    for b in range(B):
+        x[b] = torch.relu(torch.randn((h, T, N), generator=g) - 1.6449).to(torch.bfloat16)
+    v = torch.randn((B, T, d), generator=g).to(torch.bfloat16)
+    xt, vt = x.to(DEV), v.to(DEV)
+    slopes = corc.default_alibi_slopes(h)
+    pos = torch.arange(T, device=DEV, dtype=torch.float32)
+    print(f"extended prefill at the config-3 size: {mode}", flush=True)
+    if mode == "alibi-recurrent":
+        rho = torch.zeros((B, h, N, d), device=DEV)
+        out = prefill_chunked_ex(xt, vt, rho, None, 0, rotary=bda.RotaryEmbedding.ALIBI, alibi_slopes=slopes,
+                                 state_is_zero=True)
+        torch.cuda.synchronize()
+        assert not out[:, :, 0].any()
+        logd = torch.log(torch.exp(-torch.from_numpy(slopes))).to(DEV)  # log of the rounded per-token factor
+        for b in range(B):
+            q = xt[b].float()  # [h,T,N]; ALiBi does not rotate
+            w = torch.exp((T - pos)[None, :] * logd[:, None])  # [h,T]: g^(T-s)
+            ref = torch.einsum("htn,ht,td->hnd", q, w, vt[b].float())
+            err = float((rho[b] - ref).abs().max()) / float(ref.abs().max())
+            assert err < TOL, f"batch entry {b}: {err}"
+        q0 = xt[0, 1].float()
+        dec = torch.exp((pos[:, None] - pos[None, :]).clamp(min=0) * logd[1])
+        o = (torch.tril(q0 @ q0.T, -1) * dec) @ vt[0].float()
+        assert float((out[0, 1] - o).abs().max()) / float(o.abs().max()) < TOL
+        rho2 = torch.zeros((1, 2, N, d), device=DEV)
+        out2 = prefill_chunked_ex(xt[:1, :2].contiguous(), vt[:1].contiguous(), rho2, None, 0,
+                                  rotary=bda.RotaryEmbedding.ALIBI, alibi_slopes=slopes[:2], state_is_zero=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out2[0], out[0, :2]) and torch.equal(rho2[0], rho[0, :2])
+        return
+    rot = bda.RotaryEmbedding.ROPE if mode == "rope-rownorm" else bda.RotaryEmbedding.ALIBI
+    freqs = corc.build_freqs(N, rotary=orc.ROPE if mode == "rope-rownorm" else orc.ALIBI)
+    ft = torch.from_numpy(freqs).to(DEV)
+    sl = slopes if mode == "alibi-rownorm" else None
+    out = prefill_chunked_ex(xt, vt, None, ft, 0, rotary=rot, alibi_slopes=sl, row_normalize=True, block_size=bs)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    assert float(out.abs().max()) <= float(vt.float().abs().max()) * (1 + 1e-3)
+    hh = 2
+    if mode == "rope-rownorm":
+        q0 = torch.from_numpy(corc.rotate(x[0:1, hh:hh + 1].float().numpy(), freqs, orc.ROPE, 0)).to(DEV)[0, 0]
+        q0 = q0.to(torch.bfloat16).float()
+    else:
+        q0 = xt[0, hh].float()
+    s = torch.tril(q0 @ q0.T, -1)
+    if sl is not None:  # the additive term on whole causal time blocks (the diagonal block included)
+        blk = (torch.arange(T, device=DEV) // bs)
+        s = s + float(sl[hh]) * (pos[None, :] - pos[:, None]) * (blk[None, :] <= blk[:, None])
+    s = s.to(torch.bfloat16).float()
+    o = (s @ vt[0].float()) / (s.abs().sum(1, keepdim=True) + 1e-6)
+    assert float((out[0, hh] - o).abs().max()) / float(o.abs().max()) < TOL
+    out2 = prefill_chunked_ex(xt[:1, :2].contiguous(), vt[:1].contiguous(), None, ft, 0, rotary=rot,
+                              alibi_slopes=None if sl is None else sl[:2], row_normalize=True, block_size=bs)
+    torch.cuda.synchronize()
+    assert torch.equal(out2[0], out[0, :2])
