@@ -407,6 +407,39 @@ int bdh_model_forward_deferred(bdh_model *m, bdh_model_logs *logs, const int64_t
                             nullptr, logs);
 }
 
+int bdh_model_forward_deferred_layers(bdh_model *m, bdh_model_logs *logs, const int64_t *tokens, int B,
+                                      void *const *rho_layers_host, int rho_dtype, int64_t position,
+                                      const int32_t *positions_dev, float *logits, int64_t *next_tokens) {
+  if (!m) return BDH_E_INVAL;
+  bdh_ctx *ctx = m->ctx;
+  if (!logs) return bdh_fail(ctx, BDH_E_INVAL, "null model logs");
+  if ((int)logs->layer.size() != m->cfg.n_layer || B != logs->B || rho_dtype != logs->rho_dtype)
+    return bdh_fail(ctx, BDH_E_INVAL, "the logs were created for %zu layers, batch %d, state type %d", logs->layer.size(),
+                    logs->B, logs->rho_dtype);
+  if (!rho_layers_host) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  for (int l = 0; l < m->cfg.n_layer; ++l)
+    if (!rho_layers_host[l]) return bdh_fail(ctx, BDH_E_INVAL, "null state pointer of layer %d", l);
+  StateRefs st;
+  st.rho_layers = rho_layers_host;
+  return model_forward_impl(m, tokens, B, 1, st, rho_dtype, position, positions_dev, logits, next_tokens, nullptr,
+                            nullptr, logs);
+}
+
+int bdh_model_flush_layers(bdh_model *m, bdh_model_logs *logs, void *const *rho_layers_host) {
+  if (!m) return BDH_E_INVAL;
+  bdh_ctx *ctx = m->ctx;
+  if (!logs) return bdh_fail(ctx, BDH_E_INVAL, "null model logs");
+  if ((int)logs->layer.size() != m->cfg.n_layer) return bdh_fail(ctx, BDH_E_INVAL, "the logs belong to another model");
+  if (bdh_model_logs_pending(logs) == 0) return BDH_OK;
+  if (!rho_layers_host) return bdh_fail(ctx, BDH_E_INVAL, "null data pointer");
+  for (int l = 0; l < m->cfg.n_layer; ++l) {
+    if (!rho_layers_host[l]) return bdh_fail(ctx, BDH_E_INVAL, "null state pointer of layer %d", l);
+    const int rc = bdh_state_flush(ctx, logs->layer[l], rho_layers_host[l]);
+    if (rc != BDH_OK) return rc;
+  }
+  return BDH_OK;
+}
+
 int bdh_model_flush(bdh_model *m, bdh_model_logs *logs, void *rho) {
   if (!m) return BDH_E_INVAL;
   bdh_ctx *ctx = m->ctx;

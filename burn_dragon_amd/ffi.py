@@ -33,7 +33,7 @@ EXPORTS = [
     "bdh_state_log_create", "bdh_state_log_destroy", "bdh_state_log_pending", "bdh_state_log_bytes",
     "bdh_state_step_deferred", "bdh_state_flush", "bdh_model_forward_layers",
     "bdh_model_logs_create", "bdh_model_logs_destroy", "bdh_model_logs_pending", "bdh_model_forward_deferred",
-    "bdh_model_flush",
+    "bdh_model_flush", "bdh_model_forward_deferred_layers", "bdh_model_flush_layers",
 ]
 
 
@@ -105,6 +105,8 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.bdh_model_logs_pending.argtypes = [P]
     lib.bdh_model_forward_deferred.argtypes = [P, P, P, c_int, P, c_int, c_int64, P, P, P]
     lib.bdh_model_flush.argtypes = [P, P, P]
+    lib.bdh_model_forward_deferred_layers.argtypes = [P, P, P, c_int, P, c_int, c_int64, P, P, P]
+    lib.bdh_model_flush_layers.argtypes = [P, P, P]
     lib.bdh_relu_lowrank.argtypes = [P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_float, c_int, P, c_int,
                                      P, P]
     lib.bdh_layer_norm.argtypes = [P, c_int64, c_int, P, P]

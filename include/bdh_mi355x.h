@@ -524,6 +524,14 @@ int bdh_model_forward_deferred(bdh_model *model, bdh_model_logs *logs, const int
                                int rho_dtype, int64_t position, const int32_t *positions_dev, float *logits,
                                int64_t *next_tokens);
 int bdh_model_flush(bdh_model *model, bdh_model_logs *logs, void *rho);
+/* The same two calls with the state given layer by layer (rho_layers_host: HOST array of n_layer DEVICE pointers, layer
+ * l's state [B,h,N,d]), as bdh_model_forward_layers takes it: the reference's ModelState of independent per-layer
+ * tensors (src/model/state.rs:5-15) decodes with deferred updates without a copy.  A layer's log stays bound to the
+ * pointer it first saw until it is flushed. */
+int bdh_model_forward_deferred_layers(bdh_model *model, bdh_model_logs *logs, const int64_t *tokens, int B,
+                                      void *const *rho_layers_host, int rho_dtype, int64_t position,
+                                      const int32_t *positions_dev, float *logits, int64_t *next_tokens);
+int bdh_model_flush_layers(bdh_model *model, bdh_model_logs *logs, void *const *rho_layers_host);
 
 /* Draws the next token of every sequence on the device.  Replaces the temperature division of
  * sample_next_token (src/generation.rs:117) and sample_from_logits_values (src/generation.rs:26-72),

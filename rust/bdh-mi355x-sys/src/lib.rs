@@ -176,6 +176,11 @@ extern "C" {
         rho: *mut c_void, rho_dtype: c_int, position: i64, positions_dev: *const i32, logits: *mut f32,
         next_tokens: *mut i64) -> c_int;
     pub fn bdh_model_flush(model: *mut bdh_model, logs: *mut bdh_model_logs, rho: *mut c_void) -> c_int;
+    pub fn bdh_model_forward_deferred_layers(model: *mut bdh_model, logs: *mut bdh_model_logs, tokens: *const i64,
+        b: c_int, rho_layers_host: *const *mut c_void, rho_dtype: c_int, position: i64, positions_dev: *const i32,
+        logits: *mut f32, next_tokens: *mut i64) -> c_int;
+    pub fn bdh_model_flush_layers(model: *mut bdh_model, logs: *mut bdh_model_logs,
+        rho_layers_host: *const *mut c_void) -> c_int;
     pub fn bdh_sample_top_k(ctx: *mut bdh_ctx, b: c_int, v: c_int, logits: *const f32, row_stride: i64,
         temperature: f32, top_k: c_int, uniforms: *const f32, next_tokens: *mut i64) -> c_int;
     pub fn bdh_probe_chunks(ctx: *mut bdh_ctx, region: *mut c_void, region_bytes: usize,

@@ -215,6 +215,71 @@ impl<B: HipPointers> Model<B> {
     }
 }
 
+/// The pending state updates of a decode loop with deferred updates: one log per layer, for a batch of `batch`
+/// sequences.  Owned by the caller next to the ModelState it belongs to; `Model::flush_deferred` (or the
+/// `capacity`-th step by itself) applies what is pending.  No counterpart in the reference.
+pub struct ModelLogs {
+    raw: *mut bdh_model_logs,
+    model: *mut bdh_model,
+    batch: usize,
+}
+
+impl ModelLogs {
+    pub fn pending(&self) -> usize {
+        unsafe { bdh_model_logs_pending(self.raw) as usize }
+    }
+}
+
+impl Drop for ModelLogs {
+    fn drop(&mut self) {
+        unsafe { bdh_model_logs_destroy(self.model, self.raw) };
+    }
+}
+
+impl<B: HipPointers> Model<B> {
+    /// Logs for decoding `batch` sequences with the state updates deferred, flushed every `capacity` tokens
+    /// (RoPE models with n_embd 256 or 512; capacity 1..128 with capacity * n_embd <= 32768).  The logs must not
+    /// outlive the model.
+    pub fn deferred_logs(&self, batch: usize, capacity: usize) -> ModelLogs {
+        let mut raw = std::ptr::null_mut();
+        self.ctx.check(unsafe { bdh_model_logs_create(self.raw, batch as i32, BDH_F32, capacity as i32, &mut raw) });
+        ModelLogs { raw, model: self.raw, batch }
+    }
+
+    /// One decode step (tokens [B,1]) of forward_with_state with the rank-1 updates of src/model/bdh.rs:298 logged
+    /// instead of written: the layers' state tensors are read, not modified, until the logs are flushed.  Logits agree
+    /// with forward_with_state to f32 rounding.  Call `flush_deferred` before anything else reads the state tensors.
+    pub fn decode_step_deferred(&self, tokens: Tensor<B, 2, Int>, state: &mut ModelState<B>, logs: &mut ModelLogs)
+        -> Tensor<B, 3> {
+        let [b, t] = tokens.dims();
+        assert_eq!(t, 1, "a deferred step takes one token per sequence");
+        assert_eq!(b, logs.batch, "the logs were made for another batch size");
+        let device = tokens.device();
+        let ptrs: Vec<*mut c_void> = state.layers.iter().map(|layer| {
+            let rho = layer.rho.as_ref().expect("a deferred step continues a state that a prompt call has made");
+            B::device_ptr(rho) as *mut c_void
+        }).collect();
+        let logits = Tensor::<B, 3>::empty([b, 1, self.dims.vocab], &device);
+        self.ctx.check(unsafe {
+            bdh_model_forward_deferred_layers(self.raw, logs.raw, B::int_device_ptr(&tokens), b as i32, ptrs.as_ptr(),
+                BDH_F32, state.position as i64, std::ptr::null(), B::device_ptr(&logits), std::ptr::null_mut())
+        });
+        state.position = state.position.saturating_add(1);
+        logits
+    }
+
+    /// Applies the pending updates: afterwards the state tensors hold what forward_with_state would have left.
+    pub fn flush_deferred(&self, state: &mut ModelState<B>, logs: &mut ModelLogs) {
+        if logs.pending() == 0 {
+            return;
+        }
+        let ptrs: Vec<*mut c_void> = state.layers.iter().map(|layer| {
+            B::device_ptr(layer.rho.as_ref().expect("pending updates belong to a state")) as *mut c_void
+        }).collect();
+        self.ctx.check(unsafe { bdh_model_flush_layers(self.raw, logs.raw, ptrs.as_ptr()) });
+    }
+}
+
 impl<B: HipPointers> Drop for Model<B> {
     fn drop(&mut self) {
         unsafe { bdh_model_destroy(self.raw) };

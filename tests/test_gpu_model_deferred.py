@@ -191,3 +191,61 @@ def test_config4_architecture_with_deferred_updates(bda, corc, state, tol):
     e_state = rel_err(st.storage.float().cpu().numpy(), rho_ref)
     print(f"worst decode logits rel err {worst:.2e}, state rel err {e_state:.2e}", flush=True)
     assert e_state < tol
+
+
+def test_deferred_decode_with_the_state_given_layer_by_layer(bda):
+    """bdh_model_forward_deferred_layers / bdh_model_flush_layers on per-layer allocations against
+    bdh_model_forward_deferred / bdh_model_flush on one tensor: the same launches on the same bytes, so logits and
+    flushed states are equal bit for bit; 11 steps with a log capacity of 4 (two flushes by the steps themselves)."""
+    from burn_dragon_amd import ffi
+
+    L, d, h, mult, V, B, cap = 3, 256, 2, 8, 64, 2, 4
+    model, _, _ = _model(bda, orc.ROPE, L, d, h, mult, V, 7)
+    N = model.latent
+    ctx, lib = model.ctx, model.ctx.lib
+    rng = np.random.default_rng(4)
+    prompt = torch.from_numpy(rng.integers(0, V, size=(B, 5))).to(DEV)
+    steps = [torch.from_numpy(rng.integers(0, V, size=(B, 1))).to(DEV) for _ in range(11)]
+
+    def run(separate):
+        whole = torch.zeros((L, B, h, N, d), device=DEV)
+        rhos = [torch.zeros((B, h, N, d), device=DEV) for _ in range(L)] if separate else [whole[l] for l in range(L)]
+        ptrs = (ctypes.c_void_p * L)(*[t.data_ptr() for t in rhos])
+        logs = ctypes.c_void_p()
+        ctx.check(lib.bdh_model_logs_create(model.handle, B, ffi.F32, cap, ctypes.byref(logs)))
+        try:
+            logits = torch.empty((B, 5, V), device=DEV)
+            ctx.check(lib.bdh_model_forward_layers(model.handle, prompt.data_ptr(), B, 5, ptrs, ffi.F32, None, 0, None,
+                                                   logits.data_ptr(), None, None))
+            outs, pos = [], 5
+            for tok in steps:
+                lg = torch.empty((B, 1, V), device=DEV)
+                if separate:
+                    ctx.check(lib.bdh_model_forward_deferred_layers(model.handle, logs, tok.data_ptr(), B, ptrs, ffi.F32,
+                                                                    pos, None, lg.data_ptr(), None))
+                else:
+                    ctx.check(lib.bdh_model_forward_deferred(model.handle, logs, tok.data_ptr(), B, whole.data_ptr(),
+                                                             ffi.F32, pos, None, lg.data_ptr(), None))
+                pos += 1
+                outs.append(lg)
+            assert lib.bdh_model_logs_pending(logs) == 11 % cap
+            if separate:
+                ctx.check(lib.bdh_model_flush_layers(model.handle, logs, ptrs))
+            else:
+                ctx.check(lib.bdh_model_flush(model.handle, logs, whole.data_ptr()))
+            assert lib.bdh_model_logs_pending(logs) == 0
+            torch.cuda.synchronize()
+            return outs, torch.stack(list(rhos)).clone()
+        finally:
+            lib.bdh_model_logs_destroy(model.handle, logs)
+
+    model.ctx.set_option("model.one_launch", 0)  # the prompt call kernel by kernel on both sides
+    try:
+        outs_a, rho_a = run(False)
+        outs_b, rho_b = run(True)
+    finally:
+        model.ctx.set_option("model.one_launch", 1)
+    for la, lb in zip(outs_a, outs_b):
+        assert torch.equal(la, lb)
+    assert torch.equal(rho_a, rho_b)
+    assert rho_a.abs().max() > 0
