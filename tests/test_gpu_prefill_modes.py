@@ -344,3 +344,51 @@ def test_extended_prefill_at_the_config3_size(bda, corc, mode):
                               alibi_slopes=None if sl is None else sl[:2], row_normalize=True, block_size=bs)
     torch.cuda.synchronize()
     assert torch.equal(out2[0], out[0, :2])
+
+
+def test_extended_prefill_edge_shapes(bda, corc):
+    """One token, an empty batch, a latent that is not a multiple of 8, more heads than slopes can travel with."""
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.recurrent import prefill_chunked_ex
+
+    ctx = ffi.default_context(0)
+    # T = 1: the readout of the carried state alone, then one decayed update
+    B, h, N, d = 2, 2, 16, 24
+    g = torch.Generator().manual_seed(5)
+    x = torch.relu(torch.randn((B, h, 1, N), generator=g)).to(torch.bfloat16)
+    v = torch.randn((B, 1, d), generator=g).to(torch.bfloat16)
+    rho0 = (0.1 * torch.randn((B, h, N, d), generator=g)).float()
+    slopes = np.array([0.7, 0.2], np.float32)
+    out_ref, rho_ref = corc.recurrent_attention(x.float().numpy(), v.float().numpy(), rho0.numpy(),
+                                                decay=corc.alibi_decay(slopes))
+    rho = rho0.clone().to(DEV)
+    out = prefill_chunked_ex(x.to(DEV), v.to(DEV), rho, None, 3, rotary=bda.RotaryEmbedding.ALIBI, alibi_slopes=slopes)
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), out_ref) < TOL and rel_err(rho.cpu().numpy(), rho_ref) < TOL
+    # an empty batch is a no-op
+    e = torch.zeros((0, h, 4, N), dtype=torch.bfloat16, device=DEV)
+    assert prefill_chunked_ex(e, torch.zeros((0, 4, d), dtype=torch.bfloat16, device=DEV),
+                              torch.zeros((0, h, N, d), device=DEV), None, 0, rotary=bda.RotaryEmbedding.ALIBI).shape == (0, h, 4, d)
+    # N must be a multiple of 8 (x is read in 16-byte pieces)
+    xb = torch.zeros((1, 1, 4, 12), dtype=torch.bfloat16, device=DEV)
+    vb = torch.zeros((1, 4, 8), dtype=torch.bfloat16, device=DEV)
+    ob = torch.empty((1, 1, 4, 8), device=DEV)
+    rb = torch.zeros((1, 1, 12, 8), device=DEV)
+    rc = ctx.lib.bdh_prefill_chunked_ex(ctx.handle, 1, 1, 4, 12, 8, int(bda.RotaryEmbedding.ALIBI), ffi.ptr(xb), ffi.ptr(vb),
+                                        None, None, 0, 0, 0, 1, ffi.ptr(rb), ffi.ptr(ob))
+    assert rc == ffi.E_SHAPE
+    # more than 64 heads cannot carry per-head slopes in the kernel arguments
+    xh = torch.zeros((1, 65, 2, 8), dtype=torch.bfloat16, device=DEV)
+    vh = torch.zeros((1, 2, 8), dtype=torch.bfloat16, device=DEV)
+    oh = torch.empty((1, 65, 2, 8), device=DEV)
+    rh = torch.zeros((1, 65, 8, 8), device=DEV)
+    rc = ctx.lib.bdh_prefill_chunked_ex(ctx.handle, 1, 65, 2, 8, 8, int(bda.RotaryEmbedding.ALIBI), ffi.ptr(xh), ffi.ptr(vh),
+                                        None, None, 0, 0, 0, 1, ffi.ptr(rh), ffi.ptr(oh))
+    assert rc == ffi.E_SHAPE
+    # PoPE and RoPE with that many heads are fine (no per-head parameters)
+    fq = torch.from_numpy(corc.build_freqs(8, rotary=orc.POPE)).to(DEV)
+    rp = torch.zeros((1, 65, 16, 8), device=DEV)
+    rc = ctx.lib.bdh_prefill_chunked_ex(ctx.handle, 1, 65, 2, 8, 8, int(bda.RotaryEmbedding.POPE), ffi.ptr(xh), ffi.ptr(vh),
+                                        ffi.ptr(fq), None, 0, 0, 0, 1, ffi.ptr(rp), ffi.ptr(oh))
+    assert rc == 0
+    torch.cuda.synchronize()
