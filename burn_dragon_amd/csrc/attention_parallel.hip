@@ -607,8 +607,11 @@ extern "C" int bdh_fused_state_aligned(bdh_ctx *ctx, int B, int h, int T, int N,
   const int tb = (T + block_size - 1) / block_size;
   const bool sparse = block_pairs_host != nullptr;
   if (sparse && tb > 4096) return bdh_fail(ctx, BDH_E_SHAPE, "sparse time pattern with %d blocks", tb);
+  // opt-in: the dense layout, row-normalised, on the bf16 matrix cores (inputs and scores rounded to bf16: 2e-2)
+  if (ctx->opt_fsa_path == 2 && !sparse && row_normalize && (N & 7) == 0 && bdh_aligned(query, 16) && bdh_aligned(out, 16))
+    return bdh_launch_fsa_bf16(ctx, B, h, T, N, dv, query, value, freqs, alibi_slopes_host, block_size, rotary, out);
   const size_t lds = sizeof(float) * ((size_t)Nq + T);
-  int path = ctx->opt_fsa_path;  // -1 choose, 0 row kernel, 1 matrix cores
+  int path = ctx->opt_fsa_path == 2 ? -1 : ctx->opt_fsa_path;  // -1 choose, 0 row kernel, 1 matrix cores
   if (path < 0) path = T >= 128 ? 1 : 0;
   if (path == 0 && lds > 150 * 1024) path = 1;
   if (S * T > 0x7fffffffL || (S + 7) / 8 * 8 * (long)(((T + 127) / 128) * ((T + 127) / 128)) > 0x7fffffffL) return bdh_fail(ctx, BDH_E_SHAPE, "B*h*T too large");

@@ -185,7 +185,7 @@ int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value) {
     return BDH_OK;
   }
   if (strcmp(name, "fused_state_aligned.path") == 0) {
-    if (value < -1 || value > 1) return bdh_fail(ctx, BDH_E_INVAL, "fused_state_aligned.path takes -1, 0 or 1");
+    if (value < -1 || value > 2) return bdh_fail(ctx, BDH_E_INVAL, "fused_state_aligned.path takes -1, 0, 1 or 2");
     ctx->opt_fsa_path = value;
     return BDH_OK;
   }

@@ -141,6 +141,9 @@ int bdh_launch_state_chunks_f32(bdh_ctx *ctx, const StateStepParams &p, float *o
 // prefill.hip: the same T steps on the bf16 matrix cores (x, v and the scores rounded to bf16, f32 accumulation and
 // f32 state; tolerance class 2e-2): any rotary, a lazily decayed state is brought up to date first; host position only.
 int bdh_launch_state_prefill_bf16(bdh_ctx *ctx, const StateStepParams &p, float *out_ln);
+// prefill.hip: fused_state_aligned (dense causal layout, row-normalised) on the bf16 matrix cores; tolerance class 2e-2
+int bdh_launch_fsa_bf16(bdh_ctx *ctx, int B, int h, int T, int N, int dv, const float *query, const float *value,
+                        const float *freqs, const float *alibi_slopes_host, int block_size, int rotary, float *out);
 // rho <- the up-to-date state, stamps <- clock, for a lazily decayed ALiBi state
 int bdh_launch_alibi_materialize(bdh_ctx *ctx, int B, int h, int N, int d, const float *slopes_host, int64_t clock,
                                  const int32_t *clocks_dev, void *rho, int rho_dtype, int32_t *stamps);

@@ -1601,6 +1601,34 @@ int bdh_launch_state_prefill_bf16(bdh_ctx *ctx, const StateStepParams &p, float 
   return BDH_OK;
 }
 
+// kernel::linear_attention::fused_state_aligned with the dense causal layout on the bf16 matrix cores: f32 inputs
+// rounded to bf16 in the context's staging buffer, then the row-normalised form of bdh_prefill_chunked_ex.
+int bdh_launch_fsa_bf16(bdh_ctx *ctx, int B, int h, int T, int N, int dv, const float *query, const float *value,
+                        const float *freqs, const float *alibi_slopes_host, int block_size, int rotary, float *out) {
+  PassMode pm;
+  pm.rotary = rotary;
+  pm.row_norm = true;
+  pm.block_size = block_size > 0 ? block_size : 1;
+  pm.add_alibi = alibi_slopes_host != nullptr;
+  if (pm.add_alibi) {
+    if (h > 64) return bdh_fail(ctx, BDH_E_SHAPE, "at most 64 heads with ALiBi slopes (h=%d)", h);
+    memcpy(pm.head_par, alibi_slopes_host, sizeof(float) * h);
+  }
+  const size_t nx = (size_t)B * h * T * N, nv = (size_t)B * T * dv;
+  const size_t x_bytes = bdh_align_up(nx * 2, 256);
+  int rc = bdh_stage_reserve(ctx, x_bytes + bdh_align_up(nv * 2, 256));
+  if (rc != BDH_OK) return rc;
+  unsigned short *xb = static_cast<unsigned short *>(ctx->stage);
+  unsigned short *vb = reinterpret_cast<unsigned short *>(static_cast<char *>(ctx->stage) + x_bytes);
+  hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)std::min<size_t>((nx / 4 + 255) / 256 + 1, 1u << 16)), dim3(256), 0,
+                     ctx->stream, query, xb, nx);
+  BDH_LAUNCH_CHECK(ctx, "k_f32_to_bf16<query>");
+  hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)std::min<size_t>((nv / 4 + 255) / 256 + 1, 1u << 16)), dim3(256), 0,
+                     ctx->stream, value, vb, nv);
+  BDH_LAUNCH_CHECK(ctx, "k_f32_to_bf16<value>");
+  return prefill_chunked_impl(ctx, B, h, T, N, dv, xb, vb, freqs, 0, 0, 0, nullptr, out, pm);
+}
+
 extern "C" int bdh_prefill_chunked(bdh_ctx *ctx, int B, int h, int T, int N, int d, const uint16_t *x_bf16,
                                    const uint16_t *v_bf16, const float *freqs, int64_t position, int chunk,
                                    int flags, float *rho, float *out) {

@@ -132,7 +132,10 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       beyond the one above; 0 = never).
  *   "fused_state_aligned.path": -1 (default) pick by T, 0 = one workgroup per query row,
  *                       1 = the two products on the matrix cores (T >= 128 by default; operands as three
- *                       bf16 terms each, f32-level accuracy). */
+ *                       bf16 terms each, f32-level accuracy), 2 = dense-pattern row-normalised calls (N a multiple
+ *                       of 8) as bdh_prefill_chunked_ex computes them: inputs and scores rounded to bf16 once, about
+ *                       five times faster at the config-3 shape, tolerance class 2e-2 instead of 1e-3 (other calls
+ *                       as -1); reaches Attention::forward and BDH::forward_fast through bdh_model_forward_fast*. */
 int bdh_ctx_set_option(bdh_ctx *ctx, const char *name, int value);
 
 /* ---- host-side tables (computed on the host in the reference as well) --------------- */

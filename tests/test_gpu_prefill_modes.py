@@ -392,3 +392,42 @@ def test_extended_prefill_edge_shapes(bda, corc):
                                         ffi.ptr(fq), None, 0, 0, 0, 1, ffi.ptr(rp), ffi.ptr(oh))
     assert rc == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("rotary", ["rope", "alibi", "pope"])
+def test_fused_state_aligned_takes_the_bf16_form_when_asked(bda, corc, rotary):
+    """bdh_fused_state_aligned with "fused_state_aligned.path" = 2 (dense pattern, row-normalised): against the oracle's
+    blocked form at the bf16 tolerance, and a sparse pattern under the same option still takes the f32 path (1e-3)."""
+    from burn_dragon_amd import ffi
+    from burn_dragon_amd.kernel import linear_attention
+
+    B, h, T, N, dv, bs = 2, 3, 300, 200, 72, 64
+    rot = ROT[rotary]
+    rng = np.random.default_rng(8)
+    query = np.maximum(rng.standard_normal((B, h, T, N)) - 0.5, 0).astype(np.float32)
+    value = rng.standard_normal((B, T, dv)).astype(np.float32)
+    slopes = corc.default_alibi_slopes(h) if rotary == "alibi" else None
+    freqs = corc.build_freqs(N, rotary=rot)
+    qt, vt = torch.from_numpy(query).to(DEV), torch.from_numpy(value[:, None]).to(DEV)
+    st = None if slopes is None else torch.from_numpy(slopes)
+    ctx = ffi.default_context(0)
+    ctx.set_option("fused_state_aligned.path", 2)
+    try:
+        got = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs), st, bda.BlockPattern2d.dense(bs),
+                                                   bda.RotaryEmbedding.parse(rotary))
+        tb = (T + bs - 1) // bs
+        pairs = {(r, c) for r in range(tb) for c in range(r + 1) if (r + c) % 2 == 0}
+        got_sparse = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs), st,
+                                                          bda.BlockPattern2d.from_pairs(bs, pairs),
+                                                          bda.RotaryEmbedding.parse(rotary))
+    finally:
+        ctx.set_option("fused_state_aligned.path", -1)
+    exact = linear_attention.fused_state_aligned(qt, vt, torch.from_numpy(freqs), st, bda.BlockPattern2d.dense(bs),
+                                                 bda.RotaryEmbedding.parse(rotary))
+    torch.cuda.synchronize()
+    ref = corc.fused_state_aligned(query, value, freqs, slopes, bs, rot)
+    assert rel_err(got.cpu().numpy(), ref) < TOL
+    assert rel_err(exact.cpu().numpy(), ref) < 1e-3
+    assert not torch.equal(got, exact)  # the option took
+    ref_sparse = corc.fused_state_aligned(query, value, freqs, slopes, bs, rot, pairs=pairs)
+    assert rel_err(got_sparse.cpu().numpy(), ref_sparse) < 1e-3
