@@ -248,9 +248,14 @@ int model_forward_impl(bdh_model *m, const int64_t *tokens, int B, int T, StateR
   // launches per layer instead of six.  The two reductions whose inputs come from other CUs -- the readout partials with
   // their LayerNorm, the encoder partials with the two LayerNorms and the residual -- are redone by every workgroup of the
   // projection that consumes the result (D_y, the next layer's D_x), behind its first weight loads.
+  // Taken while what every workgroup adds up stays small against the weights it streams: at most 64 KiB of readout
+  // partials per head (N/128 rows of d floats) and 128 KiB of encoder partials (h*N/KB rows); beyond that the redundant
+  // sums cost more than the two launches they replace (measured at d=512, h=8, N=16384: 2.97 against 2.87 ms per token).
+  const int fused_kb = ctx->opt_model_fused_kb;
   if (B == 1 && T == 1 && !x_tap && !viz && !logs && ctx->opt_model_fused_rows != 0 && c.rotary == BDH_ROPE &&
-      (d == 256 || d == 512) && N >= 2 && (N % 2) == 0) {
-    const int KB = ctx->opt_model_fused_kb;
+      (d == 256 || d == 512) && N >= 2 && (N % 2) == 0 && (long)N * d <= (2L << 20) &&
+      (long)h * N * d <= (long)fused_kb * (1L << 15)) {
+    const int KB = fused_kb;
     const size_t K = (size_t)h * N;
     const size_t kbn_max = (K + KB - 1) / KB;
     const size_t n_row = bdh_align_up((size_t)d, 64), n_lat = bdh_align_up(K, 64);

@@ -126,7 +126,9 @@ const char *bdh_last_error(const bdh_ctx *ctx);
  *                       per layer instead of six: D_y sums the state step's readout partials and applies their
  *                       LayerNorm itself, the next layer's D_x sums the encoder's partials and applies the two
  *                       LayerNorms and the residual (the first layer's D_x makes its row from the embedding), each
- *                       behind its first weight loads.  0 = kernel by kernel (values agree to 1e-5).
+ *                       behind its first weight loads; taken while those sums stay small against the weights
+ *                       (N * n_embd <= 2 Mi and n_head * N * n_embd <= 32 Ki * fused_kb: BASELINE config 1 is the
+ *                       largest such shape).  0 = kernel by kernel (values agree to 1e-5).
  *   "model.fused_kb":   rows of E per workgroup of the encoder's first stage in that form (128 .. 2048, default 256).
  *   "model.phase_batch": the two-launch layer only for at most this many sequences (default: no limit
  *                       beyond the one above; 0 = never).

@@ -760,3 +760,5 @@ def test_single_sequence_decode_folds_the_reductions_into_the_projections(bda, c
         assert rel_err(lg1, logits_ref) < tol_orc
     assert rel_err(runs[1][1], runs[0][1]) < tol_pair
     assert rel_err(runs[1][1], rho_ref) < tol_orc
+    # other summation trees: the two forms do not give the same bits, so the option did select another path
+    assert any(not np.array_equal(a[0], b[0]) for a, b in zip(runs[1][0], runs[0][0]))
